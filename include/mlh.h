@@ -1,0 +1,181 @@
+/*
+ * mlh.h -- C ABI of the MI355X (gfx950) device layer for the mini-llm inference
+ * token loop.  This is the only interface through which host code reaches HIP:
+ * plain pointers and sizes, int status codes (0 = ok, < 0 = error; text from
+ * mlh_last_error), no C++ or torch types.
+ *
+ * Each entry point names the reference interface it replaces (file:line in
+ * daniel-chermetz/mini-llm-cuda).  The reference keeps all of this in process
+ * globals (network_globals.h:136-241); here one mlh_ctx owns every device
+ * allocation, one HIP stream and the captured decode graphs.  A context is not
+ * thread-safe; different contexts are independent.
+ */
+#ifndef MLH_H
+#define MLH_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLH_MAX_LAYERS 64
+
+#define MLH_KIND_ATTENTION 0 /* softmax attention block (inference.cu:401-610) */
+#define MLH_KIND_GDN 1       /* gated-delta-net block (no reference counterpart) */
+
+#define MLH_DTYPE_F32 0
+#define MLH_DTYPE_BF16 1 /* matrices rounded to bf16 (RNE) at upload, fp32 accumulate */
+
+/* Runtime form of the compile-time macros of network_meta.h:3-20 (same names),
+ * plus the fields the reference does not have. */
+typedef struct {
+    int32_t dim;
+    int32_t attnHeads;
+    int32_t headDim; /* attnHeads * headDim must equal dim (inference.cu:511-573 splits dim by head) */
+    int32_t ffnDim;
+    int32_t transformers;
+    int32_t maxL;
+    int32_t vocabSize;
+    float ropeDenomBase;
+    int32_t qkRmsNorm;   /* CONFIG_QK_RMS_NORM,  attention layers only */
+    int32_t queryGating; /* CONFIG_QUERY_GATING, attention layers only */
+    int32_t gdnHeads, gdnDk, gdnDv;
+    int32_t pleDim;      /* per-layer-embedding width, 0 = none */
+    int32_t weightDtype; /* MLH_DTYPE_* */
+    int32_t maxSeqs;     /* concurrent sequences held on the device (>= 1) */
+    int32_t layerKinds[MLH_MAX_LAYERS]; /* by FILE index: block 0 is the top of the stack (inference.cu:384-385) */
+} mlh_hparams;
+
+/* Tensor ids.  Per-layer ids follow the read order of load_model.cu:411-450;
+ * the tail (GDN gates, per-layer embeddings) extends it. */
+enum {
+    MLH_T_TOKEN_EMBEDDINGS = 0, /* [vocabSize, dim]   embedding_weights (network_globals.h:150-151) */
+    MLH_T_FINAL_RMS_GAMMA = 1,  /* [dim]              final_rms_weights */
+    MLH_T_RMS_GAMMA = 2,        /* [dim]              rms1_weights */
+    MLH_T_QUERY = 3,            /* [dim or Hg*dk, dim] query_weights */
+    MLH_T_KEY = 4,              /*                    key_weights */
+    MLH_T_VALUE = 5,            /* [dim or Hg*dv, dim] value_weights */
+    MLH_T_OUTPUT_PROJ = 6,      /* [dim, dim or Hg*dv] output_proj_weights */
+    MLH_T_RMS_GAMMA2 = 7,       /* [dim]              rms2_weights */
+    MLH_T_FFN_1A = 8,           /* [ffnDim, dim]      ffn_right_1_weights (gate, SiLU branch) */
+    MLH_T_FFN_1B = 9,           /* [ffnDim, dim]      ffn_right_2_weights (up) */
+    MLH_T_FFN_2 = 10,           /* [dim, ffnDim]      ffn_left_weights (down) */
+    MLH_T_QUERY_RMS_GAMMA = 11, /* [dim]              query_RMS_weights */
+    MLH_T_KEY_RMS_GAMMA = 12,   /* [dim]              key_RMS_weights */
+    MLH_T_GATED_QUERY = 13,     /* [dim, dim]         gated_query_weights */
+    MLH_T_GDN_ALPHA_W = 14,     /* [gdnHeads, dim] */
+    MLH_T_GDN_ALPHA_B = 15,     /* [gdnHeads] */
+    MLH_T_GDN_BETA_W = 16,      /* [gdnHeads, dim] */
+    MLH_T_GDN_BETA_B = 17,      /* [gdnHeads] */
+    MLH_T_PLE_TABLE = 18,       /* [vocabSize, pleDim] */
+    MLH_T_PLE_GATE = 19,        /* [pleDim, dim] */
+    MLH_T_PLE_UP = 20,          /* [dim, pleDim] */
+    MLH_T_COUNT = 21
+};
+
+typedef struct mlh_ctx mlh_ctx;
+
+/* Last error text of a context (ctx == NULL: of the last failed mlh_create on this thread). */
+const char* mlh_last_error(const mlh_ctx* ctx);
+
+/* Number of visible HIP devices (0 when there is none; never fails). */
+int mlh_device_count(void);
+
+/* Replaces allocateMemory(true) (memory_allocation.cu:326-557): validates the
+ * hyper-parameters, allocates weights, KV pages, GDN states and scratch on
+ * device `device`, creates the stream.  Weights start zeroed. */
+int mlh_create(const mlh_hparams* hp, int device, mlh_ctx** out);
+void mlh_destroy(mlh_ctx* ctx);
+
+/* Replaces the cudaMemcpy of each tensor in loadModel (load_model.cu:366-372,
+ * 383-388,429-434,456-461).  `host` is fp32, row-major [rows, cols] exactly as
+ * stored in model.bin ([out, in]; the reference transposes to column-major for
+ * cuBLAS, this layer consumes the file order directly).  layer is the FILE
+ * block index, ignored for the two global tensors.  1-D tensors: cols = 1. */
+int mlh_upload_tensor(mlh_ctx* ctx, int layer, int tensor_id, const float* host, int rows, int cols);
+
+/* Replaces the RoPE table upload of memory_allocation.cu:383-388.  tab is the
+ * host table of getPreComputedRopeTheta (inference.cu:364-374): [maxL, headDim]. */
+int mlh_upload_rope_table(mlh_ctx* ctx, const float* tab, int n);
+
+/* Must be called once after the uploads and before any forward call: checks
+ * that every tensor the hyper-parameters require has arrived. */
+int mlh_finalize(mlh_ctx* ctx);
+
+/* Empties a sequence (length 0, GDN states zero).  seq = -1: all sequences.
+ * The reference has one implicit sequence in seqTokenIndices (network_globals.h:147-148). */
+int mlh_reset(mlh_ctx* ctx, int seq);
+int mlh_seq_len(mlh_ctx* ctx, int seq);
+int mlh_max_len(const mlh_ctx* ctx);    /* maxL of the context */
+int mlh_vocab_size(const mlh_ctx* ctx); /* vocabSize of the context */
+
+/* KV pages: every attention layer keeps K and V in pages of mlh_kv_page_size()
+ * positions; sequence s, page j lives in pool slot table[s*pagesPerSeq + j].
+ * The default table is the identity.  Replaces nothing in the reference (it has
+ * no cache, inference_orchestrator.cu:64-65). */
+int mlh_kv_page_size(void);
+int mlh_set_page_table(mlh_ctx* ctx, const int32_t* table, int n);
+
+/* Appends n tokens to sequence seq and leaves the logits of the last one
+ * readable.  Together with mlh_decode_step this replaces runInference(L)
+ * (inference.cu:376-751) as used by the token loop: the reference recomputes
+ * all L columns per token, here positions already in the cache are not redone. */
+int mlh_prefill(mlh_ctx* ctx, int seq, const int32_t* ids, int n);
+
+/* One greedy decode step for sequences 0..nseq-1: feeds last_ids[s] at each
+ * sequence's current position, appends it, returns argmax of the logits
+ * (lowest index on ties) in next_ids[s].  Replaces one iteration of the loop
+ * body inference_orchestrator.cu:64-154 (runInference + D2H of vocab*L floats
+ * + host qsort + H2D of the ids). */
+int mlh_decode_step(mlh_ctx* ctx, const int32_t* last_ids, int nseq, int32_t* next_ids);
+
+/* `steps` greedy steps without returning to the host in between: the argmax of
+ * step i is fed to step i+1 on the device.  out_ids is [steps, nseq].
+ * Replaces the whole while loop of inference_orchestrator.cu:64-160. */
+int mlh_decode_loop(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, int32_t* out_ids);
+
+/* Greedy pick (argmax of the logits, lowest index on ties) made on the device
+ * for the last position of seq that went through the LM head: the element the
+ * reference takes after its host qsort (inference_orchestrator.cu:84,112). */
+int mlh_greedy_token(mlh_ctx* ctx, int seq, int32_t* id);
+
+/* Logits [vocabSize] of the last position processed for seq
+ * (vocabScores_DEVICE, network_globals.h:170; the reference copies
+ * probabilities for all L positions, inference_orchestrator.cu:68-69). */
+int mlh_read_logits(mlh_ctx* ctx, int seq, float* out);
+
+/* Softmax of those logits (vocabScores_postSoftmax_DEVICE, inference.cu:745-749). */
+int mlh_read_probs(mlh_ctx* ctx, int seq, float* out);
+
+/* Decode steps run as replays of a captured hipGraph when enabled (default on). */
+int mlh_set_graph(mlh_ctx* ctx, int enabled);
+
+int mlh_synchronize(mlh_ctx* ctx);
+
+/* Measurement support.  Times `iters` back-to-back launches of one kernel of
+ * the decode step with HIP events on the context's stream and returns the
+ * average duration in microseconds plus the algorithmic bytes one launch moves. */
+enum {
+    MLH_K_QKV = 0,
+    MLH_K_ATTN = 1,
+    MLH_K_OPROJ = 2,
+    MLH_K_FFN_GATEUP = 3,
+    MLH_K_FFN_DOWN = 4,
+    MLH_K_LMHEAD = 5,
+    MLH_K_GDN = 6,
+    MLH_K_COPY = 7, /* plain copy of nbytes (calibration of the traffic counters) */
+    MLH_K_COUNT = 8
+};
+int mlh_time_kernel(mlh_ctx* ctx, int kernel, int layer, int nseq, int iters, double* avg_us,
+                    double* algo_bytes);
+const char* mlh_kernel_name(int kernel);
+
+/* Times `steps` decode steps (graph replays, argmax fed back on the device)
+ * with HIP events on the context's stream: total milliseconds. */
+int mlh_time_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, double* total_ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,139 @@
+// Internal declarations of the gfx950 device layer (not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "mlh.h"
+
+#define MLH_KV_PAGE 64      // positions per KV page; equals the attention key tile
+#define MLH_ATTN_WG_KEYS 256 // keys one attention workgroup covers (4 waves x one 64-key tile)
+#define MLH_WAVE 64
+
+typedef uint16_t bf16_t;
+
+// Device-side description of one transformer block.
+struct LayerDev {
+    const void* Wa;       // fused first-phase matrix [rowsA, dim]: q|k|v|[g]|[pleGate]|[gdnA|gdnB]
+    const void* Wo;       // [dim, ad]
+    const void* W13;      // [2*ffnDim, dim], row 2i = gate row i, row 2i+1 = up row i
+    const void* W2;       // [dim, ffnDim]
+    const void* pleUp;    // [dim, pleDim]
+    const void* pleTable; // [vocab, pleDim]
+    const float* g1;      // rms1 gain
+    const float* g2;      // rms2 gain
+    const float* gq;      // per-head q gain [dim] (qkRmsNorm)
+    const float* gk;
+    const float* gdnBa;   // [gdnHeads]
+    const float* gdnBb;
+    float* K;             // KV page pools [numPages, MLH_KV_PAGE, dim]
+    float* V;
+    float* S;             // GDN states [maxSeqs, gdnHeads, dv, dk]
+    int kind;
+    int rowsA, offK, offV, offG, offPle, offGa, offGb;
+    int ad;               // width of the mixing output fed to Wo
+};
+
+// Arguments shared by all kernels of a decode step.
+struct StepArgs {
+    // model
+    int dim, heads, hd, ffn, vocab, maxL, ple;
+    int gdnHeads, gdnDk, gdnDv;
+    int qkNorm, gating;
+    // batch
+    int nseq;             // active slots
+    const int* sidx;      // slot -> sequence id
+    const int* tok;       // per slot: token fed this step
+    int* pos;             // per sequence: current length (position of the fed token)
+    const int* pageTable; // [maxSeqs, pagesPerSeq]
+    int pagesPerSeq;
+    int nsplit;           // attention partials per (slot, head)
+    // activations, indexed by slot
+    float* x;             // [slots, dim] residual stream
+    float* qkv;           // [slots, maxRowsA]
+    int qkvStride;
+    float* part;          // [slots, nsplit, heads, hd + 2] attention partials (m, l, acc)
+    float* mix;           // [slots, maxAd] GDN read-out
+    float* h1;            // [slots, dim]
+    float* u;             // [slots, ffn]
+    float* logits;        // [maxSeqs, vocab] indexed by sequence id
+    float* amaxVal;       // [slots, amaxParts]
+    int* amaxIdx;
+    int amaxParts;
+    const float* rope;    // [maxL, hd]
+    const void* E;        // [vocab, dim]
+    const float* gF;
+    int* nextTok;         // [maxSeqs] greedy pick per sequence id
+    int* outIds;          // [maxSteps, slots]
+    int* stepCounter;
+    int outCapacity;
+};
+
+struct mlh_ctx {
+    mlh_hparams hp;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string err;
+    bool finalized = false;
+    bool useGraph = true;
+    int wbytes = 4; // bytes per matrix element
+
+    std::vector<LayerDev> layers;
+    std::vector<std::vector<char>> have; // [layer][tensor] uploaded flags
+    bool haveE = false, haveGF = false, haveRope = false;
+    std::vector<void*> allocs;
+
+    void* E = nullptr;
+    float* gF = nullptr;
+    float* rope = nullptr;
+
+    int pagesPerSeq = 0;
+    int nsplit = 1;
+    int maxRowsA = 0, maxAd = 0;
+    int amaxParts = 0;
+    int outCapacity = 0;
+
+    int* d_sidx = nullptr;
+    int* d_tok = nullptr;
+    int* d_pos = nullptr;
+    int* d_pageTable = nullptr;
+    int* d_outIds = nullptr;
+    int* d_next = nullptr;
+    int* d_stepCounter = nullptr;
+    int* d_prompt = nullptr;
+    int promptCapacity = 0;
+    float *x = nullptr, *qkv = nullptr, *part = nullptr, *mix = nullptr, *h1 = nullptr, *u = nullptr;
+    float *logits = nullptr, *amaxVal = nullptr, *probs = nullptr;
+    int* amaxIdx = nullptr;
+    void* copySrc = nullptr; // calibration buffers for MLH_K_COPY
+    void* copyDst = nullptr;
+    size_t copyBytes = 0;
+
+    std::vector<int> h_len; // host mirror of d_pos
+    int identityNseq = 0;   // d_sidx currently holds 0..identityNseq-1 (0 = unknown)
+
+    hipGraphExec_t graphExec[MLH_MAX_LAYERS + 1] = {};
+    int graphNseq = 0;
+    hipGraphExec_t graph = nullptr;
+};
+
+// kernels_decode.hip
+int mlh_launch_step(mlh_ctx* c, int nseq, const int* tokPtr, bool lmHead);
+int mlh_launch_one(mlh_ctx* c, int kernel, int layer, int nseq);
+double mlh_kernel_bytes(mlh_ctx* c, int kernel, int layer, int nseq);
+void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr);
+int mlh_launch_copy(mlh_ctx* c);
+int mlh_launch_probs(mlh_ctx* c, int seq);
+int mlh_init_kernels(mlh_ctx* c);
+
+#define MLH_CHECK(ctx, expr)                                                               \
+    do {                                                                                   \
+        hipError_t e_ = (expr);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            (ctx)->err = std::string(#expr) + ": " + hipGetErrorString(e_);                \
+            return -2;                                                                     \
+        }                                                                                  \
+    } while (0)
