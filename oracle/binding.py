@@ -130,7 +130,9 @@ class Weights:
                 a = model.tensor(layer, tid)
                 if a is not None:
                     t[(layer, tid)] = a
-        return cls(hp, t, bf16=bf16)
+        w = cls(hp, t, bf16=bf16)
+        w._model = model  # the arrays are borrowed views of memory the model owns
+        return w
 
 
 class Decoder:
