@@ -92,6 +92,8 @@ def main():
     ap.add_argument("--steps", type=int, default=512)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
+    ap.add_argument("--graph-steps", type=int, default=1,
+                    help="decode steps per hipGraph replay; 0 = plain launches (use 0 under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the token loop runs on a single MI355X); "
@@ -107,6 +109,7 @@ def main():
     prompt = m.random_tokens(1, 0, hp.vocabSize, PROMPT_LEN)
     dev = m.Device(hp, 0)
     dev.upload(model)
+    dev.set_graph(args.graph_steps)
 
     # warm-up: W untimed steps (this also captures the decode graph)
     dev.prefill(0, prompt)
@@ -184,7 +187,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "config 2: batch-1 greedy decode, d768 x 12 layers x 12 heads x 64, ffn 2048, "
                                "vocab 8192, fp32 weights seed 1, 64-token prompt, KV to %d" % hp.maxL,
-                   "prompt_len": PROMPT_LEN, "kv_max": int(hp.maxL), "graph": True},
+                   "prompt_len": PROMPT_LEN, "kv_max": int(hp.maxL), "steps_per_graph": args.graph_steps},
         "roofline": roofline,
         "decode_roofline": {"bound": "hbm", "bytes_per_token": mean_bytes, "achieved": step_gbps,
                             "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBPS,

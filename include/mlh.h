@@ -148,8 +148,9 @@ int mlh_read_logits(mlh_ctx* ctx, int seq, float* out);
 /* Softmax of those logits (vocabScores_postSoftmax_DEVICE, inference.cu:745-749). */
 int mlh_read_probs(mlh_ctx* ctx, int seq, float* out);
 
-/* Decode steps run as replays of a captured hipGraph when enabled (default on). */
-int mlh_set_graph(mlh_ctx* ctx, int enabled);
+/* How decode steps are issued: 0 = plain kernel launches; k >= 1 = replays of a captured
+ * hipGraph that covers k consecutive decode steps (default 1; at most 64). */
+int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
 
 int mlh_synchronize(mlh_ctx* ctx);
 

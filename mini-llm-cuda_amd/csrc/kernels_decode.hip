@@ -17,6 +17,7 @@
 
 #define WG 256
 #define WAVES (WG / MLH_WAVE)
+typedef float f32x4 __attribute__((ext_vector_type(4))); // first-class vector: arrays of it stay in registers
 #define RROWS 2 // rows one wave accumulates at a time
 
 // ----------------------------------------------------------------------------
@@ -38,22 +39,26 @@ struct WVec;
 template <>
 struct WVec<float> {
     static constexpr int N = 4;
-    static __device__ __forceinline__ void load(const float* p, float (&o)[4]) {
-        float4 v = *reinterpret_cast<const float4*>(p);
+    typedef float4 Raw;
+    static __device__ __forceinline__ Raw loadRaw(const float* p) { return *reinterpret_cast<const float4*>(p); }
+    static __device__ __forceinline__ void unpack(const Raw& v, float (&o)[4]) {
         o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
     }
+    static __device__ __forceinline__ void load(const float* p, float (&o)[4]) { unpack(loadRaw(p), o); }
     static __device__ __forceinline__ float one(const float* p) { return *p; }
 };
 template <>
 struct WVec<bf16_t> {
     static constexpr int N = 8;
-    static __device__ __forceinline__ void load(const bf16_t* p, float (&o)[8]) {
-        uint4 v = *reinterpret_cast<const uint4*>(p);
+    typedef uint4 Raw;
+    static __device__ __forceinline__ Raw loadRaw(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
+    static __device__ __forceinline__ void unpack(const Raw& v, float (&o)[8]) {
         o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
         o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
         o[4] = __uint_as_float(v.z << 16); o[5] = __uint_as_float(v.z & 0xffff0000u);
         o[6] = __uint_as_float(v.w << 16); o[7] = __uint_as_float(v.w & 0xffff0000u);
     }
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&o)[8]) { unpack(loadRaw(p), o); }
     static __device__ __forceinline__ float one(const bf16_t* p) {
         return __uint_as_float(((uint32_t)*p) << 16);
     }
@@ -91,6 +96,91 @@ __device__ __forceinline__ void rows_dot(const WT* __restrict__ W, size_t ldw, i
             for (int r = 0; r < RROWS; r++)
 #pragma unroll
                 for (int j = 0; j < N; j++) acc[r][b] = fmaf(w[r][j], xv[j], acc[r][b]);
+        }
+    }
+}
+
+// The first PF_CHUNKS 16-byte vectors per lane of each of a wave's RROWS rows, loaded ahead of the
+// kernel's prologue: the weights do not depend on the activations, so their HBM latency overlaps
+// the activation load, the RMSNorm reduction and the LDS staging.
+#define PF_CHUNKS 8
+template <typename WT>
+struct Prefetched {
+    typename WVec<WT>::Raw raw[RROWS][PF_CHUNKS];
+};
+
+template <typename WT>
+__device__ __forceinline__ void prefetch_rows(Prefetched<WT>& pf, const WT* __restrict__ W, size_t ldw,
+                                              int row0, int nrows, int cols) {
+    constexpr int N = WVec<WT>::N;
+    const int lane = threadIdx.x & (MLH_WAVE - 1);
+#pragma unroll
+    for (int r = 0; r < RROWS; r++) {
+        int row = row0 + r;
+        if (row > nrows - 1) row = nrows - 1;
+        const WT* rp = W + (size_t)row * ldw;
+#pragma unroll
+        for (int ch = 0; ch < PF_CHUNKS; ch++) {
+            const int c = (ch * MLH_WAVE + lane) * N;
+            if (c < cols) pf.raw[r][ch] = WVec<WT>::loadRaw(rp + c);
+        }
+    }
+}
+
+// rows_dot for rows whose leading chunks were prefetched; columns beyond the prefetched span are streamed.
+template <typename WT, int NB>
+__device__ __forceinline__ void rows_dot_pf(const Prefetched<WT>& pf, const WT* __restrict__ W, size_t ldw,
+                                            int row0, int nrows, int cols, const float* xs, int xstride,
+                                            float (&acc)[RROWS][NB]) {
+    constexpr int N = WVec<WT>::N;
+    const int lane = threadIdx.x & (MLH_WAVE - 1);
+#pragma unroll
+    for (int ch = 0; ch < PF_CHUNKS; ch++) {
+        const int c = (ch * MLH_WAVE + lane) * N;
+        if (c < cols) {
+            float w[RROWS][N];
+#pragma unroll
+            for (int r = 0; r < RROWS; r++) WVec<WT>::unpack(pf.raw[r][ch], w[r]);
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                float xv[N];
+#pragma unroll
+                for (int j = 0; j < N; j += 4) {
+                    float4 t = *reinterpret_cast<const float4*>(xs + b * xstride + c + j);
+                    xv[j] = t.x; xv[j + 1] = t.y; xv[j + 2] = t.z; xv[j + 3] = t.w;
+                }
+#pragma unroll
+                for (int r = 0; r < RROWS; r++)
+#pragma unroll
+                    for (int j = 0; j < N; j++) acc[r][b] = fmaf(w[r][j], xv[j], acc[r][b]);
+            }
+        }
+    }
+    if (cols > PF_CHUNKS * MLH_WAVE * N) {
+        const WT* rp[RROWS];
+#pragma unroll
+        for (int r = 0; r < RROWS; r++) {
+            int row = row0 + r;
+            if (row > nrows - 1) row = nrows - 1;
+            rp[r] = W + (size_t)row * ldw;
+        }
+        for (int c = (PF_CHUNKS * MLH_WAVE + lane) * N; c < cols; c += MLH_WAVE * N) {
+            float w[RROWS][N];
+#pragma unroll
+            for (int r = 0; r < RROWS; r++) WVec<WT>::load(rp[r] + c, w[r]);
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                float xv[N];
+#pragma unroll
+                for (int j = 0; j < N; j += 4) {
+                    float4 t = *reinterpret_cast<const float4*>(xs + b * xstride + c + j);
+                    xv[j] = t.x; xv[j + 1] = t.y; xv[j + 2] = t.z; xv[j + 3] = t.w;
+                }
+#pragma unroll
+                for (int r = 0; r < RROWS; r++)
+#pragma unroll
+                    for (int j = 0; j < N; j++) acc[r][b] = fmaf(w[r][j], xv[j], acc[r][b]);
+            }
         }
     }
 }
@@ -153,14 +243,17 @@ __global__ void __launch_bounds__(WG) k_phaseA(StepArgs a, LayerDev L, int rowsP
     float* xs = lds;
     float* red = lds + NB * a.dim;
     const int slot0 = blockIdx.y * NB;
-    rmsnorm_to_lds<NB>(a.x, a.dim, slot0, a.nseq, L.g1, a.dim, xs, a.dim, red);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int rowBase = blockIdx.x * rowsPerWg;
+    Prefetched<WT> pf;
+    prefetch_rows<WT>(pf, (const WT*)L.Wa, a.dim, rowBase + wave * RROWS, L.rowsA, a.dim);
+    rmsnorm_to_lds<NB>(a.x, a.dim, slot0, a.nseq, L.g1, a.dim, xs, a.dim, red);
     for (int r0 = wave * RROWS; r0 < rowsPerWg; r0 += WAVES * RROWS) {
         const int row0 = rowBase + r0;
         if (row0 >= L.rowsA) break;
         float acc[RROWS][NB] = {};
-        rows_dot<WT, NB>((const WT*)L.Wa, a.dim, row0, L.rowsA, a.dim, xs, a.dim, acc);
+        if (r0 == wave * RROWS) rows_dot_pf<WT, NB>(pf, (const WT*)L.Wa, a.dim, row0, L.rowsA, a.dim, xs, a.dim, acc);
+        else rows_dot<WT, NB>((const WT*)L.Wa, a.dim, row0, L.rowsA, a.dim, xs, a.dim, acc);
 #pragma unroll
         for (int r = 0; r < RROWS; r++)
 #pragma unroll
@@ -205,6 +298,32 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
     const int dim = a.dim;
     const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
 
+    // Row layout of a 64 x HD tile over the wave: LPR lanes cover one row with 16-byte pieces,
+    // RPI rows per load instruction, NLD instructions per tile.
+    constexpr int LPR = HD / 4, RPI = 64 / LPR, NLD = 64 / RPI;
+    const int lrow = lane / LPR, c4 = (lane % LPR) * 4;
+    const int ntiles = (T + 63) >> 6;
+    const int newTile = p >> 6;
+    const int tstep = a.nsplit * NW;
+    int t = sp * NW + wave;
+
+    // K tile of this wave's first tile: issued before anything else, nothing below depends on it
+    // until it is stored to LDS.  Rows at or beyond p are not read (row p comes from this step).
+    f32x4 kreg[NLD], vreg[NLD];
+#pragma unroll
+    for (int it = 0; it < NLD; it++) { kreg[it] = (f32x4)(0.f); vreg[it] = (f32x4)(0.f); }
+    size_t base = 0;
+    if (t < ntiles) {
+        const int page = a.pageTable[seq * a.pagesPerSeq + t];
+        base = ((size_t)page * MLH_KV_PAGE) * dim + h * HD;
+#pragma unroll
+        for (int it = 0; it < NLD; it++) {
+            const int row = it * RPI + lrow;
+            kreg[it] = ((t << 6) + row < p) ? *reinterpret_cast<const f32x4*>(L.K + base + (size_t)row * dim + c4)
+                                            : (f32x4)(0.f);
+        }
+    }
+
     for (int i = tid; i < HD; i += NW * 64) {
         qs[i] = qkv[h * HD + i];
         ks[i] = qkv[L.offK + h * HD + i];
@@ -231,8 +350,6 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
     }
     __syncthreads();
 
-    const int ntiles = (T + 63) >> 6;
-    const int newTile = p >> 6;
     float* tile = tiles + wave * 64 * LDK;
     const float scale = sqrtf((float)HD);
     float m_run = -1.0e30f, l_run = 0.f;
@@ -240,9 +357,7 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
 #pragma unroll
     for (int e = 0; e < EPL; e++) acc[e] = 0.f;
 
-    for (int t = sp * NW + wave; t < ntiles; t += a.nsplit * NW) {
-        const int page = a.pageTable[seq * a.pagesPerSeq + t];
-        const size_t base = ((size_t)page * MLH_KV_PAGE) * dim + h * HD;
+    for (; t < ntiles; t += tstep) {
         const int j0 = t << 6;
         if (t == newTile) { // append this step's K/V row (only the owning wave writes it)
             const size_t o = base + (size_t)(p - j0) * dim;
@@ -251,18 +366,20 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
                 L.V[o + i] = vn[i];
             }
         }
-        // ---- stage K tile: 64 rows x HD floats, coalesced 16-byte loads ----
-        constexpr int LPR = HD / 4; // lanes per row
-        constexpr int RPI = 64 / LPR; // rows per load instruction
+        // ---- V tile loads in flight while the scores are computed ----
 #pragma unroll
-        for (int it = 0; it < 64 / RPI; it++) {
-            const int row = it * RPI + lane / LPR;
-            const int c4 = (lane % LPR) * 4;
-            const int j = j0 + row;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (j < p) v = *reinterpret_cast<const float4*>(L.K + base + (size_t)row * dim + c4);
-            else if (j == p) v = *reinterpret_cast<const float4*>(ks + c4);
-            *reinterpret_cast<float4*>(tile + row * LDK + c4) = v;
+        for (int it = 0; it < NLD; it++) {
+            const int row = it * RPI + lrow;
+            vreg[it] = (j0 + row < p) ? *reinterpret_cast<const f32x4*>(L.V + base + (size_t)row * dim + c4)
+                                      : (f32x4)(0.f);
+        }
+        // ---- K tile to LDS (row p taken from this step's key) ----
+#pragma unroll
+        for (int it = 0; it < NLD; it++) {
+            const int row = it * RPI + lrow;
+            f32x4 v = kreg[it];
+            if (j0 + row == p) v = *reinterpret_cast<const f32x4*>(ks + c4);
+            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
         }
         __builtin_amdgcn_wave_barrier();
         // ---- scores: lane <-> key ----
@@ -284,16 +401,25 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
         l_run = l_run * corr + wave_sum(e);
         m_run = m_new;
         __builtin_amdgcn_wave_barrier();
-        // ---- stage V tile over the K tile ----
+        // ---- V tile over the K tile ----
 #pragma unroll
-        for (int it = 0; it < 64 / RPI; it++) {
-            const int row = it * RPI + lane / LPR;
-            const int c4 = (lane % LPR) * 4;
-            const int j = j0 + row;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (j < p) v = *reinterpret_cast<const float4*>(L.V + base + (size_t)row * dim + c4);
-            else if (j == p) v = *reinterpret_cast<const float4*>(vn + c4);
-            *reinterpret_cast<float4*>(tile + row * LDK + c4) = v;
+        for (int it = 0; it < NLD; it++) {
+            const int row = it * RPI + lrow;
+            f32x4 v = vreg[it];
+            if (j0 + row == p) v = *reinterpret_cast<const f32x4*>(vn + c4);
+            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
+        }
+        // ---- next tile's K loads in flight during the P.V accumulation ----
+        const int tn = t + tstep;
+        if (tn < ntiles) {
+            const int page = a.pageTable[seq * a.pagesPerSeq + tn];
+            base = ((size_t)page * MLH_KV_PAGE) * dim + h * HD;
+#pragma unroll
+            for (int it = 0; it < NLD; it++) {
+                const int row = it * RPI + lrow;
+                kreg[it] = ((tn << 6) + row < p) ? *reinterpret_cast<const f32x4*>(L.K + base + (size_t)row * dim + c4)
+                                                 : (f32x4)(0.f);
+            }
         }
         __builtin_amdgcn_wave_barrier();
         // ---- acc[dim] = acc*corr + sum_j e_j V[j][dim] : lane <-> dim ----
@@ -407,6 +533,8 @@ __global__ void __launch_bounds__(WG) k_oproj(StepArgs a, LayerDev L, int rowsPe
     float* as = lds;             // [NB][ad]
     float* es = lds + NB * ad;   // [NB][pl]
     const int slot0 = blockIdx.y * NB, tid = threadIdx.x;
+    Prefetched<WT> pf;
+    prefetch_rows<WT>(pf, (const WT*)L.Wo, ad, blockIdx.x * rowsPerWg + (tid >> 6) * RROWS, a.dim, ad);
 #pragma unroll
     for (int b = 0; b < NB; b++) {
         const int slot = slot0 + b;
@@ -454,7 +582,8 @@ __global__ void __launch_bounds__(WG) k_oproj(StepArgs a, LayerDev L, int rowsPe
         const int row0 = rowBase + r0;
         if (row0 >= a.dim) break;
         float acc[RROWS][NB] = {};
-        rows_dot<WT, NB>((const WT*)L.Wo, ad, row0, a.dim, ad, as, ad, acc);
+        if (r0 == wave * RROWS) rows_dot_pf<WT, NB>(pf, (const WT*)L.Wo, ad, row0, a.dim, ad, as, ad, acc);
+        else rows_dot<WT, NB>((const WT*)L.Wo, ad, row0, a.dim, ad, as, ad, acc);
         if (pl > 0) rows_dot<WT, NB>((const WT*)L.pleUp, pl, row0, a.dim, pl, es, pl, acc);
 #pragma unroll
         for (int r = 0; r < RROWS; r++)
@@ -480,15 +609,18 @@ __global__ void __launch_bounds__(WG) k_ffn13(StepArgs a, LayerDev L, int pairsP
     float* xs = lds;
     float* red = lds + NB * a.dim;
     const int slot0 = blockIdx.y * NB;
-    rmsnorm_to_lds<NB>(a.h1, a.dim, slot0, a.nseq, L.g2, a.dim, xs, a.dim, red);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int pairBase = blockIdx.x * pairsPerWg;
+    Prefetched<WT> pf;
+    prefetch_rows<WT>(pf, (const WT*)L.W13, a.dim, 2 * (pairBase + wave), 2 * a.ffn, a.dim);
+    rmsnorm_to_lds<NB>(a.h1, a.dim, slot0, a.nseq, L.g2, a.dim, xs, a.dim, red);
     static_assert(RROWS == 2, "one wave handles one gate/up pair per pass");
     for (int p0 = wave; p0 < pairsPerWg; p0 += WAVES) {
         const int pr = pairBase + p0;
         if (pr >= a.ffn) break;
         float acc[RROWS][NB] = {};
-        rows_dot<WT, NB>((const WT*)L.W13, a.dim, 2 * pr, 2 * a.ffn, a.dim, xs, a.dim, acc);
+        if (p0 == wave) rows_dot_pf<WT, NB>(pf, (const WT*)L.W13, a.dim, 2 * pr, 2 * a.ffn, a.dim, xs, a.dim, acc);
+        else rows_dot<WT, NB>((const WT*)L.W13, a.dim, 2 * pr, 2 * a.ffn, a.dim, xs, a.dim, acc);
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             const float g = wave_sum(acc[0][b]);
@@ -506,6 +638,8 @@ __global__ void __launch_bounds__(WG) k_down(StepArgs a, LayerDev L, int rowsPer
     extern __shared__ float lds[];
     float* us = lds;
     const int slot0 = blockIdx.y * NB, tid = threadIdx.x;
+    Prefetched<WT> pf;
+    prefetch_rows<WT>(pf, (const WT*)L.W2, a.ffn, blockIdx.x * rowsPerWg + (tid >> 6) * RROWS, a.dim, a.ffn);
 #pragma unroll
     for (int b = 0; b < NB; b++)
         for (int i = tid; i < a.ffn; i += WG)
@@ -517,7 +651,8 @@ __global__ void __launch_bounds__(WG) k_down(StepArgs a, LayerDev L, int rowsPer
         const int row0 = rowBase + r0;
         if (row0 >= a.dim) break;
         float acc[RROWS][NB] = {};
-        rows_dot<WT, NB>((const WT*)L.W2, a.ffn, row0, a.dim, a.ffn, us, a.ffn, acc);
+        if (r0 == wave * RROWS) rows_dot_pf<WT, NB>(pf, (const WT*)L.W2, a.ffn, row0, a.dim, a.ffn, us, a.ffn, acc);
+        else rows_dot<WT, NB>((const WT*)L.W2, a.ffn, row0, a.dim, a.ffn, us, a.ffn, acc);
 #pragma unroll
         for (int r = 0; r < RROWS; r++)
 #pragma unroll
@@ -545,9 +680,11 @@ __global__ void __launch_bounds__(WG) k_lmhead(StepArgs a, int rowsPerWg) {
     float* bv = red + WAVES;                 // [WAVES][NB]
     int* bi = (int*)(bv + WAVES * NB);       // [WAVES][NB]
     const int slot0 = blockIdx.y * NB;
-    rmsnorm_to_lds<NB>(a.x, a.dim, slot0, a.nseq, a.gF, a.dim, xs, a.dim, red);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int rowBase = blockIdx.x * rowsPerWg;
+    Prefetched<WT> pf;
+    prefetch_rows<WT>(pf, (const WT*)a.E, a.dim, rowBase + wave * RROWS, a.vocab, a.dim);
+    rmsnorm_to_lds<NB>(a.x, a.dim, slot0, a.nseq, a.gF, a.dim, xs, a.dim, red);
     float best[NB];
     int bidx[NB];
 #pragma unroll
@@ -556,7 +693,8 @@ __global__ void __launch_bounds__(WG) k_lmhead(StepArgs a, int rowsPerWg) {
         const int row0 = rowBase + r0;
         if (row0 >= a.vocab) break;
         float acc[RROWS][NB] = {};
-        rows_dot<WT, NB>((const WT*)a.E, a.dim, row0, a.vocab, a.dim, xs, a.dim, acc);
+        if (r0 == wave * RROWS) rows_dot_pf<WT, NB>(pf, (const WT*)a.E, a.dim, row0, a.vocab, a.dim, xs, a.dim, acc);
+        else rows_dot<WT, NB>((const WT*)a.E, a.dim, row0, a.vocab, a.dim, xs, a.dim, acc);
 #pragma unroll
         for (int r = 0; r < RROWS; r++)
 #pragma unroll
@@ -687,7 +825,7 @@ void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr) {
     a.nextTok = c->d_next; a.outIds = c->d_outIds; a.stepCounter = c->d_stepCounter; a.outCapacity = c->outCapacity;
 }
 
-#define LMHEAD_ROWS_PER_WG 32
+#define LMHEAD_ROWS_PER_WG 16
 #define GEMV_ROWS_PER_WG 8
 
 template <typename WT, int NB>

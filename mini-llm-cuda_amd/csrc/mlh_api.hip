@@ -74,7 +74,7 @@ extern "C" void mlh_destroy(mlh_ctx* c) {
     if (!c) return;
     (void)hipSetDevice(c->device);
     if (c->stream) (void)hipStreamSynchronize(c->stream);
-    if (c->graph) (void)hipGraphExecDestroy(c->graph);
+    for (int i = 0; i < 2; i++) if (c->graphExec[i]) (void)hipGraphExecDestroy(c->graphExec[i]);
     for (void* p : c->allocs) (void)hipFree(p);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
@@ -168,7 +168,7 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         return bail(-1);
     }
 
-    c->amaxParts = (V + 31) / 32;
+    c->amaxParts = (V + 15) / 16; // one partial per LM-head workgroup (16 rows each)
     c->outCapacity = hp.maxL;
     c->promptCapacity = hp.maxL;
     if ((rc = dev_alloc(c, &c->d_sidx, S)) || (rc = dev_alloc(c, &c->d_tok, S)) ||
@@ -437,27 +437,38 @@ extern "C" int mlh_prefill(mlh_ctx* c, int seq, const int32_t* ids, int n) {
     return 0;
 }
 
-static int ensure_graph(mlh_ctx* c, int nseq) {
-    if (c->graph && c->graphNseq == nseq) return 0;
-    if (c->graph) { (void)hipGraphExecDestroy(c->graph); c->graph = nullptr; }
+// Captures `k` consecutive decode steps into one executable graph (slot 0: one step, slot 1: graphSteps steps).
+static int ensure_graph(mlh_ctx* c, int slot, int nseq, int k) {
+    if (c->graphExec[slot] && c->graphNseqOf[slot] == nseq && c->graphStepsOf[slot] == k) return 0;
+    if (c->graphExec[slot]) { (void)hipGraphExecDestroy(c->graphExec[slot]); c->graphExec[slot] = nullptr; }
     hipGraph_t g = nullptr;
     MLH_CHECK(c, hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal));
-    int rc = mlh_launch_step(c, nseq, c->d_tok, true);
+    int rc = 0;
+    for (int i = 0; i < k && rc == 0; i++) rc = mlh_launch_step(c, nseq, c->d_tok, true);
     hipError_t e = hipStreamEndCapture(c->stream, &g);
     if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
     if (e != hipSuccess) { c->err = std::string("hipStreamEndCapture: ") + hipGetErrorString(e); return -2; }
-    e = hipGraphInstantiate(&c->graph, g, nullptr, nullptr, 0);
+    e = hipGraphInstantiate(&c->graphExec[slot], g, nullptr, nullptr, 0);
     (void)hipGraphDestroy(g);
-    if (e != hipSuccess) { c->graph = nullptr; c->err = std::string("hipGraphInstantiate: ") + hipGetErrorString(e); return -2; }
-    c->graphNseq = nseq;
+    if (e != hipSuccess) { c->graphExec[slot] = nullptr; c->err = std::string("hipGraphInstantiate: ") + hipGetErrorString(e); return -2; }
+    c->graphNseqOf[slot] = nseq;
+    c->graphStepsOf[slot] = k;
     return 0;
 }
 
 static int run_steps(mlh_ctx* c, int nseq, int steps) {
     int rc;
-    if (c->useGraph) {
-        if ((rc = ensure_graph(c, nseq))) return rc;
-        for (int i = 0; i < steps; i++) MLH_CHECK(c, hipGraphLaunch(c->graph, c->stream));
+    if (c->graphSteps >= 1) {
+        const int k = c->graphSteps;
+        int done = 0;
+        if (k > 1 && steps >= k) {
+            if ((rc = ensure_graph(c, 1, nseq, k))) return rc;
+            for (; done + k <= steps; done += k) MLH_CHECK(c, hipGraphLaunch(c->graphExec[1], c->stream));
+        }
+        if (done < steps) {
+            if ((rc = ensure_graph(c, 0, nseq, 1))) return rc;
+            for (; done < steps; done++) MLH_CHECK(c, hipGraphLaunch(c->graphExec[0], c->stream));
+        }
     } else {
         for (int i = 0; i < steps; i++)
             if ((rc = mlh_launch_step(c, nseq, c->d_tok, true))) return rc;
@@ -500,7 +511,6 @@ extern "C" int mlh_time_decode(mlh_ctx* c, const int32_t* first, int nseq, int s
     int rc = check_decode(c, first, nseq, steps);
     if (rc) return rc;
     if (!totalMs) { c->err = "null output"; return -1; }
-    if (c->useGraph && (rc = ensure_graph(c, nseq))) return rc;
     hipEvent_t e0, e1;
     MLH_CHECK(c, hipEventCreate(&e0));
     MLH_CHECK(c, hipEventCreate(&e1));
@@ -540,9 +550,10 @@ extern "C" int mlh_read_probs(mlh_ctx* c, int seq, float* out) {
     return 0;
 }
 
-extern "C" int mlh_set_graph(mlh_ctx* c, int enabled) {
+extern "C" int mlh_set_graph(mlh_ctx* c, int stepsPerGraph) {
     if (!c) return -1;
-    c->useGraph = enabled != 0;
+    if (stepsPerGraph < 0 || stepsPerGraph > 64) { c->err = "steps per graph must be 0..64"; return -1; }
+    c->graphSteps = stepsPerGraph;
     return 0;
 }
 

@@ -78,7 +78,6 @@ struct mlh_ctx {
     hipStream_t stream = nullptr;
     std::string err;
     bool finalized = false;
-    bool useGraph = true;
     int wbytes = 4; // bytes per matrix element
 
     std::vector<LayerDev> layers;
@@ -115,9 +114,10 @@ struct mlh_ctx {
     std::vector<int> h_len; // host mirror of d_pos
     int identityNseq = 0;   // d_sidx currently holds 0..identityNseq-1 (0 = unknown)
 
-    hipGraphExec_t graphExec[MLH_MAX_LAYERS + 1] = {};
-    int graphNseq = 0;
-    hipGraphExec_t graph = nullptr;
+    int graphSteps = 1;                 // 0: eager launches; k >= 1: one graph replay covers k decode steps
+    hipGraphExec_t graphExec[2] = {};   // [0]: one step, [1]: graphSteps steps
+    int graphNseqOf[2] = {0, 0};
+    int graphStepsOf[2] = {0, 0};
 };
 
 // kernels_decode.hip
