@@ -152,6 +152,12 @@ int mlh_read_probs(mlh_ctx* ctx, int seq, float* out);
  * hipGraph that covers k consecutive decode steps (default 1; at most 64). */
 int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
 
+/* Batch-1 decode (nseq = 1) runs, when enabled (default) and the shape allows it, as ONE
+ * cooperative launch of a persistent kernel that decodes all requested steps: the ~60 dependent
+ * phases of a token are separated by grid barriers instead of kernel launches.  Disabled, or for
+ * nseq > 1, the step is a sequence of kernels issued as mlh_set_graph says. */
+int mlh_set_persistent(mlh_ctx* ctx, int enabled);
+
 int mlh_synchronize(mlh_ctx* ctx);
 
 /* Measurement support.  Times `iters` back-to-back launches of one kernel of

@@ -84,6 +84,7 @@ _sigs_dev = {
     "mlh_read_logits": (c_int, [c_void_p, c_int, c_void_p]),
     "mlh_read_probs": (c_int, [c_void_p, c_int, c_void_p]),
     "mlh_set_graph": (c_int, [c_void_p, c_int]),
+    "mlh_set_persistent": (c_int, [c_void_p, c_int]),
     "mlh_synchronize": (c_int, [c_void_p]),
     "mlh_time_kernel": (c_int, [c_void_p, c_int, c_int, c_int, c_int, _P(c_double), _P(c_double)]),
     "mlh_kernel_name": (c_char_p, [c_int]),
@@ -299,6 +300,9 @@ class Device:
 
     def set_graph(self, enabled):
         self._check(dev.mlh_set_graph(self._h, int(enabled)))
+
+    def set_persistent(self, enabled):
+        self._check(dev.mlh_set_persistent(self._h, int(enabled)))
 
     def synchronize(self):
         self._check(dev.mlh_synchronize(self._h))

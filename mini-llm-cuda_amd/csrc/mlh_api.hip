@@ -1,5 +1,7 @@
 // C ABI of the device layer: context life cycle, weight upload, sequence state,
 // decode/prefill entry points, hipGraph capture and measurement helpers.
+#include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -182,6 +184,17 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         (rc = dev_alloc(c, &c->probs, V)) || (rc = dev_alloc(c, &c->amaxVal, (size_t)S * c->amaxParts)) ||
         (rc = dev_alloc(c, &c->amaxIdx, (size_t)S * c->amaxParts)))
         return bail(rc);
+    {
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, device) != hipSuccess) { c->err = "hipGetDeviceProperties failed"; return bail(-2); }
+        c->numCUs = prop.multiProcessorCount;
+        c->coopLaunch = prop.cooperativeLaunch != 0;
+    }
+    if ((rc = dev_alloc(c, &c->d_layers, (size_t)hp.transformers)) || (rc = dev_alloc(c, &c->d_sync, 64 * 24)) ||
+        (rc = dev_alloc(c, &c->pamaxVal, (size_t)c->numCUs)) || (rc = dev_alloc(c, &c->pamaxIdx, (size_t)c->numCUs)) ||
+        (rc = dev_alloc(c, &c->kvPart, (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2))))
+        return bail(rc);
+    if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1)))) return bail(rc);
     c->copyBytes = (size_t)256 << 20;
     char *cs, *cd;
     if ((rc = dev_alloc(c, &cs, c->copyBytes)) || (rc = dev_alloc(c, &cd, c->copyBytes))) return bail(rc);
@@ -344,6 +357,7 @@ extern "C" int mlh_finalize(mlh_ctx* c) {
     (void)hipSetDevice(c->device);
     int rc = mlh_init_kernels(c);
     if (rc) return rc;
+    MLH_CHECK(c, hipMemcpy(c->d_layers, c->layers.data(), c->layers.size() * sizeof(LayerDev), hipMemcpyHostToDevice));
     MLH_CHECK(c, hipDeviceSynchronize());
     c->finalized = true;
     return 0;
@@ -456,8 +470,41 @@ static int ensure_graph(mlh_ctx* c, int slot, int nseq, int k) {
     return 0;
 }
 
+static bool use_persistent(const mlh_ctx* c, int nseq) {
+    return nseq == 1 && c->usePersistent && mlh_persistent_supported(c);
+}
+
+// After the stream has drained: a persistent launch that gave up a bounded wait leaves its flag set.
+static void dump_persistent_timing(mlh_ctx* c) {
+    if (!c->d_timing) return;
+    const int n = 16 * c->hp.transformers;
+    std::vector<unsigned long long> t(n);
+    if (hipMemcpy(t.data(), c->d_timing, (size_t)n * 8, hipMemcpyDeviceToHost) != hipSuccess) return;
+    static const char* names[15] = {"A.norm", "A.rows", "A->B sync", "B.mix", "B->C sync", "C.prologue", "C.rows", "C->D sync",
+                                    "D.norm", "D.rows", "D->E sync", "E.load", "E.rows", "E->A sync", "x.load"};
+    double tot[15] = {0};
+    for (int l = 0; l < c->hp.transformers; l++)
+        for (int k = 0; k < 15; k++) tot[k] += (double)(t[l * 16 + k + 1] - t[l * 16 + k]) / 100.0; // 100 MHz clock
+    fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
+    double sum = 0;
+    for (int k = 0; k < 15; k++) { fprintf(stderr, " %s=%.2f", names[k], tot[k] / c->hp.transformers); sum += tot[k] / c->hp.transformers; }
+    fprintf(stderr, " | layer total %.2f\n", sum);
+}
+
+static int check_persistent_abort(mlh_ctx* c) {
+    dump_persistent_timing(c);
+    unsigned flag = 0;
+    MLH_CHECK(c, hipMemcpy(&flag, c->d_sync + 64 * 20, 4, hipMemcpyDeviceToHost));
+    if (flag) {
+        c->err = "persistent decode kernel abandoned a grid-barrier wait (were all workgroups resident?)";
+        return -3;
+    }
+    return 0;
+}
+
 static int run_steps(mlh_ctx* c, int nseq, int steps) {
     int rc;
+    if (use_persistent(c, nseq)) return mlh_launch_persistent(c, steps);
     if (c->graphSteps >= 1) {
         const int k = c->graphSteps;
         int done = 0;
@@ -499,6 +546,7 @@ extern "C" int mlh_decode_loop(mlh_ctx* c, const int32_t* first, int nseq, int s
     if ((rc = run_steps(c, nseq, steps))) return rc;
     MLH_CHECK(c, hipMemcpyAsync(out, c->d_outIds, (size_t)steps * nseq * 4, hipMemcpyDeviceToHost, c->stream));
     MLH_CHECK(c, hipStreamSynchronize(c->stream));
+    if (use_persistent(c, nseq) && (rc = check_persistent_abort(c))) return rc;
     for (int s = 0; s < nseq; s++) c->h_len[s] += steps;
     return 0;
 }
@@ -526,6 +574,7 @@ extern "C" int mlh_time_decode(mlh_ctx* c, const int32_t* first, int nseq, int s
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (rc) return rc;
+    if (use_persistent(c, nseq) && (rc = check_persistent_abort(c))) return rc;
     *totalMs = ms;
     for (int s = 0; s < nseq; s++) c->h_len[s] += steps;
     return 0;
@@ -554,6 +603,12 @@ extern "C" int mlh_set_graph(mlh_ctx* c, int stepsPerGraph) {
     if (!c) return -1;
     if (stepsPerGraph < 0 || stepsPerGraph > 64) { c->err = "steps per graph must be 0..64"; return -1; }
     c->graphSteps = stepsPerGraph;
+    return 0;
+}
+
+extern "C" int mlh_set_persistent(mlh_ctx* c, int enabled) {
+    if (!c) return -1;
+    c->usePersistent = enabled != 0;
     return 0;
 }
 

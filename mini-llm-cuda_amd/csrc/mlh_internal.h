@@ -111,6 +111,17 @@ struct mlh_ctx {
     void* copyDst = nullptr;
     size_t copyBytes = 0;
 
+    // persistent batch-1 decode kernel
+    int numCUs = 0;
+    bool coopLaunch = false;
+    bool usePersistent = true;
+    LayerDev* d_layers = nullptr;  // device copy of `layers`
+    unsigned* d_sync = nullptr;    // barrier words + abort flag
+    float* pamaxVal = nullptr;     // [numCUs]
+    int* pamaxIdx = nullptr;
+    float* kvPart = nullptr;       // [heads, pagesPerSeq, headDim + 2]
+    unsigned long long* d_timing = nullptr; // phase timestamps (set MLH_PERSIST_TIMING=1), 16 per layer
+
     std::vector<int> h_len; // host mirror of d_pos
     int identityNseq = 0;   // d_sidx currently holds 0..identityNseq-1 (0 = unknown)
 
@@ -128,6 +139,10 @@ void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr);
 int mlh_launch_copy(mlh_ctx* c);
 int mlh_launch_probs(mlh_ctx* c, int seq);
 int mlh_init_kernels(mlh_ctx* c);
+
+// kernels_persistent.hip
+bool mlh_persistent_supported(const mlh_ctx* c);
+int mlh_launch_persistent(mlh_ctx* c, int steps);
 
 #define MLH_CHECK(ctx, expr)                                                               \
     do {                                                                                   \

@@ -49,12 +49,15 @@ def make(pkg, orc, hp, seed, bf16=False):
     return model, dev, w
 
 
+@pytest.mark.parametrize("persistent", [1, 0], ids=["persistent", "kernels"])
 @pytest.mark.parametrize("kind,plen,steps", [("attn", 16, 40), ("attn_flags", 16, 40), ("hybrid", 16, 40),
                                              ("hybrid_flags", 16, 40), ("hd128", 16, 40), ("attn_long", 300, 12)])
-def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps):
-    """Every decode step's logits against the float64 oracle, ids by the gap rule."""
+def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
+    """Every decode step's logits against the float64 oracle, ids by the gap rule -- once through the
+    persistent single-launch kernel, once through the per-phase kernel sequence."""
     hp = small_cfg(pkg, kind)
     model, dev, w = make(pkg, orc, hp, seed=11)
+    dev.set_persistent(persistent)
     prompt = pkg.random_tokens(11, 0, hp.vocabSize, plen)
     dev.prefill(0, prompt)
     ids, logits = [], []
@@ -69,16 +72,26 @@ def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps):
     dev.close()
 
 
-def test_config1_golden_horizon(pkg, orc):
-    """Configuration 1 at full size: 16-token prompt, 128 greedy steps on the device loop."""
+@pytest.mark.parametrize("persistent", [1, 0], ids=["persistent", "kernels"])
+def test_config1_golden_horizon(pkg, orc, persistent):
+    """Configuration 1 at full size: 16-token prompt, 128 greedy steps on the device loop, checked
+    against the oracle and against the committed golden ids."""
+    import os
+    from conftest import GOLDEN
     hp = pkg.config(1)
     model, dev, w = make(pkg, orc, hp, seed=0)
+    dev.set_persistent(persistent)
     prompt = pkg.random_tokens(0, 0, hp.vocabSize, 16)
     ids, _ = dev.generate(prompt, 128)
     assert len(ids) == 128
     dec = orc.Decoder(w, "f64")
     exact, tol = check_greedy_against_oracle(dec, prompt, ids, GAP_TOL, what="cfg1")
     assert exact + tol == 128
+    g = np.load(os.path.join(GOLDEN, "cfg1_golden.npz"))
+    if tol == 0:
+        assert np.array_equal(ids, g["ids"])
+    # logits after the last fed token (generated token 127 of 128) against the golden full logits of step 127
+    assert_logits_close(dev.logits(0), g["full_logits"][3], FP32_RTOL, "cfg1 golden step 127")
     dev.close()
 
 
@@ -87,9 +100,10 @@ def test_graph_replay_equals_eager(pkg, orc):
     with host work and synchronisation in between."""
     hp = small_cfg(pkg, "hybrid")
     model, dev, w = make(pkg, orc, hp, seed=5)
+    dev.set_persistent(0)  # graphs concern the per-phase kernel sequence
     prompt = pkg.random_tokens(5, 0, hp.vocabSize, 12)
     out = {}
-    for mode in (0, 1):
+    for mode in (0, 1, 4):
         dev.set_graph(mode)
         dev.reset()
         dev.prefill(0, prompt)
@@ -101,8 +115,15 @@ def test_graph_replay_equals_eager(pkg, orc):
             tok = int(o[-1, 0])
             dev.synchronize()
         out[mode] = (np.concatenate(chunks), dev.logits(0))
-    assert np.array_equal(out[0][0], out[1][0])
-    assert np.array_equal(out[0][1], out[1][1])
+    for mode in (1, 4):
+        assert np.array_equal(out[0][0], out[mode][0])
+        assert np.array_equal(out[0][1], out[mode][1])
+    # and the persistent kernel produces the same ids from the same state
+    dev.set_persistent(1)
+    dev.reset()
+    dev.prefill(0, prompt)
+    o = dev.decode_loop([dev.greedy_token(0)], 32)
+    assert np.array_equal(o[:, 0], out[0][0])
     dev.close()
 
 
