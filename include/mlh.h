@@ -152,7 +152,7 @@ int mlh_read_probs(mlh_ctx* ctx, int seq, float* out);
  * hipGraph that covers k consecutive decode steps (default 1; at most 64). */
 int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
 
-/* Batch-1 decode (nseq = 1) runs, when enabled (default) and the shape allows it, as ONE
+/* Batch-1 decode (nseq = 1) runs, when enabled (default off) and the shape allows it, as ONE
  * cooperative launch of a persistent kernel that decodes all requested steps: the ~60 dependent
  * phases of a token are separated by grid barriers instead of kernel launches.  Disabled, or for
  * nseq > 1, the step is a sequence of kernels issued as mlh_set_graph says. */
@@ -172,11 +172,20 @@ enum {
     MLH_K_LMHEAD = 5,
     MLH_K_GDN = 6,
     MLH_K_COPY = 7, /* plain copy of nbytes (calibration of the traffic counters) */
-    MLH_K_COUNT = 8
+    MLH_K_EMBED = 8,
+    MLH_K_FINISH = 9,
+    MLH_K_COUNT = 10
 };
 int mlh_time_kernel(mlh_ctx* ctx, int kernel, int layer, int nseq, int iters, double* avg_us,
                     double* algo_bytes);
 const char* mlh_kernel_name(int kernel);
+
+/* In-sequence kernel times: runs `steps` decode steps as plain launches with a HIP event after
+ * every kernel on the context's stream and returns, per kernel id, the mean time from the previous
+ * event to its own (its run time plus the launch gap before it) in us_per_launch[MLH_K_COUNT] and
+ * the launches per step in launches_per_step[MLH_K_COUNT].  The sequences advance by `steps`. */
+int mlh_profile_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, double* us_per_launch,
+                       int32_t* launches_per_step);
 
 /* Times `steps` decode steps (graph replays, argmax fed back on the device)
  * with HIP events on the context's stream: total milliseconds. */

@@ -29,7 +29,8 @@ DTYPE_F32, DTYPE_BF16 = 0, 1
  T_GDN_BETA_W, T_GDN_BETA_B, T_PLE_TABLE, T_PLE_GATE, T_PLE_UP, T_COUNT) = range(22)
 
 # kernel ids (include/mlh.h)
-K_QKV, K_ATTN, K_OPROJ, K_FFN_GATEUP, K_FFN_DOWN, K_LMHEAD, K_GDN, K_COPY = range(8)
+K_QKV, K_ATTN, K_OPROJ, K_FFN_GATEUP, K_FFN_DOWN, K_LMHEAD, K_GDN, K_COPY, K_EMBED, K_FINISH = range(10)
+K_COUNT = 10
 
 
 class HParams(ctypes.Structure):
@@ -89,6 +90,7 @@ _sigs_dev = {
     "mlh_time_kernel": (c_int, [c_void_p, c_int, c_int, c_int, c_int, _P(c_double), _P(c_double)]),
     "mlh_kernel_name": (c_char_p, [c_int]),
     "mlh_time_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double)]),
+    "mlh_profile_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double), _P(c_int32)]),
 }
 _sigs_host = {
     "mll_hparams_reference_defaults": (None, [_P(HParams)]),
@@ -311,6 +313,15 @@ class Device:
         us, nbytes = c_double(), c_double()
         self._check(dev.mlh_time_kernel(self._h, kernel, layer, nseq, iters, byref(us), byref(nbytes)))
         return us.value, nbytes.value
+
+    def profile_decode(self, first_ids, steps):
+        """In-sequence mean microseconds per launch (run time plus the launch gap before it) and
+        launches per step, by kernel name, over `steps` plain-launch decode steps."""
+        a = np.ascontiguousarray(first_ids, dtype=np.int32)
+        us = (c_double * K_COUNT)()
+        n = (c_int32 * K_COUNT)()
+        self._check(dev.mlh_profile_decode(self._h, a.ctypes.data, a.size, steps, us, n))
+        return {dev.mlh_kernel_name(k).decode(): (us[k], n[k]) for k in range(K_COUNT) if n[k] > 0}
 
     def generate(self, prompt, max_new):
         """Greedy generation on sequence 0 (mll_generate): returns (ids, elapsed ms)."""

@@ -930,22 +930,39 @@ int mlh_launch_step(mlh_ctx* c, int nseq, const int* tokPtr, bool lmHead) {
     StepArgs a;
     mlh_fill_args(c, a, nseq, tokPtr);
     hipStream_t st = c->stream;
+    // measurement hook: an event after every launch, tagged with the kernel id
+    auto mark = [&](int id) {
+        if (!c->profEvents) return;
+        hipEvent_t ev;
+        if (hipEventCreate(&ev) != hipSuccess) return;
+        (void)hipEventRecord(ev, st);
+        c->profEvents->push_back(ev);
+        c->profIds->push_back(id);
+    };
     if (c->hp.weightDtype == MLH_DTYPE_BF16)
         hipLaunchKernelGGL((k_embed<bf16_t>), dim3(ceil_div(a.dim, WG), nseq), dim3(WG), 0, st, a);
     else
         hipLaunchKernelGGL((k_embed<float>), dim3(ceil_div(a.dim, WG), nseq), dim3(WG), 0, st, a);
+    mark(MLH_K_EMBED);
     for (int t = c->hp.transformers - 1; t >= 0; t--) { // file block 0 is the top (inference.cu:384-385)
         const LayerDev& L = c->layers[t];
         launch_gemv(c, MLH_K_QKV, a, L);
+        mark(MLH_K_QKV);
         if (launch_mix(c, a, L) != 0) return -1;
+        mark(L.kind == MLH_KIND_ATTENTION ? MLH_K_ATTN : MLH_K_GDN);
         launch_gemv(c, MLH_K_OPROJ, a, L);
+        mark(MLH_K_OPROJ);
         launch_gemv(c, MLH_K_FFN_GATEUP, a, L);
+        mark(MLH_K_FFN_GATEUP);
         launch_gemv(c, MLH_K_FFN_DOWN, a, L);
+        mark(MLH_K_FFN_DOWN);
     }
     if (lmHead) {
         launch_gemv(c, MLH_K_LMHEAD, a, c->layers[0]);
+        mark(MLH_K_LMHEAD);
         hipLaunchKernelGGL(k_finish, dim3(1), dim3(WG), 0, st, a, c->d_tok,
                            ceil_div(a.vocab, LMHEAD_ROWS_PER_WG));
+        mark(MLH_K_FINISH);
     } else {
         hipLaunchKernelGGL(k_advance, dim3(ceil_div(nseq, 64)), dim3(64), 0, st, a);
     }

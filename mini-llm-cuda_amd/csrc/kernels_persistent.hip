@@ -20,6 +20,8 @@
 // atomic load (served from the memory side), with workgroup-scope fences for ordering.  Weights are
 // read-only and use ordinary cached loads; each wave issues the loads of its next phase's weight
 // rows before it enters the barrier, so HBM latency overlaps the synchronisation.
+#include <stdlib.h>
+
 #include "mlh_internal.h"
 
 #define PWG 512
@@ -699,6 +701,11 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
     }
 }
 
+__global__ void k_zero_words(unsigned* p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
 // ----------------------------------------------------------------------------
 // host side
 // ----------------------------------------------------------------------------
@@ -710,7 +717,17 @@ static int launch_persistent(mlh_ctx* c, PersistArgs& P, size_t ldsBytes) {
     MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, fn, PWG, ldsBytes));
     if (perCu < 1) { c->err = "persistent decode kernel does not fit on a compute unit"; return -1; }
     void* args[] = {&P};
-    MLH_CHECK(c, hipLaunchCooperativeKernel(fn, dim3(c->numCUs), dim3(PWG), args, (unsigned)ldsBytes, c->stream));
+    // All workgroups must be resident at once: the grid is one workgroup per compute unit and the
+    // occupancy query above says each unit can hold one.  A plain launch then behaves like a
+    // cooperative one (and, unlike it, is visible to rocprofv3 and capturable in a graph); if some
+    // unit were busy with other work the bounded barrier wait gives up and the call reports it.
+    static const bool coop = getenv("MLH_PERSIST_COOPERATIVE") != nullptr;
+    if (coop) {
+        MLH_CHECK(c, hipLaunchCooperativeKernel(fn, dim3(c->numCUs), dim3(PWG), args, (unsigned)ldsBytes, c->stream));
+    } else {
+        hipLaunchKernelGGL((k_decode_persistent<WT, HD, GDK>), dim3(c->numCUs), dim3(PWG), ldsBytes, c->stream, P);
+        MLH_CHECK(c, hipGetLastError());
+    }
     return 0;
 }
 
@@ -722,7 +739,7 @@ bool mlh_persistent_supported(const mlh_ctx* c) {
     if (hp.headDim != 64 && hp.headDim != 128) return false;
     if (gdn && !(hp.gdnDk == hp.headDim && hp.gdnDv == hp.headDim)) return false;
     if (gdn && hp.gdnHeads > c->numCUs) return false;
-    return c->numCUs >= 8 && c->coopLaunch;
+    return c->numCUs >= 8;
 }
 
 // Enqueues `steps` decode steps of sequence 0 (slot 0) in one cooperative launch.
@@ -750,7 +767,7 @@ int mlh_launch_persistent(mlh_ctx* c, int steps) {
     const size_t tileFloats = hd == 64 ? (size_t)PAttn<64>::NW * PAttn<64>::TILE_FLOATS : (size_t)PAttn<128>::NW * PAttn<128>::TILE_FLOATS;
     const size_t ldsBytes = ((size_t)6 * hp.dim + stage + 4 * PWAVES + tileFloats) * 4;
     if (ldsBytes > 160 * 1024) { c->err = "model too wide for the persistent decode kernel"; return -1; }
-    MLH_CHECK(c, hipMemsetAsync(c->d_sync, 0, 64 * 24 * sizeof(unsigned), c->stream));
+    hipLaunchKernelGGL(k_zero_words, dim3(6), dim3(256), 0, c->stream, c->d_sync, 64 * 24); // barrier words and abort flag
     const bool bf = hp.weightDtype == MLH_DTYPE_BF16;
     if (hd == 64) {
         if (gdn) return bf ? launch_persistent<bf16_t, 64, 64>(c, P, ldsBytes) : launch_persistent<float, 64, 64>(c, P, ldsBytes);

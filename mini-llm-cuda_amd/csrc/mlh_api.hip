@@ -26,7 +26,7 @@ extern "C" int mlh_device_count(void) {
 extern "C" int mlh_kv_page_size(void) { return MLH_KV_PAGE; }
 
 static const char* const kKernelNames[MLH_K_COUNT] = {
-    "k_phaseA", "k_attn", "k_oproj", "k_ffn13", "k_down", "k_lmhead", "k_gdn", "k_copy"};
+    "k_phaseA", "k_attn", "k_oproj", "k_ffn13", "k_down", "k_lmhead", "k_gdn", "k_copy", "k_embed", "k_finish"};
 extern "C" const char* mlh_kernel_name(int kernel) {
     return (kernel >= 0 && kernel < MLH_K_COUNT) ? kKernelNames[kernel] : "";
 }
@@ -576,6 +576,55 @@ extern "C" int mlh_time_decode(mlh_ctx* c, const int32_t* first, int nseq, int s
     if (rc) return rc;
     if (use_persistent(c, nseq) && (rc = check_persistent_abort(c))) return rc;
     *totalMs = ms;
+    for (int s = 0; s < nseq; s++) c->h_len[s] += steps;
+    return 0;
+}
+
+extern "C" int mlh_profile_decode(mlh_ctx* c, const int32_t* first, int nseq, int steps, double* usPerLaunch,
+                                  int32_t* launchesPerStep) {
+    int rc = check_decode(c, first, nseq, steps);
+    if (rc) return rc;
+    if (!usPerLaunch || !launchesPerStep || steps > 64) { c->err = "bad argument (at most 64 steps)"; return -1; }
+    std::vector<hipEvent_t> events;
+    std::vector<int> ids;
+    hipEvent_t e0;
+    MLH_CHECK(c, hipEventCreate(&e0));
+    MLH_CHECK(c, hipMemcpyAsync(c->d_tok, first, (size_t)nseq * 4, hipMemcpyHostToDevice, c->stream));
+    MLH_CHECK(c, hipMemsetAsync(c->d_stepCounter, 0, 4, c->stream));
+    MLH_CHECK(c, hipStreamSynchronize(c->stream));
+    c->profEvents = &events;
+    c->profIds = &ids;
+    std::vector<size_t> stepStart;
+    for (int i = 0; i < steps && rc == 0; i++) {
+        stepStart.push_back(events.size());
+        if (i == 0) { // start marker; later steps measure from the previous step's last kernel
+            (void)hipEventRecord(e0, c->stream);
+            events.push_back(e0);
+            ids.push_back(-1);
+        }
+        rc = mlh_launch_step(c, nseq, c->d_tok, true);
+    }
+    c->profEvents = nullptr;
+    c->profIds = nullptr;
+    hipError_t e = hipStreamSynchronize(c->stream);
+    double sum[MLH_K_COUNT] = {0};
+    long cnt[MLH_K_COUNT] = {0};
+    if (rc == 0 && e == hipSuccess) {
+        for (size_t i = 1; i < events.size(); i++) {
+            float ms = 0.f;
+            if (ids[i] < 0 || hipEventElapsedTime(&ms, events[i - 1], events[i]) != hipSuccess || ms < 0.f) continue;
+            sum[ids[i]] += (double)ms * 1000.0;
+            cnt[ids[i]]++;
+        }
+    }
+    for (size_t i = 1; i < events.size(); i++) (void)hipEventDestroy(events[i]);
+    (void)hipEventDestroy(e0);
+    if (rc) return rc;
+    if (e != hipSuccess) { c->err = std::string("hipStreamSynchronize: ") + hipGetErrorString(e); return -2; }
+    for (int k = 0; k < MLH_K_COUNT; k++) {
+        usPerLaunch[k] = cnt[k] ? sum[k] / (double)cnt[k] : 0.0;
+        launchesPerStep[k] = (int32_t)(cnt[k] / steps);
+    }
     for (int s = 0; s < nseq; s++) c->h_len[s] += steps;
     return 0;
 }

@@ -114,7 +114,7 @@ struct mlh_ctx {
     // persistent batch-1 decode kernel
     int numCUs = 0;
     bool coopLaunch = false;
-    bool usePersistent = true;
+    bool usePersistent = false;
     LayerDev* d_layers = nullptr;  // device copy of `layers`
     unsigned* d_sync = nullptr;    // barrier words + abort flag
     float* pamaxVal = nullptr;     // [numCUs]
@@ -122,10 +122,13 @@ struct mlh_ctx {
     float* kvPart = nullptr;       // [heads, pagesPerSeq, headDim + 2]
     unsigned long long* d_timing = nullptr; // phase timestamps (set MLH_PERSIST_TIMING=1), 16 per layer
 
+    std::vector<hipEvent_t>* profEvents = nullptr; // set while mlh_profile_decode runs
+    std::vector<int>* profIds = nullptr;
+
     std::vector<int> h_len; // host mirror of d_pos
     int identityNseq = 0;   // d_sidx currently holds 0..identityNseq-1 (0 = unknown)
 
-    int graphSteps = 1;                 // 0: eager launches; k >= 1: one graph replay covers k decode steps
+    int graphSteps = 0;                 // 0: eager launches; k >= 1: one graph replay covers k decode steps
     hipGraphExec_t graphExec[2] = {};   // [0]: one step, [1]: graphSteps steps
     int graphNseqOf[2] = {0, 0};
     int graphStepsOf[2] = {0, 0};
