@@ -123,6 +123,19 @@ int mlh_set_page_table(mlh_ctx* ctx, const int32_t* table, int n);
  * all L columns per token, here positions already in the cache are not redone. */
 int mlh_prefill(mlh_ctx* ctx, int seq, const int32_t* ids, int n);
 
+/* The same for nseg distinct sequences in one pass: segment s appends lens[s]
+ * tokens (ids holds the segments back to back) to sequence seqs[s].  With 16
+ * or more tokens in the call, every projection is one MFMA GEMM over all
+ * tokens (cuBLAS SGEMM over the L columns in the reference, inference.cu:409-449,
+ * 575-596, 634-699), attention is tiled and causal over the pages
+ * (inference.cu:511-573), GDN layers run their recurrence over the segment. */
+int mlh_prefill_batch(mlh_ctx* ctx, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens);
+
+/* 0 (default): GEMM prefill when the call has 16 or more tokens and dim, ffnDim,
+ * pleDim and the mixing widths are multiples of 32 (fp32) / 64 (bf16);
+ * 1: always token by token through the decode kernels. */
+int mlh_set_prefill_mode(mlh_ctx* ctx, int mode);
+
 /* One greedy decode step for sequences 0..nseq-1: feeds last_ids[s] at each
  * sequence's current position, appends it, returns argmax of the logits
  * (lowest index on ties) in next_ids[s].  Replaces one iteration of the loop
@@ -190,6 +203,15 @@ int mlh_profile_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int ste
 /* Times `steps` decode steps (graph replays, argmax fed back on the device)
  * with HIP events on the context's stream: total milliseconds. */
 int mlh_time_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, double* total_ms);
+
+/* Stand-alone run of the MFMA GEMM used by prefill and batched decode (no context needed):
+ * C[M,N] = A[M,K] . B[N,K]^T (+ R[M,N]), host fp32 arrays in and out; with MLH_DTYPE_BF16 both
+ * operands are rounded to bf16 first.  K*4 (fp32) or K*2 (bf16) must be a multiple of 128.
+ * iters > 0 additionally times that many launches with HIP events (mean microseconds in avg_us).
+ * Replaces nothing in the reference by itself: it exposes the kernel that stands in for the
+ * cublasGemmEx calls of inference.cu:401-743 so that it can be checked and measured alone. */
+int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A, const float* B, const float* R, float* C,
+                      int iters, double* avg_us);
 
 #ifdef __cplusplus
 }

@@ -79,6 +79,8 @@ _sigs_dev = {
     "mlh_kv_page_size": (c_int, []),
     "mlh_set_page_table": (c_int, [c_void_p, c_void_p, c_int]),
     "mlh_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int]),
+    "mlh_prefill_batch": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p]),
+    "mlh_set_prefill_mode": (c_int, [c_void_p, c_int]),
     "mlh_decode_step": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "mlh_decode_loop": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "mlh_greedy_token": (c_int, [c_void_p, c_int, _P(c_int32)]),
@@ -90,6 +92,7 @@ _sigs_dev = {
     "mlh_time_kernel": (c_int, [c_void_p, c_int, c_int, c_int, c_int, _P(c_double), _P(c_double)]),
     "mlh_kernel_name": (c_char_p, [c_int]),
     "mlh_time_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double)]),
+    "mlh_selftest_gemm": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, _P(c_double)]),
     "mlh_profile_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double), _P(c_int32)]),
 }
 _sigs_host = {
@@ -267,6 +270,16 @@ class Device:
         a = np.ascontiguousarray(ids, dtype=np.int32)
         self._check(dev.mlh_prefill(self._h, seq, a.ctypes.data, a.size))
 
+    def prefill_batch(self, seqs, prompts):
+        """Appends prompts[i] to sequence seqs[i] for all i in one pass."""
+        sq = np.ascontiguousarray(seqs, dtype=np.int32)
+        lens = np.array([len(p) for p in prompts], dtype=np.int32)
+        ids = np.ascontiguousarray(np.concatenate([np.asarray(p, dtype=np.int32) for p in prompts]), dtype=np.int32)
+        self._check(dev.mlh_prefill_batch(self._h, sq.size, sq.ctypes.data, ids.ctypes.data, lens.ctypes.data))
+
+    def set_prefill_mode(self, mode):
+        self._check(dev.mlh_set_prefill_mode(self._h, int(mode)))
+
     def decode_step(self, last_ids):
         a = np.ascontiguousarray(last_ids, dtype=np.int32)
         out = np.empty_like(a)
@@ -382,6 +395,23 @@ class Vocab:
             self.close()
         except Exception:
             pass
+
+
+def selftest_gemm(a, b, r=None, bf16=False, iters=0):
+    """C = a . b^T (+ r) through the device GEMM kernel; returns (C, mean microseconds or None)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    m, k = a.shape
+    n = b.shape[0]
+    if r is not None:
+        r = np.ascontiguousarray(r, dtype=np.float32)
+    c = np.empty((m, n), dtype=np.float32)
+    us = c_double()
+    rc = dev.mlh_selftest_gemm(DTYPE_BF16 if bf16 else DTYPE_F32, m, n, k, a.ctypes.data, b.ctypes.data,
+                               r.ctypes.data if r is not None else None, c.ctypes.data, iters, byref(us))
+    if rc != 0:
+        raise MlhError(f"GEMM self-test failed ({rc}): unsupported shape or no device")
+    return c, (us.value if iters > 0 else None)
 
 
 def device_count():

@@ -1,0 +1,522 @@
+// Prefill: many tokens of one or more sequences through the stack at once.
+//
+// Rows of the activation matrices are tokens (all segments concatenated); the projections are MFMA
+// GEMMs (kernels_gemm.hip) against the same weight buffers the decode path streams; per layer
+//
+//   rmsnorm rows -> GEMM Wa -> attention: per-head QK-norm + RoPE + KV-page write, tiled causal attention
+//                              GDN:       chunked recurrence, one head of one sequence per workgroup
+//                -> (PLE rows) -> GEMM Wo (+ residual) (+ GEMM pleUp accumulate)
+//                -> rmsnorm rows -> GEMM W13 -> SiLU*up rows -> GEMM W2 (+ residual)
+//
+// and at the end the LM head runs for the last row of every segment only (the reference computes
+// logits for all L columns, inference.cu:723-743, and uses the last one).  With bf16 weights the GEMM
+// inputs (normed activations, mixing output, FFN activations) are rounded to bf16; accumulation, the
+// residual stream, K/V and GDN states stay fp32.  This is what runInference(L) (inference.cu:376-751)
+// does for L columns, minus the columns that are already in the cache.
+#include <algorithm>
+
+#include "mlh_internal.h"
+
+#define PWG 256
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+struct PfArgs {
+    StepArgs a;        // model dimensions and shared pointers (rope, page table, E, gains ...)
+    int n;             // rows (tokens) in this call
+    int nseg;
+    const int* ids;    // [n]
+    const int* rowSeq; // [n] sequence of the row
+    const int* rowPos; // [n] position of the row's token in its sequence
+    const int* segStart;
+    const int* segLen;
+    const int* segSeq;
+    const int* segPos0;
+    const int* blkSeg; // attention query blocks: segment and first query of the block
+    const int* blkQ0;
+    float* X;          // [n, dim] residual stream
+    void* Xn;          // [n, dim] GEMM input (weight dtype)
+    float* QKV;        // [n, qkvLd]
+    int qkvLd;
+    void* Amix;        // [n, aLd] mixing output (weight dtype)
+    int aLd;
+    void* Eple;        // [n, ple]
+    float* H1;         // [n, dim]
+    float* GU;         // [n, 2 ffn]
+    void* U;           // [n, ffn]
+};
+
+__device__ __forceinline__ float pf_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float pf_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float pf_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); } // inference.cu:248
+__device__ __forceinline__ float pf_silu(float v) { return v / (1.0f + expf(-v)); }       // inference.cu:270
+
+// store a float as the GEMM input type (fp32, or bf16 with round-to-nearest-even)
+template <typename AT> __device__ __forceinline__ void put(AT* p, float v);
+template <> __device__ __forceinline__ void put<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void put<bf16_t>(bf16_t* p, float v) {
+    uint32_t u = __float_as_uint(v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) u |= 0x00400000u;
+    else u += 0x7fffu + ((u >> 16) & 1u);
+    *p = (bf16_t)(u >> 16);
+}
+template <typename WT> __device__ __forceinline__ float getw(const WT* p);
+template <> __device__ __forceinline__ float getw<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float getw<bf16_t>(const bf16_t* p) { return __uint_as_float(((uint32_t)*p) << 16); }
+
+// inference.cu:9-22
+template <typename WT>
+__global__ void k_pf_embed(PfArgs P) {
+    const int row = blockIdx.y, i = blockIdx.x * PWG + threadIdx.x;
+    if (i >= P.a.dim) return;
+    P.X[(size_t)row * P.a.dim + i] = getw<WT>((const WT*)P.a.E + (size_t)P.ids[row] * P.a.dim + i);
+}
+
+// inference.cu:24-50 + 83-95, one wave per row
+template <typename AT>
+__global__ void __launch_bounds__(PWG) k_pf_rmsnorm(const float* __restrict__ X, const float* __restrict__ gamma, AT* out, int n, int d) {
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (row >= n) return;
+    const float* x = X + (size_t)row * d;
+    float s = 0.f;
+    for (int i = lane; i < d; i += 64) s = fmaf(x[i], x[i], s);
+    s = pf_wave_sum(s);
+    const float r = sqrtf(s / (float)d + 1e-8f);
+    for (int i = lane; i < d; i += 64) put<AT>(out + (size_t)row * d + i, gamma[i] * (x[i] / r));
+}
+
+// Per (head, row): per-head RMSNorm of q and k (inference.cu:52-81, 97-111), RoPE on adjacent pairs at the
+// row's position (inference.cu:113-134), q written back in place, k and v written to the KV pages.
+template <int HD>
+__global__ void __launch_bounds__(64) k_pf_qk_rope_kv(PfArgs P, LayerDev L) {
+    constexpr int EPL = HD / 64;
+    const StepArgs& a = P.a;
+    const int h = blockIdx.x, row = blockIdx.y, lane = threadIdx.x;
+    const int seq = P.rowSeq[row], pos = P.rowPos[row];
+    float* qkv = P.QKV + (size_t)row * P.qkvLd;
+    float qv[EPL], kv[EPL], vv[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+        const int i = lane * EPL + e;
+        qv[e] = qkv[h * HD + i]; kv[e] = qkv[L.offK + h * HD + i]; vv[e] = qkv[L.offV + h * HD + i];
+    }
+    if (a.qkNorm) {
+        float sq = 0.f, sk = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) { sq = fmaf(qv[e], qv[e], sq); sk = fmaf(kv[e], kv[e], sk); }
+        sq = pf_wave_sum(sq); sk = pf_wave_sum(sk);
+        const float rq = sqrtf(sq / (float)HD + 1e-8f), rk = sqrtf(sk / (float)HD + 1e-8f);
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            const int i = lane * EPL + e;
+            qv[e] = L.gq[h * HD + i] * (qv[e] / rq);
+            kv[e] = L.gk[h * HD + i] * (kv[e] / rk);
+        }
+    }
+    if (EPL == 1) {
+        const float c = a.rope[(size_t)pos * HD + (lane & ~1)], s = a.rope[(size_t)pos * HD + (lane | 1)];
+        const float qo = __shfl_xor(qv[0], 1, 64), ko = __shfl_xor(kv[0], 1, 64);
+        if (lane & 1) { qv[0] = s * qo + c * qv[0]; kv[0] = s * ko + c * kv[0]; }
+        else { qv[0] = c * qv[0] - s * qo; kv[0] = c * kv[0] - s * ko; }
+    } else {
+        const float c = a.rope[(size_t)pos * HD + 2 * lane], s = a.rope[(size_t)pos * HD + 2 * lane + 1];
+        const float q0 = qv[0], q1 = qv[EPL - 1], k0 = kv[0], k1 = kv[EPL - 1];
+        qv[0] = c * q0 - s * q1; qv[EPL - 1] = s * q0 + c * q1;
+        kv[0] = c * k0 - s * k1; kv[EPL - 1] = s * k0 + c * k1;
+    }
+    const int page = a.pageTable[seq * a.pagesPerSeq + (pos >> 6)];
+    const size_t o = ((size_t)page * MLH_KV_PAGE + (pos & 63)) * a.dim + h * HD;
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+        const int i = lane * EPL + e;
+        qkv[h * HD + i] = qv[e];
+        L.K[o + i] = kv[e];
+        L.V[o + i] = vv[e];
+    }
+}
+
+// Tiled causal attention for 16 queries of one head: K and V of 64 positions at a time in LDS, online
+// softmax per query (inference.cu:136-239, 511-573 for these columns), optional sigmoid gate (:241-250).
+#define PF_QB 16
+template <int HD, typename AT>
+__global__ void __launch_bounds__(PWG) k_pf_attn(PfArgs P, LayerDev L) {
+    constexpr int LDK = HD + 4, EPL = HD / 64, QPW = PF_QB / 4;
+    extern __shared__ float lds[];
+    float* Kt = lds;              // [64][LDK]
+    float* Vt = Kt + 64 * LDK;    // [64][LDK]
+    float* qs = Vt + 64 * LDK;    // [PF_QB][HD]
+    const StepArgs& a = P.a;
+    const int h = blockIdx.x, blk = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int seg = P.blkSeg[blk], q0 = P.blkQ0[blk];
+    const int seq = P.segSeq[seg], pos0 = P.segPos0[seg], len = P.segLen[seg], row0 = P.segStart[seg] + q0;
+    const int nq = min(PF_QB, len - q0);
+    const int maxPos = pos0 + q0 + nq - 1;
+    for (int i = tid; i < PF_QB * HD; i += PWG) {
+        const int q = i / HD, e = i - q * HD;
+        qs[i] = q < nq ? P.QKV[(size_t)(row0 + q) * P.qkvLd + h * HD + e] : 0.f;
+    }
+    float m[QPW], l[QPW], acc[QPW][EPL];
+#pragma unroll
+    for (int q = 0; q < QPW; q++) {
+        m[q] = -1.0e30f; l[q] = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) acc[q][e] = 0.f;
+    }
+    const float scale = sqrtf((float)HD);
+    const int ntiles = (maxPos >> 6) + 1;
+    for (int t = 0; t < ntiles; t++) {
+        const int j0 = t << 6;
+        const int page = a.pageTable[seq * a.pagesPerSeq + t];
+        const size_t base = ((size_t)page * MLH_KV_PAGE) * a.dim + h * HD;
+        __syncthreads();
+        for (int i = tid; i < 64 * (HD / 4); i += PWG) {
+            const int r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+            f32x4 kk = (f32x4)(0.f), vv = (f32x4)(0.f);
+            if (j0 + r <= maxPos) {
+                kk = *reinterpret_cast<const f32x4*>(L.K + base + (size_t)r * a.dim + c4);
+                vv = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)r * a.dim + c4);
+            }
+            *reinterpret_cast<f32x4*>(Kt + r * LDK + c4) = kk;
+            *reinterpret_cast<f32x4*>(Vt + r * LDK + c4) = vv;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int qq = 0; qq < QPW; qq++) {
+            const int q = wave * QPW + qq;
+            const int qpos = pos0 + q0 + q;
+            if (q >= nq || j0 > qpos) continue; // wave-uniform
+            float s = 0.f;
+            const float* kr = Kt + lane * LDK;
+            const float* qr = qs + q * HD;
+#pragma unroll
+            for (int i = 0; i < HD; i += 4) {
+                const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + i);
+                const f32x4 qv = *reinterpret_cast<const f32x4*>(qr + i);
+                s = fmaf(kk.x, qv.x, s); s = fmaf(kk.y, qv.y, s); s = fmaf(kk.z, qv.z, s); s = fmaf(kk.w, qv.w, s);
+            }
+            const bool valid = j0 + lane <= qpos;
+            s = valid ? s / scale : -1.0e30f;
+            const float mn = fmaxf(m[qq], pf_wave_max(s));
+            const float e = valid ? expf(s - mn) : 0.f;
+            const float corr = expf(m[qq] - mn);
+            l[qq] = l[qq] * corr + pf_wave_sum(e);
+            m[qq] = mn;
+#pragma unroll
+            for (int ee = 0; ee < EPL; ee++) acc[qq][ee] *= corr;
+#pragma unroll 16
+            for (int j = 0; j < 64; j++) {
+                const float pj = __shfl(e, j, 64);
+#pragma unroll
+                for (int ee = 0; ee < EPL; ee++) acc[qq][ee] = fmaf(pj, Vt[j * LDK + lane + 64 * ee], acc[qq][ee]);
+            }
+        }
+    }
+#pragma unroll
+    for (int qq = 0; qq < QPW; qq++) {
+        const int q = wave * QPW + qq;
+        if (q >= nq) continue;
+        const size_t row = (size_t)(row0 + q);
+#pragma unroll
+        for (int ee = 0; ee < EPL; ee++) {
+            const int dcol = h * HD + lane + 64 * ee;
+            float v = acc[qq][ee] / l[qq];
+            if (a.gating) v = v * pf_sigmoid(P.QKV[row * P.qkvLd + L.offG + dcol]);
+            put<AT>((AT*)P.Amix + row * P.aLd + dcol, v);
+        }
+    }
+}
+
+// Chunked gated-delta-net prefill: one head of one segment per workgroup, the state in registers over
+// the whole segment, inputs staged eight tokens at a time in LDS (same update as the decode kernel).
+#define PF_GC 8
+template <int DK, typename AT>
+__global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
+    constexpr int DV = DK, TPR = PWG / DV, CPT = DK / TPR;
+    __shared__ __attribute__((aligned(16))) float qs[PF_GC][DK];
+    __shared__ __attribute__((aligned(16))) float ks[PF_GC][DK];
+    __shared__ float vs[PF_GC][DV];
+    __shared__ float gate[PF_GC][4]; // alpha, beta, 1/|q|, 1/|k|
+    const StepArgs& a = P.a;
+    const int h = blockIdx.x, seg = blockIdx.y, tid = threadIdx.x;
+    const int seq = P.segSeq[seg], len = P.segLen[seg], row0 = P.segStart[seg];
+    const int r = tid / TPR, cg = tid % TPR, c0 = cg * CPT;
+    float* Srow = L.S + (((size_t)seq * a.gdnHeads + h) * DV + r) * DK + c0;
+    float S[CPT];
+#pragma unroll
+    for (int c = 0; c < CPT; c += 4) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(Srow + c);
+        S[c] = v.x; S[c + 1] = v.y; S[c + 2] = v.z; S[c + 3] = v.w;
+    }
+    for (int t0 = 0; t0 < len; t0 += PF_GC) {
+        const int nt = min(PF_GC, len - t0);
+        __syncthreads();
+        for (int i = tid; i < PF_GC * DK; i += PWG) {
+            const int c = i / DK, e = i - c * DK;
+            const float* qkv = P.QKV + (size_t)(row0 + t0 + min(c, nt - 1)) * P.qkvLd;
+            qs[c][e] = qkv[h * DK + e];
+            ks[c][e] = qkv[L.offK + h * DK + e];
+            vs[c][e] = qkv[L.offV + h * DV + e];
+        }
+        __syncthreads();
+        { // norms and gates of the chunk: 16 vectors, 16 threads each
+            const int vec = tid >> 4, sub = tid & 15, c = vec >> 1;
+            const float* src = (vec & 1) ? ks[c] : qs[c];
+            float s = 0.f;
+            for (int e = sub; e < DK; e += 16) s = fmaf(src[e], src[e], s);
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+            if (sub == 0) gate[c][2 + (vec & 1)] = sqrtf(s + 1e-6f);
+            if (tid < PF_GC) {
+                const float* qkv = P.QKV + (size_t)(row0 + t0 + min(tid, nt - 1)) * P.qkvLd;
+                const float za = qkv[L.offGa + h] + L.gdnBa[h], zb = qkv[L.offGb + h] + L.gdnBb[h];
+                gate[tid][0] = expf(-(fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
+                gate[tid][1] = pf_sigmoid(zb);
+            }
+        }
+        __syncthreads();
+        for (int c = 0; c < nt; c++) {
+            const float alpha = gate[c][0], beta = gate[c][1], rq = gate[c][2], rk = gate[c][3];
+            const float vr = vs[c][r];
+            float u = 0.f;
+#pragma unroll
+            for (int e = 0; e < CPT; e++) u = fmaf(S[e], ks[c][c0 + e] / rk, u);
+#pragma unroll
+            for (int o = TPR / 2; o > 0; o >>= 1) u += __shfl_xor(u, o, 64);
+            float oacc = 0.f;
+#pragma unroll
+            for (int e = 0; e < CPT; e++) {
+                const float kn = ks[c][c0 + e] / rk;
+                S[e] = alpha * (S[e] - beta * u * kn) + beta * vr * kn;
+                oacc = fmaf(S[e], qs[c][c0 + e] / rq, oacc);
+            }
+#pragma unroll
+            for (int o = TPR / 2; o > 0; o >>= 1) oacc += __shfl_xor(oacc, o, 64);
+            if (cg == 0) put<AT>((AT*)P.Amix + (size_t)(row0 + t0 + c) * P.aLd + h * DV + r, oacc);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CPT; c += 4) {
+        f32x4 v; v.x = S[c]; v.y = S[c + 1]; v.z = S[c + 2]; v.w = S[c + 3];
+        *reinterpret_cast<f32x4*>(Srow + c) = v;
+    }
+}
+
+// e[row][j] = silu(ple gate output) * P[tok][j]
+template <typename WT>
+__global__ void k_pf_ple(PfArgs P, LayerDev L) {
+    const int row = blockIdx.x, j = threadIdx.x;
+    if (j >= P.a.ple) return;
+    const float g = P.QKV[(size_t)row * P.qkvLd + L.offPle + j];
+    put<WT>((WT*)P.Eple + (size_t)row * P.a.ple + j, pf_silu(g) * getw<WT>((const WT*)L.pleTable + (size_t)P.ids[row] * P.a.ple + j));
+}
+
+// u[row][j] = silu(GU[row][2j]) * GU[row][2j+1]   (inference.cu:262-281)
+template <typename AT>
+__global__ void k_pf_silu_mul(PfArgs P) {
+    const size_t i = (size_t)blockIdx.x * PWG + threadIdx.x, total = (size_t)P.n * P.a.ffn;
+    if (i >= total) return;
+    const size_t row = i / P.a.ffn, j = i - row * P.a.ffn;
+    const float* gu = P.GU + row * 2 * P.a.ffn + 2 * j;
+    put<AT>((AT*)P.U + i, pf_silu(gu[0]) * gu[1]);
+}
+
+// residual of the last row of every segment -> decode slot buffer x[slot]
+__global__ void k_pf_gather_last(PfArgs P) {
+    const int seg = blockIdx.y, i = blockIdx.x * PWG + threadIdx.x;
+    if (i >= P.a.dim) return;
+    const int row = P.segStart[seg] + P.segLen[seg] - 1;
+    P.a.x[(size_t)seg * P.a.dim + i] = P.X[(size_t)row * P.a.dim + i];
+}
+
+// argmax over the LM-head partials of every segment's last row; sequence lengths advance by the segment length
+__global__ void __launch_bounds__(PWG) k_pf_finish(PfArgs P, int nparts, int* tokOut) {
+    __shared__ float sv[PWG];
+    __shared__ int si[PWG];
+    const StepArgs& a = P.a;
+    const int tid = threadIdx.x;
+    for (int seg = 0; seg < P.nseg; seg++) {
+        float v = -3.0e38f;
+        int idx = 0x7fffffff;
+        for (int i = tid; i < nparts; i += PWG) {
+            const float v2 = a.amaxVal[(size_t)seg * a.amaxParts + i];
+            const int i2 = a.amaxIdx[(size_t)seg * a.amaxParts + i];
+            if (v2 > v || (v2 == v && i2 < idx)) { v = v2; idx = i2; }
+        }
+        sv[tid] = v; si[tid] = idx;
+        __syncthreads();
+        for (int s = PWG / 2; s > 0; s >>= 1) {
+            if (tid < s && (sv[tid + s] > sv[tid] || (sv[tid + s] == sv[tid] && si[tid + s] < si[tid]))) { sv[tid] = sv[tid + s]; si[tid] = si[tid + s]; }
+            __syncthreads();
+        }
+        if (tid == 0) {
+            int nxt = si[0];
+            if (nxt < 0 || nxt >= a.vocab) nxt = 0;
+            const int seq = P.segSeq[seg];
+            tokOut[seg] = nxt;
+            a.nextTok[seq] = nxt;
+            a.pos[seq] += P.segLen[seg];
+        }
+        __syncthreads();
+    }
+}
+
+// ----------------------------------------------------------------------------
+// host side
+// ----------------------------------------------------------------------------
+static int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+bool mlh_prefill_gemm_supported(const mlh_ctx* c) {
+    const mlh_hparams& hp = c->hp;
+    const int esz = c->wbytes, kmul = 128 / esz;
+    if (hp.dim % kmul || hp.ffnDim % kmul || (hp.pleDim && hp.pleDim % kmul)) return false;
+    for (const LayerDev& L : c->layers)
+        if (L.ad % kmul) return false;
+    return true;
+}
+
+// The headDim-128 attention tiles exceed the 64 KB a launch may use without opting in.
+int mlh_init_prefill_kernels(mlh_ctx* c) {
+    const int lds = (2 * 64 * 132 + PF_QB * 128) * 4;
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_pf_attn<128, float>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_pf_attn<128, bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
+    return 0;
+}
+
+static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
+    if (rows <= c->pfRows) return 0;
+    const mlh_hparams& hp = c->hp;
+    (void)hipStreamSynchronize(c->stream);
+    for (void* p : c->pfAllocs) (void)hipFree(p);
+    c->pfAllocs.clear();
+    c->pfRows = 0;
+    const size_t n = (size_t)rows, wb = c->wbytes;
+    auto alloc = [&](void** p, size_t bytes) -> int {
+        MLH_CHECK(c, hipMalloc(p, std::max<size_t>(bytes, 16)));
+        c->pfAllocs.push_back(*p);
+        return 0;
+    };
+    int rc;
+    const int nblk = cdiv(rows, PF_QB) + hp.maxSeqs;
+    if ((rc = alloc((void**)&c->pfX, n * hp.dim * 4)) || (rc = alloc(&c->pfXn, n * hp.dim * wb)) ||
+        (rc = alloc((void**)&c->pfQKV, n * c->maxRowsA * 4)) || (rc = alloc(&c->pfA, n * c->maxAd * wb)) ||
+        (rc = alloc(&c->pfE, n * std::max(hp.pleDim, 8) * wb)) || (rc = alloc((void**)&c->pfH1, n * hp.dim * 4)) ||
+        (rc = alloc((void**)&c->pfGU, n * 2 * hp.ffnDim * 4)) || (rc = alloc(&c->pfU, n * hp.ffnDim * wb)) ||
+        (rc = alloc((void**)&c->pfMeta, (3 * n + 4 * (size_t)hp.maxSeqs + 2 * (size_t)nblk) * 4)))
+        return rc;
+    c->pfRows = rows;
+    c->pfBlkCap = nblk;
+    return 0;
+}
+
+#define PF_DISPATCH_WT(c, expr_f32, expr_bf16) do { if ((c)->hp.weightDtype == MLH_DTYPE_BF16) { expr_bf16; } else { expr_f32; } } while (0)
+
+// Appends lens[s] tokens to sequence seqs[s] for every segment s (token ids concatenated in `ids`).
+int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens) {
+    const mlh_hparams& hp = c->hp;
+    int n = 0;
+    for (int s = 0; s < nseg; s++) n += lens[s];
+    int rc = ensure_prefill_buffers(c, n);
+    if (rc) return rc;
+    // ---- metadata ----
+    std::vector<int> meta;
+    std::vector<int> rowSeq(n), rowPos(n), segStart(nseg), segPos0(nseg), blkSeg, blkQ0;
+    int r = 0;
+    for (int s = 0; s < nseg; s++) {
+        segStart[s] = r;
+        segPos0[s] = c->h_len[seqs[s]];
+        for (int i = 0; i < lens[s]; i++, r++) { rowSeq[r] = seqs[s]; rowPos[r] = segPos0[s] + i; }
+        for (int q0 = 0; q0 < lens[s]; q0 += PF_QB) { blkSeg.push_back(s); blkQ0.push_back(q0); }
+    }
+    const int nblk = (int)blkSeg.size();
+    if (nblk > c->pfBlkCap) { c->err = "prefill: too many attention blocks"; return -1; }
+    int* d = c->pfMeta;
+    int* d_ids = d; int* d_rowSeq = d + n; int* d_rowPos = d + 2 * n;
+    int* d_seg = d + 3 * n; // segStart, segLen, segSeq, segPos0 (maxSeqs each)
+    int* d_blk = d_seg + 4 * hp.maxSeqs;
+    hipStream_t st = c->stream;
+    MLH_CHECK(c, hipMemcpyAsync(d_ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_rowSeq, rowSeq.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_rowPos, rowPos.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_seg, segStart.data(), (size_t)nseg * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_seg + hp.maxSeqs, lens, (size_t)nseg * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_seg + 2 * hp.maxSeqs, seqs, (size_t)nseg * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_seg + 3 * hp.maxSeqs, segPos0.data(), (size_t)nseg * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_blk, blkSeg.data(), (size_t)nblk * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(d_blk + c->pfBlkCap, blkQ0.data(), (size_t)nblk * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipMemcpyAsync(c->d_sidx, seqs, (size_t)nseg * 4, hipMemcpyHostToDevice, st));
+    MLH_CHECK(c, hipStreamSynchronize(st)); // the host vectors above go out of scope
+    c->identityNseq = 0;
+
+    PfArgs P;
+    mlh_fill_args(c, P.a, nseg, c->d_tok);
+    P.n = n; P.nseg = nseg; P.ids = d_ids; P.rowSeq = d_rowSeq; P.rowPos = d_rowPos;
+    P.segStart = d_seg; P.segLen = d_seg + hp.maxSeqs; P.segSeq = d_seg + 2 * hp.maxSeqs; P.segPos0 = d_seg + 3 * hp.maxSeqs;
+    P.blkSeg = d_blk; P.blkQ0 = d_blk + c->pfBlkCap;
+    P.X = c->pfX; P.Xn = c->pfXn; P.QKV = c->pfQKV; P.qkvLd = c->maxRowsA; P.Amix = c->pfA; P.aLd = c->maxAd;
+    P.Eple = c->pfE; P.H1 = c->pfH1; P.GU = c->pfGU; P.U = c->pfU;
+    const int d_ = hp.dim, F = hp.ffnDim, dt = hp.weightDtype;
+#define GEMM(A, lda, B, ldb, C, ldc, R, ldr, M, N, K)                                                       \
+    do {                                                                                                    \
+        hipError_t e_ = mlh_gemm_tn(st, dt, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);                       \
+        if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; } \
+    } while (0)
+
+    PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_embed<float>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, P),
+                   hipLaunchKernelGGL((k_pf_embed<bf16_t>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, P));
+    for (int t = hp.transformers - 1; t >= 0; t--) { // file block 0 is the top (inference.cu:384-385)
+        const LayerDev& L = c->layers[t];
+        PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, L.g1, (float*)P.Xn, n, d_),
+                       hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, L.g1, (bf16_t*)P.Xn, n, d_));
+        GEMM(P.Xn, d_, L.Wa, d_, P.QKV, P.qkvLd, nullptr, 0, n, L.rowsA, d_);
+        if (L.kind == MLH_KIND_ATTENTION) {
+            if (hp.headDim == 64) {
+                hipLaunchKernelGGL((k_pf_qk_rope_kv<64>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
+                const size_t lds = (size_t)(2 * 64 * 68 + PF_QB * 64) * 4;
+                PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_attn<64, float>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L),
+                               hipLaunchKernelGGL((k_pf_attn<64, bf16_t>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L));
+            } else {
+                hipLaunchKernelGGL((k_pf_qk_rope_kv<128>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
+                const size_t lds = (size_t)(2 * 64 * 132 + PF_QB * 128) * 4;
+                PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_attn<128, float>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L),
+                               hipLaunchKernelGGL((k_pf_attn<128, bf16_t>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L));
+            }
+        } else if (hp.gdnDk == 64) {
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<64, float>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L),
+                           hipLaunchKernelGGL((k_pf_gdn<64, bf16_t>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L));
+        } else {
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<128, float>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L),
+                           hipLaunchKernelGGL((k_pf_gdn<128, bf16_t>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L));
+        }
+        GEMM(P.Amix, P.aLd, L.Wo, L.ad, P.H1, d_, P.X, d_, n, d_, L.ad);
+        if (hp.pleDim > 0) {
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_ple<float>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L),
+                           hipLaunchKernelGGL((k_pf_ple<bf16_t>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L));
+            GEMM(P.Eple, hp.pleDim, L.pleUp, hp.pleDim, P.H1, d_, P.H1, d_, n, d_, hp.pleDim);
+        }
+        PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (float*)P.Xn, n, d_),
+                       hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (bf16_t*)P.Xn, n, d_));
+        GEMM(P.Xn, d_, L.W13, d_, P.GU, 2 * F, nullptr, 0, n, 2 * F, d_);
+        {
+            const size_t total = (size_t)n * F;
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_silu_mul<float>), dim3((unsigned)((total + PWG - 1) / PWG)), dim3(PWG), 0, st, P),
+                           hipLaunchKernelGGL((k_pf_silu_mul<bf16_t>), dim3((unsigned)((total + PWG - 1) / PWG)), dim3(PWG), 0, st, P));
+        }
+        GEMM(P.U, F, L.W2, F, P.X, d_, P.H1, d_, n, d_, F);
+    }
+#undef GEMM
+    hipLaunchKernelGGL(k_pf_gather_last, dim3(cdiv(d_, PWG), nseg), dim3(PWG), 0, st, P);
+    if ((rc = mlh_launch_one(c, MLH_K_LMHEAD, 0, nseg))) return rc;
+    hipLaunchKernelGGL(k_pf_finish, dim3(1), dim3(PWG), 0, st, P, c->amaxParts, c->d_tok);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { c->err = std::string("prefill launch: ") + hipGetErrorString(e); return -2; }
+    MLH_CHECK(c, hipStreamSynchronize(st));
+    for (int s = 0; s < nseg; s++) c->h_len[seqs[s]] += lens[s];
+    return 0;
+}

@@ -78,6 +78,7 @@ extern "C" void mlh_destroy(mlh_ctx* c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (int i = 0; i < 2; i++) if (c->graphExec[i]) (void)hipGraphExecDestroy(c->graphExec[i]);
     for (void* p : c->allocs) (void)hipFree(p);
+    for (void* p : c->pfAllocs) (void)hipFree(p);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
 }
@@ -356,6 +357,7 @@ extern "C" int mlh_finalize(mlh_ctx* c) {
     }
     (void)hipSetDevice(c->device);
     int rc = mlh_init_kernels(c);
+    if (rc == 0) rc = mlh_init_prefill_kernels(c);
     if (rc) return rc;
     MLH_CHECK(c, hipMemcpy(c->d_layers, c->layers.data(), c->layers.size() * sizeof(LayerDev), hipMemcpyHostToDevice));
     MLH_CHECK(c, hipDeviceSynchronize());
@@ -433,21 +435,54 @@ static int set_identity_slots(mlh_ctx* c, int nseq) {
     return set_slots(c, id.data(), nseq);
 }
 
-extern "C" int mlh_prefill(mlh_ctx* c, int seq, const int32_t* ids, int n) {
-    int rc = check_ready(c);
-    if (rc) return rc;
-    const mlh_hparams& hp = c->hp;
-    if (seq < 0 || seq >= hp.maxSeqs) { c->err = "sequence index out of range"; return -1; }
-    if (!ids || n <= 0) { c->err = "empty prompt"; return -1; }
-    if (c->h_len[seq] + n > hp.maxL) { c->err = "prompt does not fit in maxL"; return -1; }
-    for (int i = 0; i < n; i++)
-        if (ids[i] < 0 || ids[i] >= hp.vocabSize) { c->err = "token id out of range"; return -1; }
+// Below this many rows the GEMM tiles are mostly padding and the decode kernels are faster.
+#define MLH_PREFILL_GEMM_MIN_ROWS 16
+
+static int prefill_token_by_token(mlh_ctx* c, int seq, const int32_t* ids, int n) {
+    int rc;
     if ((rc = set_slots(c, &seq, 1))) return rc;
     MLH_CHECK(c, hipMemcpyAsync(c->d_prompt, ids, (size_t)n * 4, hipMemcpyHostToDevice, c->stream));
     for (int i = 0; i < n; i++)
         if ((rc = mlh_launch_step(c, 1, c->d_prompt + i, i == n - 1))) return rc;
     MLH_CHECK(c, hipStreamSynchronize(c->stream));
     c->h_len[seq] += n;
+    return 0;
+}
+
+extern "C" int mlh_prefill_batch(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens) {
+    int rc = check_ready(c);
+    if (rc) return rc;
+    const mlh_hparams& hp = c->hp;
+    if (nseg <= 0 || nseg > hp.maxSeqs || !seqs || !ids || !lens) { c->err = "bad argument"; return -1; }
+    std::vector<char> seen(hp.maxSeqs, 0);
+    long total = 0;
+    for (int s = 0; s < nseg; s++) {
+        if (seqs[s] < 0 || seqs[s] >= hp.maxSeqs || seen[seqs[s]]) { c->err = "sequence indices must be distinct and in range"; return -1; }
+        seen[seqs[s]] = 1;
+        if (lens[s] <= 0) { c->err = "empty prompt"; return -1; }
+        if (c->h_len[seqs[s]] + lens[s] > hp.maxL) { c->err = "prompt does not fit in maxL"; return -1; }
+        total += lens[s];
+    }
+    for (long i = 0; i < total; i++)
+        if (ids[i] < 0 || ids[i] >= hp.vocabSize) { c->err = "token id out of range"; return -1; }
+    if (c->prefillMode == 0 && total >= MLH_PREFILL_GEMM_MIN_ROWS && mlh_prefill_gemm_supported(c))
+        return mlh_run_prefill_gemm(c, nseg, seqs, ids, lens);
+    long off = 0;
+    for (int s = 0; s < nseg; s++) {
+        if ((rc = prefill_token_by_token(c, seqs[s], ids + off, lens[s]))) return rc;
+        off += lens[s];
+    }
+    return 0;
+}
+
+extern "C" int mlh_prefill(mlh_ctx* c, int seq, const int32_t* ids, int n) {
+    return mlh_prefill_batch(c, 1, &seq, ids, &n);
+}
+
+extern "C" int mlh_set_prefill_mode(mlh_ctx* c, int mode) {
+    if (!c) return -1;
+    if (mode != 0 && mode != 1) { c->err = "prefill mode must be 0 (auto) or 1 (token by token)"; return -1; }
+    c->prefillMode = mode;
     return 0;
 }
 

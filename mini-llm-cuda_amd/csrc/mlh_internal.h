@@ -125,6 +125,14 @@ struct mlh_ctx {
     std::vector<hipEvent_t>* profEvents = nullptr; // set while mlh_profile_decode runs
     std::vector<int>* profIds = nullptr;
 
+    // prefill work buffers, sized on first use for the largest row count seen
+    int pfRows = 0, pfBlkCap = 0;
+    int prefillMode = 0; // 0: GEMM path when the shape allows and the call is long enough; 1: token by token
+    std::vector<void*> pfAllocs;
+    float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr, *pfGU = nullptr;
+    void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
+    int* pfMeta = nullptr;
+
     std::vector<int> h_len; // host mirror of d_pos
     int identityNseq = 0;   // d_sidx currently holds 0..identityNseq-1 (0 = unknown)
 
@@ -142,6 +150,15 @@ void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr);
 int mlh_launch_copy(mlh_ctx* c);
 int mlh_launch_probs(mlh_ctx* c, int seq);
 int mlh_init_kernels(mlh_ctx* c);
+
+// kernels_gemm.hip
+hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, const void* B, int ldb, float* C, int ldc,
+                       const float* R, int ldr, int M, int N, int K);
+
+// kernels_prefill.hip
+bool mlh_prefill_gemm_supported(const mlh_ctx* c);
+int mlh_init_prefill_kernels(mlh_ctx* c);
+int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens);
 
 // kernels_persistent.hip
 bool mlh_persistent_supported(const mlh_ctx* c);

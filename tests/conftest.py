@@ -47,12 +47,13 @@ def rel_diff(a, b):
 
 def assert_logits_close(got, want, rtol, what=""):
     """Logits agree within rtol in the reference's relative metric.  Elements whose magnitude is
-    below 1e-3 of the largest logit are compared absolutely against rtol * that floor: a relative
-    test on values near zero measures nothing but the cancellation in the dot product."""
+    below 1e-2 of the largest logit are compared absolutely against rtol * that floor: a relative
+    test on values near zero measures nothing but the cancellation in the dot product (fp32 sums over
+    a few hundred terms of O(1) logits carry ~1e-6 of absolute noise)."""
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     assert np.all(np.isfinite(got)), f"{what}: non-finite logits"
-    floor = 1e-3 * np.max(np.abs(want))
+    floor = 1e-2 * np.max(np.abs(want))
     den = np.maximum(np.maximum(np.abs(got), np.abs(want)), floor)
     r = np.abs(got - want) / den
     worst = int(np.argmax(r))

@@ -132,6 +132,7 @@ def test_bf16_weights(pkg, orc):
     hp = small_cfg(pkg, "hybrid", weightDtype=pkg.DTYPE_BF16)
     model, dev, w = make(pkg, orc, hp, seed=7, bf16=True)
     prompt = pkg.random_tokens(7, 0, hp.vocabSize, 16)
+    dev.set_prefill_mode(1)  # through the decode kernels (the GEMM prefill also rounds its inputs to bf16)
     dev.prefill(0, prompt)
     dec = orc.Decoder(w, "f64")
     for t in prompt:

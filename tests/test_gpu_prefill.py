@@ -1,0 +1,161 @@
+"""GPU parity of the GEMM prefill path (MFMA GEMMs + tiled causal attention + chunked GDN recurrence)
+against the CPU oracle and against the token-by-token path, through the C ABI.
+
+Tolerances as for decode: logits within 1e-3 relative (fp32 weights) and 2e-2 (bf16 weights, where the
+GEMM inputs are additionally rounded to bf16).
+"""
+import numpy as np
+import pytest
+
+from conftest import assert_logits_close, check_greedy_against_oracle, rel_diff
+from test_gpu_decode import small_cfg, make, FP32_RTOL, BF16_RTOL, GAP_TOL
+
+pytestmark = pytest.mark.gpu
+
+
+# ---- the GEMM by itself -------------------------------------------------------------------------
+@pytest.mark.parametrize("m,n,k", [(128, 128, 32), (1, 1, 32), (17, 300, 96), (130, 257, 704), (64, 1160, 256),
+                                   (300, 128, 2048), (257, 4096, 256)])
+def test_gemm_fp32(pkg, m, n, k):
+    """C = A.B^T (+R) on the fp32 MFMA path against float64 NumPy; ragged M and N, K a multiple of 32."""
+    rng = np.random.default_rng(m * 1000 + n + k)
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    b = rng.standard_normal((n, k), dtype=np.float32)
+    r = rng.standard_normal((m, n), dtype=np.float32)
+    for res in (None, r):
+        c, _ = pkg.selftest_gemm(a, b, res)
+        want = a.astype(np.float64) @ b.astype(np.float64).T + (0 if res is None else res)
+        err = np.max(np.abs(c - want))
+        # fp32 products summed in fp32: error grows like sqrt(k) * eps * |a||b|
+        assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
+
+
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 1, 64), (17, 300, 128), (130, 257, 704), (300, 128, 2048)])
+def test_gemm_bf16(pkg, orc, m, n, k):
+    """bf16 operands (already representable, so the product is exact in fp32) with fp32 accumulation."""
+    rng = np.random.default_rng(m * 1000 + n + k + 1)
+    a = orc.round_bf16(rng.standard_normal((m, k), dtype=np.float32))
+    b = orc.round_bf16(rng.standard_normal((n, k), dtype=np.float32))
+    r = rng.standard_normal((m, n), dtype=np.float32)
+    for res in (None, r):
+        c, _ = pkg.selftest_gemm(a, b, res, bf16=True)
+        want = a.astype(np.float64) @ b.astype(np.float64).T + (0 if res is None else res)
+        err = np.max(np.abs(c - want))
+        assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
+
+
+def test_gemm_rejects_bad_k(pkg):
+    a = np.zeros((4, 40), dtype=np.float32)
+    with pytest.raises(RuntimeError):
+        pkg.selftest_gemm(a, a)
+
+
+# ---- prefill ------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kind,plen", [("attn", 100), ("attn_flags", 77), ("hybrid", 130), ("hybrid_flags", 64),
+                                       ("hd128", 150), ("attn_long", 333)])
+def test_prefill_logits_vs_oracle_and_tokenwise(pkg, orc, kind, plen):
+    """Last-position logits of a GEMM prefill against the float64 oracle's full forward and against the
+    token-by-token path; then greedy decoding continues from the prefilled cache."""
+    hp = small_cfg(pkg, kind)
+    model, dev, w = make(pkg, orc, hp, seed=21)
+    prompt = pkg.random_tokens(21, 0, hp.vocabSize, plen)
+    want = orc.forward_full(w, prompt, "f64", last_only=True)["logits"][-1]
+    dev.prefill(0, prompt)
+    assert dev.seq_len(0) == plen
+    got = dev.logits(0)
+    assert_logits_close(got, want, FP32_RTOL, f"{kind} gemm prefill")
+    tok = dev.greedy_token(0)
+    ids = [tok]
+    for _ in range(11):
+        ids.append(int(dev.decode_step([ids[-1]])[0]))
+    dec = orc.Decoder(w, "f64")
+    exact, tol = check_greedy_against_oracle(dec, prompt, ids, GAP_TOL, what=kind)
+    assert exact + tol == len(ids)
+    # token-by-token through the decode kernels
+    dev.reset()
+    dev.set_prefill_mode(1)
+    dev.prefill(0, prompt)
+    assert_logits_close(dev.logits(0), want, FP32_RTOL, f"{kind} tokenwise prefill")
+    assert_logits_close(got, dev.logits(0), FP32_RTOL, f"{kind} gemm vs tokenwise")
+    dev.close()
+
+
+def test_prefill_in_pieces(pkg, orc):
+    """A prompt appended in three calls (GEMM, GEMM, short token-by-token tail) gives the logits of one call."""
+    hp = small_cfg(pkg, "hybrid_flags")
+    model, dev, w = make(pkg, orc, hp, seed=22)
+    prompt = pkg.random_tokens(22, 0, hp.vocabSize, 150)
+    want = orc.forward_full(w, prompt, "f64", last_only=True)["logits"][-1]
+    dev.prefill(0, prompt[:70])
+    dev.prefill(0, prompt[70:141])
+    dev.prefill(0, prompt[141:])
+    assert dev.seq_len(0) == 150
+    assert_logits_close(dev.logits(0), want, FP32_RTOL, "pieces")
+    dev.close()
+
+
+def test_prefill_batch_ragged(pkg, orc):
+    """Several sequences of different lengths in one pass: each equals its own single prefill and the
+    oracle; decoding the batch afterwards follows the oracle."""
+    hp = small_cfg(pkg, "hybrid", maxSeqs=4)
+    model, dev, w = make(pkg, orc, hp, seed=23)
+    lens = [17, 64, 1, 131]
+    prompts = [pkg.random_tokens(100 + i, 0, hp.vocabSize, n) for i, n in enumerate(lens)]
+    dev.prefill_batch([2, 0, 3, 1], prompts)
+    seqs = [2, 0, 3, 1]
+    firsts = {}
+    for s, p in zip(seqs, prompts):
+        assert dev.seq_len(s) == len(p)
+        want = orc.forward_full(w, p, "f64", last_only=True)["logits"][-1]
+        assert_logits_close(dev.logits(s), want, FP32_RTOL, f"batch seq {s}")
+        firsts[s] = dev.greedy_token(s)
+        best = int(np.argmax(want))
+        assert firsts[s] == best or want[best] - want[firsts[s]] <= GAP_TOL
+    out = dev.decode_loop([firsts[s] for s in range(4)], 6)
+    by_seq = {s: p for s, p in zip(seqs, prompts)}
+    for s in range(4):
+        ids = [firsts[s]] + [int(t) for t in out[:, s]]
+        dec = orc.Decoder(w, "f64")
+        exact, tol = check_greedy_against_oracle(dec, by_seq[s], ids, GAP_TOL, what=f"batch decode seq {s}")
+        assert exact + tol == len(ids)
+    dev.close()
+
+
+def test_prefill_paged(pkg, orc):
+    """A permuted page table changes nothing."""
+    hp = small_cfg(pkg, "attn_long", maxSeqs=2)
+    model, dev, w = make(pkg, orc, hp, seed=24)
+    prompt = pkg.random_tokens(24, 0, hp.vocabSize, 200)
+    dev.prefill(1, prompt)
+    ref = dev.logits(1)
+    dev.reset()
+    n = ((hp.maxL + 63) // 64) * hp.maxSeqs
+    perm = np.random.default_rng(3).permutation(n).astype(np.int32)
+    dev.set_page_table(perm)
+    dev.prefill(1, prompt)
+    assert np.array_equal(ref, dev.logits(1))
+    dev.close()
+
+
+@pytest.mark.parametrize("kind,plen", [("attn_flags", 90), ("hybrid", 100), ("hd128", 128)])
+def test_prefill_bf16(pkg, orc, kind, plen):
+    """bf16 weights: GEMM prefill (bf16 GEMM inputs) within 2e-2 of the float64 oracle on bf16-rounded
+    weights, and of the token-by-token path (fp32 activations)."""
+    hp = small_cfg(pkg, kind, weightDtype=pkg.DTYPE_BF16)
+    model, dev, w = make(pkg, orc, hp, seed=25, bf16=True)
+    prompt = pkg.random_tokens(25, 0, hp.vocabSize, plen)
+    want = orc.forward_full(w, prompt, "f64", last_only=True)["logits"][-1]
+    dev.prefill(0, prompt)
+    got = dev.logits(0)
+    floor = 1e-3 * np.max(np.abs(want))
+    den = np.maximum(np.maximum(np.abs(got), np.abs(want)), floor)
+    worst = float(np.max(np.abs(got - want) / den))
+    scale_err = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+    print(f"{kind}: bf16 prefill worst rel {worst:.3e}, max|diff|/max|logit| {scale_err:.3e}")
+    assert scale_err <= BF16_RTOL
+    dev.reset()
+    dev.set_prefill_mode(1)
+    dev.prefill(0, prompt)
+    scale_err2 = float(np.max(np.abs(dev.logits(0) - want)) / np.max(np.abs(want)))
+    assert scale_err2 <= BF16_RTOL
+    dev.close()
