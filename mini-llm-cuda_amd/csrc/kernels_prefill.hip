@@ -233,72 +233,288 @@ __global__ void __launch_bounds__(PWG) k_pf_attn(PfArgs P, LayerDev L) {
     }
 }
 
-// Chunked gated-delta-net prefill: one head of one segment per workgroup, the state in registers over
-// the whole segment, inputs staged eight tokens at a time in LDS (same update as the decode kernel).
-#define PF_GC 8
+// ----------------------------------------------------------------------------
+// bf16 MFMA causal attention (bf16-weight models).  A workgroup owns one head and 128 consecutive
+// queries of one segment, a wave 32 of them.  Per 64-key page:
+//   S^T[key, query] = K . Q^T      (A = K tile from LDS, B = Q^T held in registers)
+//   online softmax down the key axis -- with the transposed product every lane owns ONE query column
+//   (accumulator element i of lane l is row 8(i/4) + 4(l/32) + i%4, column l%32), so the running max,
+//   the running sum and the rescale of the output are in-lane, plus one exchange between lane halves
+//   O^T[hd, query] += V^T . P^T    (B = the lane's own P values, A = V transposed in LDS)
+// The contraction index of the second product may be permuted freely as long as A and B agree: slot
+// (half, e) of 16-key step t is the key the accumulator layout puts there, and the V tile is written
+// to LDS transposed in exactly that order, so P never leaves its registers.
+// K and V come from the fp32 pages and are rounded to bf16 on the way into LDS; scores, softmax
+// statistics and the output accumulate in fp32.
+// ----------------------------------------------------------------------------
+#define PF_MQB 128
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t bf16_bits(float v) {
+    uint32_t u = __float_as_uint(v);
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return bf16_bits(lo) | (bf16_bits(hi) << 16); }
+
+// position of key k (0..63) of a page along the permuted contraction axis of O^T += V^T . P^T
+__device__ __forceinline__ int pv_slot(int k) {
+    const int b = k >> 5, k32 = k & 31;
+    const int i = 4 * (k32 >> 3) + (k32 & 3), hh = (k32 >> 2) & 1;
+    return 16 * (2 * b + (i >> 3)) + 8 * hh + (i & 7);
+}
+
+template <int HD>
+__global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
+    constexpr int KP = HD + 8;   // K tile row pitch (bf16 elements): 16-byte reads, rows 4 banks apart
+    constexpr int VP = 64 + 8;   // V^T row pitch
+    constexpr int KS = HD / 16;  // 16-wide contraction steps of K . Q^T
+    constexpr int MB = HD / 32;  // 32-row blocks of O^T
+    __shared__ __attribute__((aligned(16))) uint16_t Kt[64 * KP];
+    __shared__ __attribute__((aligned(16))) uint16_t Vt[HD * VP];
+    const StepArgs& a = P.a;
+    const int h = blockIdx.x, blk = blockIdx.y, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int seg = P.blkSeg[blk], q0 = P.blkQ0[blk];
+    const int seq = P.segSeq[seg], pos0 = P.segPos0[seg], len = P.segLen[seg];
+    const int n32 = lane & 31, half = lane >> 5;
+    const int qi = q0 + wave * 32 + n32;              // this lane's query within the segment
+    const int qrow = P.segStart[seg] + min(qi, len - 1);
+    const int qpos = pos0 + qi;
+    const int waveMaxPos = pos0 + min(q0 + wave * 32 + 31, len - 1);
+    const int maxPos = pos0 + min(q0 + PF_MQB, len) - 1;
+    const bool waveActive = q0 + wave * 32 < len;
+
+    // Q^T operand: for step s the lane holds q[16 s + 8 half .. +7] of its query
+    u32x4 qop[KS];
+    {
+        const float* q = P.QKV + (size_t)qrow * P.qkvLd + h * HD + 8 * half;
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(q + 16 * s), hi = *reinterpret_cast<const f32x4*>(q + 16 * s + 4);
+            qop[s].x = pack_bf16(lo.x, lo.y); qop[s].y = pack_bf16(lo.z, lo.w);
+            qop[s].z = pack_bf16(hi.x, hi.y); qop[s].w = pack_bf16(hi.z, hi.w);
+        }
+    }
+    f32x16 oacc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; b++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oacc[b][i] = 0.f;
+    float m_run = -1.0e30f, l_run = 0.f;
+    const float inv_scale = 1.0f / sqrtf((float)HD);
+    const int ntiles = (maxPos >> 6) + 1;
+
+    for (int t = 0; t < ntiles; t++) {
+        const int j0 = t << 6;
+        const int page = a.pageTable[seq * a.pagesPerSeq + t];
+        const size_t base = ((size_t)page * MLH_KV_PAGE) * a.dim + h * HD;
+        __syncthreads(); // the previous tile has been consumed
+        // ---- K tile: natural layout ----
+        for (int i = tid; i < 64 * (HD / 4); i += PWG) {
+            const int r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+            f32x4 kk = (f32x4)(0.f);
+            if (j0 + r <= maxPos) kk = *reinterpret_cast<const f32x4*>(L.K + base + (size_t)r * a.dim + c4);
+            u32x2 w; w.x = pack_bf16(kk.x, kk.y); w.y = pack_bf16(kk.z, kk.w);
+            *reinterpret_cast<u32x2*>(Kt + r * KP + c4) = w;
+        }
+        // ---- V tile: transposed, keys in contraction-slot order; a lane carries two keys that are neighbours there ----
+        for (int i = tid; i < 32 * (HD / 4); i += PWG) {
+            const int kp = i & 7, g = (i >> 3) % (HD / 4), ko = (i >> 3) / (HD / 4); // key pair, column chunk, group of 8 pairs
+            const int k = 16 * ko + 2 * kp, c4 = 4 * g;
+            f32x4 v0 = (f32x4)(0.f), v1 = (f32x4)(0.f);
+            if (j0 + k <= maxPos) v0 = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)k * a.dim + c4);
+            if (j0 + k + 1 <= maxPos) v1 = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)(k + 1) * a.dim + c4);
+            const int slot = pv_slot(k); // even, and pv_slot(k + 1) == slot + 1
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 0) * VP + slot) = pack_bf16(v0.x, v1.x);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 1) * VP + slot) = pack_bf16(v0.y, v1.y);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 2) * VP + slot) = pack_bf16(v0.z, v1.z);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 3) * VP + slot) = pack_bf16(v0.w, v1.w);
+        }
+        __syncthreads();
+        if (!waveActive || j0 > waveMaxPos) continue; // wave-uniform; the barriers above are still reached by every wave
+        // ---- S^T = K . Q^T for the two 32-key blocks ----
+        f32x16 sacc[2];
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) sacc[b][i] = 0.f;
+#pragma unroll
+            for (int s = 0; s < KS; s++) {
+                const u32x4 kop = *reinterpret_cast<const u32x4*>(Kt + (32 * b + n32) * KP + 16 * s + 8 * half);
+                sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kop), __builtin_bit_cast(bf16x8, qop[s]), sacc[b], 0, 0, 0);
+            }
+        }
+        // ---- scale, causal mask, online softmax down the key axis ----
+        float mx = -1.0e30f;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int key = j0 + 32 * b + 8 * (i >> 2) + 4 * half + (i & 3);
+                const float sv = key <= qpos ? sacc[b][i] * inv_scale : -1.0e30f;
+                sacc[b][i] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float mn = fmaxf(m_run, mx);
+        const float corr = __expf(m_run - mn);
+        float ls = 0.f;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float pv = sacc[b][i] > -1.0e29f ? __expf(sacc[b][i] - mn) : 0.f;
+                sacc[b][i] = pv;
+                ls += pv;
+            }
+        ls += __shfl_xor(ls, 32, 64);
+        l_run = l_run * corr + ls;
+        m_run = mn;
+#pragma unroll
+        for (int b = 0; b < MB; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) oacc[b][i] *= corr;
+        // ---- O^T += V^T . P^T ----
+#pragma unroll
+        for (int st = 0; st < 4; st++) {
+            const int b = st >> 1, e0 = 8 * (st & 1);
+            u32x4 pop;
+            pop.x = pack_bf16(sacc[b][e0 + 0], sacc[b][e0 + 1]); pop.y = pack_bf16(sacc[b][e0 + 2], sacc[b][e0 + 3]);
+            pop.z = pack_bf16(sacc[b][e0 + 4], sacc[b][e0 + 5]); pop.w = pack_bf16(sacc[b][e0 + 6], sacc[b][e0 + 7]);
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+                const u32x4 vop = *reinterpret_cast<const u32x4*>(Vt + (32 * mb + n32) * VP + 16 * st + 8 * half);
+                oacc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vop), __builtin_bit_cast(bf16x8, pop), oacc[mb], 0, 0, 0);
+            }
+        }
+    }
+    if (qi >= len) return;
+    const float inv_l = 1.0f / l_run;
+    const size_t row = (size_t)qrow;
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int i4 = 0; i4 < 4; i4++) {
+            const int dcol = h * HD + 32 * mb + 8 * i4 + 4 * half;
+            f32x4 o;
+            o.x = oacc[mb][4 * i4] * inv_l; o.y = oacc[mb][4 * i4 + 1] * inv_l; o.z = oacc[mb][4 * i4 + 2] * inv_l; o.w = oacc[mb][4 * i4 + 3] * inv_l;
+            if (a.gating) {
+                const f32x4 gt = *reinterpret_cast<const f32x4*>(P.QKV + row * P.qkvLd + L.offG + dcol);
+                o.x *= pf_sigmoid(gt.x); o.y *= pf_sigmoid(gt.y); o.z *= pf_sigmoid(gt.z); o.w *= pf_sigmoid(gt.w);
+            }
+            u32x2 w; w.x = pack_bf16(o.x, o.y); w.y = pack_bf16(o.z, o.w);
+            *reinterpret_cast<u32x2*>((bf16_t*)P.Amix + row * P.aLd + dcol) = w;
+        }
+}
+
+// Gated-delta-net prefill.  The rows of a head's state evolve independently of each other
+//   S[r,:] <- alpha S[r,:] + beta (v_r - alpha u_r) k^T,  u_r = S[r,:].k,   o_r = S_new[r,:].q
+// (the decode kernel's update, regrouped; k, q L2-normalised), so one workgroup carries PF_GR rows of
+// one head of one segment in registers across the whole segment: 8 lanes per row, each with DK/8
+// columns.  Sixteen tokens of q, k, v and gate inputs are staged in LDS at a time, the next sixteen
+// being loaded into registers meanwhile.  With p = S_old[r,:].q the read-out needs no second pass:
+// o_r = (alpha p + w (k.q)) / |q|,  w = beta (v_r - alpha u_r) / |k|.
+#define PF_GC 16
+#define PF_GR 32
 template <int DK, typename AT>
 __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
-    constexpr int DV = DK, TPR = PWG / DV, CPT = DK / TPR;
+    constexpr int DV = DK, TPR = PWG / PF_GR, CPT = DK / TPR;
+    constexpr int NQK = PF_GC * DK / 4 / PWG; // f32x4 loads per thread for each of q and k
     __shared__ __attribute__((aligned(16))) float qs[PF_GC][DK];
     __shared__ __attribute__((aligned(16))) float ks[PF_GC][DK];
-    __shared__ float vs[PF_GC][DV];
-    __shared__ float gate[PF_GC][4]; // alpha, beta, 1/|q|, 1/|k|
+    __shared__ float vs[PF_GC][PF_GR];
+    __shared__ float zs[PF_GC][2];
+    __shared__ float gate[PF_GC][5]; // alpha, beta, 1/|q|, 1/|k|, k.q
     const StepArgs& a = P.a;
-    const int h = blockIdx.x, seg = blockIdx.y, tid = threadIdx.x;
+    const int h = blockIdx.x, seg = blockIdx.y, r0 = blockIdx.z * PF_GR, tid = threadIdx.x;
     const int seq = P.segSeq[seg], len = P.segLen[seg], row0 = P.segStart[seg];
     const int r = tid / TPR, cg = tid % TPR, c0 = cg * CPT;
-    float* Srow = L.S + (((size_t)seq * a.gdnHeads + h) * DV + r) * DK + c0;
+    float* Srow = L.S + (((size_t)seq * a.gdnHeads + h) * DV + r0 + r) * DK + c0;
     float S[CPT];
 #pragma unroll
     for (int c = 0; c < CPT; c += 4) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(Srow + c);
         S[c] = v.x; S[c + 1] = v.y; S[c + 2] = v.z; S[c + 3] = v.w;
     }
+    f32x4 qreg[NQK], kreg[NQK];
+    float vreg[2], zreg = 0.f;
+    auto fetch = [&](int t0) {
+        const int last = len - 1 - t0; // >= 0
+#pragma unroll
+        for (int it = 0; it < NQK; it++) {
+            const int i = it * PWG + tid, c = i / (DK / 4), e4 = (i % (DK / 4)) * 4;
+            const float* qkv = P.QKV + (size_t)(row0 + t0 + min(c, last)) * P.qkvLd;
+            qreg[it] = *reinterpret_cast<const f32x4*>(qkv + h * DK + e4);
+            kreg[it] = *reinterpret_cast<const f32x4*>(qkv + L.offK + h * DK + e4);
+        }
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int i = it * PWG + tid, c = i / PF_GR, e = i % PF_GR;
+            vreg[it] = P.QKV[(size_t)(row0 + t0 + min(c, last)) * P.qkvLd + L.offV + h * DV + r0 + e];
+        }
+        if (tid < 2 * PF_GC) {
+            const int c = tid >> 1;
+            zreg = P.QKV[(size_t)(row0 + t0 + min(c, last)) * P.qkvLd + ((tid & 1) ? L.offGb : L.offGa) + h];
+        }
+    };
+    fetch(0);
     for (int t0 = 0; t0 < len; t0 += PF_GC) {
         const int nt = min(PF_GC, len - t0);
-        __syncthreads();
-        for (int i = tid; i < PF_GC * DK; i += PWG) {
-            const int c = i / DK, e = i - c * DK;
-            const float* qkv = P.QKV + (size_t)(row0 + t0 + min(c, nt - 1)) * P.qkvLd;
-            qs[c][e] = qkv[h * DK + e];
-            ks[c][e] = qkv[L.offK + h * DK + e];
-            vs[c][e] = qkv[L.offV + h * DV + e];
-        }
-        __syncthreads();
-        { // norms and gates of the chunk: 16 vectors, 16 threads each
-            const int vec = tid >> 4, sub = tid & 15, c = vec >> 1;
-            const float* src = (vec & 1) ? ks[c] : qs[c];
-            float s = 0.f;
-            for (int e = sub; e < DK; e += 16) s = fmaf(src[e], src[e], s);
+        __syncthreads(); // the previous chunk has been consumed
 #pragma unroll
-            for (int o = 8; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-            if (sub == 0) gate[c][2 + (vec & 1)] = sqrtf(s + 1e-6f);
-            if (tid < PF_GC) {
-                const float* qkv = P.QKV + (size_t)(row0 + t0 + min(tid, nt - 1)) * P.qkvLd;
-                const float za = qkv[L.offGa + h] + L.gdnBa[h], zb = qkv[L.offGb + h] + L.gdnBb[h];
-                gate[tid][0] = expf(-(fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
-                gate[tid][1] = pf_sigmoid(zb);
+        for (int it = 0; it < NQK; it++) {
+            const int i = it * PWG + tid, c = i / (DK / 4), e4 = (i % (DK / 4)) * 4;
+            *reinterpret_cast<f32x4*>(&qs[c][e4]) = qreg[it];
+            *reinterpret_cast<f32x4*>(&ks[c][e4]) = kreg[it];
+        }
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int i = it * PWG + tid;
+            vs[i / PF_GR][i % PF_GR] = vreg[it];
+        }
+        if (tid < 2 * PF_GC) zs[tid >> 1][tid & 1] = zreg;
+        __syncthreads();
+        if (t0 + PF_GC < len) fetch(t0 + PF_GC); // in flight during this chunk's arithmetic
+        { // per token: |q|, |k|, k.q and the gates -- 16 threads per token
+            const int c = tid >> 4, sub = tid & 15;
+            float sq = 0.f, sk = 0.f, kq = 0.f;
+            for (int e = sub; e < DK; e += 16) {
+                const float qv = qs[c][e], kv = ks[c][e];
+                sq = fmaf(qv, qv, sq); sk = fmaf(kv, kv, sk); kq = fmaf(kv, qv, kq);
+            }
+#pragma unroll
+            for (int o = 8; o > 0; o >>= 1) { sq += __shfl_xor(sq, o, 64); sk += __shfl_xor(sk, o, 64); kq += __shfl_xor(kq, o, 64); }
+            if (sub == 0) {
+                const float za = zs[c][0] + L.gdnBa[h], zb = zs[c][1] + L.gdnBb[h];
+                const float rq = 1.0f / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+                gate[c][0] = expf(-(fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
+                gate[c][1] = pf_sigmoid(zb);
+                gate[c][2] = rq; gate[c][3] = rk; gate[c][4] = kq * rq * rk; // k.q of the normalised vectors
             }
         }
         __syncthreads();
         for (int c = 0; c < nt; c++) {
-            const float alpha = gate[c][0], beta = gate[c][1], rq = gate[c][2], rk = gate[c][3];
-            const float vr = vs[c][r];
-            float u = 0.f;
+            const float alpha = gate[c][0], beta = gate[c][1], rq = gate[c][2], rk = gate[c][3], kqn = gate[c][4];
+            float kk[CPT];
+            float u = 0.f, p = 0.f;
 #pragma unroll
-            for (int e = 0; e < CPT; e++) u = fmaf(S[e], ks[c][c0 + e] / rk, u);
-#pragma unroll
-            for (int o = TPR / 2; o > 0; o >>= 1) u += __shfl_xor(u, o, 64);
-            float oacc = 0.f;
-#pragma unroll
-            for (int e = 0; e < CPT; e++) {
-                const float kn = ks[c][c0 + e] / rk;
-                S[e] = alpha * (S[e] - beta * u * kn) + beta * vr * kn;
-                oacc = fmaf(S[e], qs[c][c0 + e] / rq, oacc);
+            for (int e = 0; e < CPT; e += 4) {
+                const f32x4 k4 = *reinterpret_cast<const f32x4*>(&ks[c][c0 + e]);
+                const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[c][c0 + e]);
+                kk[e] = k4.x; kk[e + 1] = k4.y; kk[e + 2] = k4.z; kk[e + 3] = k4.w;
+                u = fmaf(S[e], k4.x, u); u = fmaf(S[e + 1], k4.y, u); u = fmaf(S[e + 2], k4.z, u); u = fmaf(S[e + 3], k4.w, u);
+                p = fmaf(S[e], q4.x, p); p = fmaf(S[e + 1], q4.y, p); p = fmaf(S[e + 2], q4.z, p); p = fmaf(S[e + 3], q4.w, p);
             }
 #pragma unroll
-            for (int o = TPR / 2; o > 0; o >>= 1) oacc += __shfl_xor(oacc, o, 64);
-            if (cg == 0) put<AT>((AT*)P.Amix + (size_t)(row0 + t0 + c) * P.aLd + h * DV + r, oacc);
+            for (int o = TPR / 2; o > 0; o >>= 1) { u += __shfl_xor(u, o, 64); p += __shfl_xor(p, o, 64); }
+            u *= rk; p *= rq;                                  // against the normalised k and q
+            const float wn = beta * (vs[c][r] - alpha * u);    // coefficient of the normalised k
+            const float w = wn * rk;
+#pragma unroll
+            for (int e = 0; e < CPT; e++) S[e] = fmaf(w, kk[e], alpha * S[e]);
+            if (cg == 0) put<AT>((AT*)P.Amix + (size_t)(row0 + t0 + c) * P.aLd + h * DV + r0 + r, alpha * p + wn * kqn);
         }
     }
 #pragma unroll
@@ -385,7 +601,6 @@ bool mlh_prefill_gemm_supported(const mlh_ctx* c) {
 int mlh_init_prefill_kernels(mlh_ctx* c) {
     const int lds = (2 * 64 * 132 + PF_QB * 128) * 4;
     MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_pf_attn<128, float>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
-    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_pf_attn<128, bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     return 0;
 }
 
@@ -425,14 +640,15 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     int rc = ensure_prefill_buffers(c, n);
     if (rc) return rc;
     // ---- metadata ----
-    std::vector<int> meta;
+    const bool mfmaAttn = hp.weightDtype == MLH_DTYPE_BF16; // bf16 models: bf16 MFMA attention, 128 queries per workgroup
+    const int qb = mfmaAttn ? PF_MQB : PF_QB;
     std::vector<int> rowSeq(n), rowPos(n), segStart(nseg), segPos0(nseg), blkSeg, blkQ0;
     int r = 0;
     for (int s = 0; s < nseg; s++) {
         segStart[s] = r;
         segPos0[s] = c->h_len[seqs[s]];
         for (int i = 0; i < lens[s]; i++, r++) { rowSeq[r] = seqs[s]; rowPos[r] = segPos0[s] + i; }
-        for (int q0 = 0; q0 < lens[s]; q0 += PF_QB) { blkSeg.push_back(s); blkQ0.push_back(q0); }
+        for (int q0 = 0; q0 < lens[s]; q0 += qb) { blkSeg.push_back(s); blkQ0.push_back(q0); }
     }
     const int nblk = (int)blkSeg.size();
     if (nblk > c->pfBlkCap) { c->err = "prefill: too many attention blocks"; return -1; }
@@ -478,21 +694,19 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
         if (L.kind == MLH_KIND_ATTENTION) {
             if (hp.headDim == 64) {
                 hipLaunchKernelGGL((k_pf_qk_rope_kv<64>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
-                const size_t lds = (size_t)(2 * 64 * 68 + PF_QB * 64) * 4;
-                PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_attn<64, float>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L),
-                               hipLaunchKernelGGL((k_pf_attn<64, bf16_t>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L));
+                if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<64>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
+                else hipLaunchKernelGGL((k_pf_attn<64, float>), dim3(hp.attnHeads, nblk), dim3(PWG), (size_t)(2 * 64 * 68 + PF_QB * 64) * 4, st, P, L);
             } else {
                 hipLaunchKernelGGL((k_pf_qk_rope_kv<128>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
-                const size_t lds = (size_t)(2 * 64 * 132 + PF_QB * 128) * 4;
-                PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_attn<128, float>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L),
-                               hipLaunchKernelGGL((k_pf_attn<128, bf16_t>), dim3(hp.attnHeads, nblk), dim3(PWG), lds, st, P, L));
+                if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<128>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
+                else hipLaunchKernelGGL((k_pf_attn<128, float>), dim3(hp.attnHeads, nblk), dim3(PWG), (size_t)(2 * 64 * 132 + PF_QB * 128) * 4, st, P, L);
             }
         } else if (hp.gdnDk == 64) {
-            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<64, float>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_gdn<64, bf16_t>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L));
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<64, float>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L),
+                           hipLaunchKernelGGL((k_pf_gdn<64, bf16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
         } else {
-            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<128, float>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_gdn<128, bf16_t>), dim3(hp.gdnHeads, nseg), dim3(PWG), 0, st, P, L));
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<128, float>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L),
+                           hipLaunchKernelGGL((k_pf_gdn<128, bf16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
         }
         GEMM(P.Amix, P.aLd, L.Wo, L.ad, P.H1, d_, P.X, d_, n, d_, L.ad);
         if (hp.pleDim > 0) {

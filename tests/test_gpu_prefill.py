@@ -137,7 +137,7 @@ def test_prefill_paged(pkg, orc):
     dev.close()
 
 
-@pytest.mark.parametrize("kind,plen", [("attn_flags", 90), ("hybrid", 100), ("hd128", 128)])
+@pytest.mark.parametrize("kind,plen", [("attn_flags", 90), ("hybrid", 100), ("hd128", 199), ("attn_long", 333)])
 def test_prefill_bf16(pkg, orc, kind, plen):
     """bf16 weights: GEMM prefill (bf16 GEMM inputs) within 2e-2 of the float64 oracle on bf16-rounded
     weights, and of the token-by-token path (fp32 activations)."""
