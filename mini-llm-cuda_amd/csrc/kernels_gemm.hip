@@ -21,7 +21,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-#define GT 128            // tile rows (M) and columns (N)
 #define GKB 128           // bytes of K per row and slice
 #define GLD 144           // padded LDS row pitch in bytes
 #define GTHREADS 256
@@ -36,59 +35,81 @@ template <> struct GemmTraits<float> {
         c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
         c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ void put(float* p, float v) { *p = v; }
 };
 template <> struct GemmTraits<bf16_t> {
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x16& c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
+    static __device__ __forceinline__ void put(bf16_t* p, float v) {
+        uint32_t u = __float_as_uint(v);
+        *p = (bf16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+    }
 };
 
+// Workgroups that run at the same time on one XCD (ids congruent mod 8 go to the same XCD and share its
+// L2) get tiles that are neighbours: every XCD takes a contiguous eighth of the tile sequence, and
+// the sequence walks panels of four N tiles top to bottom, so ~32 resident workgroups cover about
+// 8 M tiles x 4 N tiles and re-read each other's A rows and B rows from L2.
+__device__ __forceinline__ void gemm_tile_of(int id, int tilesM, int tilesN, int& tm, int& tn) {
+    const int total = tilesM * tilesN;
+    const int per = (total + 7) / 8;
+    int t = (id & 7) * per + (id >> 3);
+    if (t >= total) { tm = -1; tn = -1; return; }
+    const int panel = t / (4 * tilesM);
+    const int pw = min(4, tilesN - 4 * panel);
+    const int r = t - panel * 4 * tilesM;
+    tm = r / pw;
+    tn = 4 * panel + r % pw;
+}
+
+#define GEMM_EPI_PLAIN 0  // C = acc (+ R), fp32
+#define GEMM_EPI_SWIGLU 1 // columns 2j, 2j+1 are gate and up of unit j: U[m, j] = silu(gate) * up, stored as T
+
 // lda/ldb in elements; K * sizeof(T) must be a multiple of 128.  R may be null, and may alias C.
-template <typename T>
+// BM x BN 32x32 blocks per wave, waves arranged 2 x 2: the workgroup tile is 64 BM x 64 BN.
+template <typename T, int BM, int BN, int EPI>
 __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
-                                                      float* C, int ldc, const float* R, int ldr, int M, int N, int K) {
-    __shared__ __attribute__((aligned(16))) unsigned char As[GT * GLD];
-    __shared__ __attribute__((aligned(16))) unsigned char Bs[GT * GLD];
+                                                      void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN) {
+    constexpr int TM = 64 * BM, TN = 64 * BN;
+    constexpr int PA = TM / 32, PB = TN / 32; // 16-byte pieces per thread and slice
+    extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
+    unsigned char* As = gsm;
+    unsigned char* Bs = gsm + TM * GLD;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+    int tm, tn;
+    gemm_tile_of(blockIdx.x, tilesM, tilesN, tm, tn);
+    if (tm < 0) return;
+    const int m0 = tm * TM, n0 = tn * TN;
     const int nslices = (int)(((size_t)K * sizeof(T)) / GKB);
     const unsigned char* Ab = reinterpret_cast<const unsigned char*>(A);
     const unsigned char* Bb = reinterpret_cast<const unsigned char*>(B);
     const size_t ldaB = (size_t)lda * sizeof(T), ldbB = (size_t)ldb * sizeof(T);
 
-    // global -> register staging: 128 rows x 8 pieces of 16 bytes per operand, 4 pieces per thread each
-    int rowA[4], rowB[4], piece[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int id = tid + GTHREADS * i;
-        const int r = id >> 3;
-        piece[i] = id & 7;
-        rowA[i] = min(m0 + r, M - 1); // rows past the edge repeat the last row; their results are never stored
-        rowB[i] = min(n0 + r, N - 1);
-    }
-    u32x4 ra[4], rb[4];
+    // global -> register staging; rows past the edge repeat the last row, their results are never stored
+    const int piece = tid & 7, srow = tid >> 3; // piece i of a thread is row srow + 32 i
+    u32x4 ra[PA], rb[PB];
     auto load_slice = [&](int s) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            ra[i] = *reinterpret_cast<const u32x4*>(Ab + (size_t)rowA[i] * ldaB + (size_t)s * GKB + piece[i] * 16);
-            rb[i] = *reinterpret_cast<const u32x4*>(Bb + (size_t)rowB[i] * ldbB + (size_t)s * GKB + piece[i] * 16);
-        }
+        for (int i = 0; i < PA; i++)
+            ra[i] = *reinterpret_cast<const u32x4*>(Ab + (size_t)min(m0 + srow + 32 * i, M - 1) * ldaB + (size_t)s * GKB + piece * 16);
+#pragma unroll
+        for (int i = 0; i < PB; i++)
+            rb[i] = *reinterpret_cast<const u32x4*>(Bb + (size_t)min(n0 + srow + 32 * i, N - 1) * ldbB + (size_t)s * GKB + piece * 16);
     };
     auto store_slice = [&]() {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int id = tid + GTHREADS * i;
-            *reinterpret_cast<u32x4*>(As + (id >> 3) * GLD + piece[i] * 16) = ra[i];
-            *reinterpret_cast<u32x4*>(Bs + (id >> 3) * GLD + piece[i] * 16) = rb[i];
-        }
+        for (int i = 0; i < PA; i++) *reinterpret_cast<u32x4*>(As + (srow + 32 * i) * GLD + piece * 16) = ra[i];
+#pragma unroll
+        for (int i = 0; i < PB; i++) *reinterpret_cast<u32x4*>(Bs + (srow + 32 * i) * GLD + piece * 16) = rb[i];
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[BM][BN];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < BM; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) acc[i][j] = (f32x16)(0.f);
+        for (int j = 0; j < BN; j++) acc[i][j] = (f32x16)(0.f);
 
     load_slice(0);
     store_slice();
@@ -98,16 +119,15 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
         if (s + 1 < nslices) load_slice(s + 1);
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
-            u32x4 fa[2], fb[2];
+            u32x4 fa[BM], fb[BN];
 #pragma unroll
-            for (int b = 0; b < 2; b++) {
-                fa[b] = *reinterpret_cast<const u32x4*>(As + (wm * 64 + b * 32 + lrow) * GLD + (2 * jj + half) * 16);
-                fb[b] = *reinterpret_cast<const u32x4*>(Bs + (wn * 64 + b * 32 + lrow) * GLD + (2 * jj + half) * 16);
-            }
+            for (int b = 0; b < BM; b++) fa[b] = *reinterpret_cast<const u32x4*>(As + (wm * 32 * BM + b * 32 + lrow) * GLD + (2 * jj + half) * 16);
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++)
+            for (int b = 0; b < BN; b++) fb[b] = *reinterpret_cast<const u32x4*>(Bs + (wn * 32 * BN + b * 32 + lrow) * GLD + (2 * jj + half) * 16);
 #pragma unroll
-                for (int bn = 0; bn < 2; bn++) GemmTraits<T>::mma(fa[bm], fb[bn], acc[bm][bn]);
+            for (int bm = 0; bm < BM; bm++)
+#pragma unroll
+                for (int bn = 0; bn < BN; bn++) GemmTraits<T>::mma(fa[bm], fb[bn], acc[bm][bn]);
         }
         __syncthreads();
         if (s + 1 < nslices) {
@@ -118,34 +138,205 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 
     // accumulator layout of the 32x32 tile: element i of lane l is row 8*(i/4) + 4*(l/32) + i%4, column l%32
 #pragma unroll
-    for (int bm = 0; bm < 2; bm++)
+    for (int bm = 0; bm < BM; bm++)
 #pragma unroll
-        for (int bn = 0; bn < 2; bn++) {
-            const int col = n0 + wn * 64 + bn * 32 + lrow;
+        for (int bn = 0; bn < BN; bn++) {
+            const int col = n0 + wn * 32 * BN + bn * 32 + lrow;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
-                const int row = m0 + wm * 64 + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
-                if (row < M && col < N) {
-                    float v = acc[bm][bn][i];
+                const int row = m0 + wm * 32 * BM + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
+                float v = acc[bm][bn][i];
+                if (EPI == GEMM_EPI_SWIGLU) {
+                    const float o = __shfl_xor(v, 1, 64); // the up value sits in the odd neighbour lane
+                    if (!(lane & 1) && row < M && col < N) GemmTraits<T>::put((T*)Cv + (size_t)row * ldc + (col >> 1), (v / (1.0f + expf(-v))) * o);
+                } else if (row < M && col < N) {
                     if (R) v += R[(size_t)row * ldr + col];
-                    C[(size_t)row * ldc + col] = v;
+                    ((float*)Cv)[(size_t)row * ldc + col] = v;
                 }
             }
         }
 }
 
+// ----------------------------------------------------------------------------
+// Large-tile variant for long M (prefill): 256 x 256 output tile per workgroup, each of the 2 x 2
+// waves owning 128 x 128 (sixteen 32x32 accumulators).  K slices of 128 bytes per row go from global
+// memory straight into LDS (no register staging), two stages deep: the loads of slice s+1 are in
+// flight while slice s is multiplied, and one barrier per slice separates the stages.
+//
+// A direct load puts lane i's 16 bytes at (wave-uniform base) + 16 i, so rows cannot be padded.  The
+// 8 pieces of a 128-byte row are stored permuted instead: slot j of row r holds piece j ^ ((r >> 1) & 7)
+// -- the lane picks which piece it fetches, not where it lands.  Sixteen consecutive rows reading the
+// same piece then touch sixteen different 16-byte bank groups.
+// ----------------------------------------------------------------------------
+#define GB_T 256
+#define GB_STAGE (2 * GB_T * GKB) // bytes per stage: A rows then B rows
+
+template <typename T, int EPI>
+__global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
+                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm, tn;
+    gemm_tile_of(blockIdx.x, tilesM, tilesN, tm, tn);
+    if (tm < 0) return;
+    const int m0 = tm * GB_T, n0 = tn * GB_T;
+    const int nslices = (int)(((size_t)K * sizeof(T)) / GKB);
+    const size_t ldaB = (size_t)lda * sizeof(T), ldbB = (size_t)ldb * sizeof(T);
+
+    // this wave fills rows [64 wave, 64 wave + 64) of A and of B, eight rows per load instruction
+    const unsigned char* srcA[8];
+    const unsigned char* srcB[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        const int r = wave * 64 + q * 8 + (lane >> 3);
+        const int pc = (lane & 7) ^ ((r >> 1) & 7);
+        srcA[q] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(m0 + r, M - 1) * ldaB + pc * 16;
+        srcB[q] = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + r, N - 1) * ldbB + pc * 16;
+    }
+    auto issue = [&](int s, int stage) {
+        unsigned char* dst = gsm + stage * GB_STAGE + wave * 64 * GKB;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            __builtin_amdgcn_global_load_lds(srcA[q] + (size_t)s * GKB, dst + q * 8 * GKB, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(srcB[q] + (size_t)s * GKB, dst + GB_T * GKB + q * 8 * GKB, 16, 0, 0);
+        }
+    };
+
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = (f32x16)(0.f);
+
+    const int half = lane >> 5, lrow = lane & 31;
+    // row offsets and swizzle keys of this lane's operand rows: rows wm*128 + 32 b + lrow; (row >> 1) & 7 does not depend on b
+    const int keyA = ((wm * 128 + lrow) >> 1) & 7, keyB = ((wn * 128 + lrow) >> 1) & 7;
+    const int offA = (wm * 128 + lrow) * GKB, offB = GB_T * GKB + (wn * 128 + lrow) * GKB;
+
+    issue(0, 0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int s = 0; s < nslices; s++) {
+        const int stage = s & 1;
+        if (s + 1 < nslices) issue(s + 1, stage ^ 1);
+        const unsigned char* base = gsm + stage * GB_STAGE;
+        // operand fragments one 16-wide step ahead of the MFMAs that use them
+        u32x4 fa[2][4], fb[2][4];
+        auto frags = [&](int jj, int buf) {
+            const int pa = ((2 * jj + half) ^ keyA) * 16, pb = ((2 * jj + half) ^ keyB) * 16;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                fa[buf][b] = *reinterpret_cast<const u32x4*>(base + offA + b * 32 * GKB + pa);
+                fb[buf][b] = *reinterpret_cast<const u32x4*>(base + offB + b * 32 * GKB + pb);
+            }
+        };
+        frags(0, 0);
+#pragma unroll
+        for (int jj = 0; jj < 4; jj++) {
+            // the reads of step jj+1 go out in the middle of step jj's MFMAs: early enough to have landed when
+            // they are needed, late enough that waiting for step jj's operands does not wait for them too.
+            // The scheduling barriers pin that order (the scheduler would sink every read to its first use).
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+                for (int bn = 0; bn < 4; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (jj < 3) frags(jj + 1, (jj + 1) & 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int bm = 2; bm < 4; bm++)
+#pragma unroll
+                for (int bn = 0; bn < 4; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // slice s+1 has landed
+        __syncthreads();                                  // ... for every wave, and everyone is done with slice s
+    }
+
+#pragma unroll
+    for (int bm = 0; bm < 4; bm++)
+#pragma unroll
+        for (int bn = 0; bn < 4; bn++) {
+            const int col = n0 + wn * 128 + bn * 32 + lrow;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int row = m0 + wm * 128 + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
+                float v = acc[bm][bn][i];
+                if (EPI == GEMM_EPI_SWIGLU) {
+                    const float o = __shfl_xor(v, 1, 64);
+                    if (!(lane & 1) && row < M && col < N) GemmTraits<T>::put((T*)Cv + (size_t)row * ldc + (col >> 1), (v / (1.0f + expf(-v))) * o);
+                } else if (row < M && col < N) {
+                    if (R) v += R[(size_t)row * ldr + col];
+                    ((float*)Cv)[(size_t)row * ldc + col] = v;
+                }
+            }
+        }
+}
+
+template <typename T>
+static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                                  const float* R, int ldr, int M, int N, int K) {
+    const int tilesM = (M + GB_T - 1) / GB_T, tilesN = (N + GB_T - 1) / GB_T;
+    const unsigned grid = (unsigned)(((tilesM * tilesN + 7) / 8) * 8);
+    const size_t lds = 2 * GB_STAGE;
+    static bool attr = false;
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_big<T, GEMM_EPI_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+    else
+        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+    return hipGetLastError();
+}
+
+template <typename T, int BM, int BN>
+static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                              const float* R, int ldr, int M, int N, int K) {
+    constexpr int TM = 64 * BM, TN = 64 * BN;
+    const int tilesM = (M + TM - 1) / TM, tilesN = (N + TN - 1) / TN;
+    const int total = tilesM * tilesN;
+    const unsigned grid = (unsigned)(((total + 7) / 8) * 8);
+    const size_t lds = (size_t)(TM + TN) * GLD;
+    static bool attr[2] = {false, false};
+    if (lds > 64 * 1024 && !attr[epi]) {
+        hipError_t e = hipFuncSetAttribute(epi ? reinterpret_cast<const void*>(&k_gemm_tn<T, BM, BN, GEMM_EPI_SWIGLU>)
+                                               : reinterpret_cast<const void*>(&k_gemm_tn<T, BM, BN, GEMM_EPI_PLAIN>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr[epi] = true;
+    }
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_tn<T, BM, BN, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+    else
+        hipLaunchKernelGGL((k_gemm_tn<T, BM, BN, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+    return hipGetLastError();
+}
+
 // Enqueues the GEMM on `stream`.  Returns hipSuccess, or an error when the shape is not supported.
-hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, const void* B, int ldb, float* C, int ldc,
-                       const float* R, int ldr, int M, int N, int K) {
+// epi = GEMM_EPI_PLAIN: C fp32 [M, N] (+ R).  epi = GEMM_EPI_SWIGLU: C is [M, N/2] in the operand type.
+hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                           const float* R, int ldr, int M, int N, int K) {
     const size_t esz = dtype == MLH_DTYPE_BF16 ? 2 : 4;
     if (M <= 0 || N <= 0 || K <= 0 || ((size_t)K * esz) % GKB != 0 || ((size_t)lda * esz) % 16 != 0 || ((size_t)ldb * esz) % 16 != 0)
         return hipErrorInvalidValue;
-    const dim3 grid((N + GT - 1) / GT, (M + GT - 1) / GT);
-    if (dtype == MLH_DTYPE_BF16)
-        hipLaunchKernelGGL((k_gemm_tn<bf16_t>), grid, dim3(GTHREADS), 0, stream, (const bf16_t*)A, lda, (const bf16_t*)B, ldb, C, ldc, R, ldr, M, N, K);
-    else
-        hipLaunchKernelGGL((k_gemm_tn<float>), grid, dim3(GTHREADS), 0, stream, (const float*)A, lda, (const float*)B, ldb, C, ldc, R, ldr, M, N, K);
-    return hipGetLastError();
+    if (epi == GEMM_EPI_SWIGLU && (N & 1)) return hipErrorInvalidValue;
+    // long M: 256 x 256 tiles fed by direct-to-LDS loads; short M (batched decode, short prompts): 128 x 128 tiles
+    if (M > 128)
+        return dtype == MLH_DTYPE_BF16 ? launch_gemm_big<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
+                                       : launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+    return dtype == MLH_DTYPE_BF16 ? launch_gemm<bf16_t, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
+                                   : launch_gemm<float, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+}
+
+hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, const void* B, int ldb, float* C, int ldc,
+                       const float* R, int ldr, int M, int N, int K) {
+    return mlh_gemm_tn_epi(stream, dtype, GEMM_EPI_PLAIN, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
 }
 
 static void host_to_bf16(const float* src, bf16_t* dst, size_t n) {

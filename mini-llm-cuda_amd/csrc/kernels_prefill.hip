@@ -6,7 +6,7 @@
 //   rmsnorm rows -> GEMM Wa -> attention: per-head QK-norm + RoPE + KV-page write, tiled causal attention
 //                              GDN:       chunked recurrence, one head of one sequence per workgroup
 //                -> (PLE rows) -> GEMM Wo (+ residual) (+ GEMM pleUp accumulate)
-//                -> rmsnorm rows -> GEMM W13 -> SiLU*up rows -> GEMM W2 (+ residual)
+//                -> rmsnorm rows -> GEMM W13 with SiLU(gate)*up epilogue -> GEMM W2 (+ residual)
 //
 // and at the end the LM head runs for the last row of every segment only (the reference computes
 // logits for all L columns, inference.cu:723-743, and uses the last one).  With bf16 weights the GEMM
@@ -41,7 +41,6 @@ struct PfArgs {
     int aLd;
     void* Eple;        // [n, ple]
     float* H1;         // [n, dim]
-    float* GU;         // [n, 2 ffn]
     void* U;           // [n, ffn]
 };
 
@@ -533,16 +532,6 @@ __global__ void k_pf_ple(PfArgs P, LayerDev L) {
     put<WT>((WT*)P.Eple + (size_t)row * P.a.ple + j, pf_silu(g) * getw<WT>((const WT*)L.pleTable + (size_t)P.ids[row] * P.a.ple + j));
 }
 
-// u[row][j] = silu(GU[row][2j]) * GU[row][2j+1]   (inference.cu:262-281)
-template <typename AT>
-__global__ void k_pf_silu_mul(PfArgs P) {
-    const size_t i = (size_t)blockIdx.x * PWG + threadIdx.x, total = (size_t)P.n * P.a.ffn;
-    if (i >= total) return;
-    const size_t row = i / P.a.ffn, j = i - row * P.a.ffn;
-    const float* gu = P.GU + row * 2 * P.a.ffn + 2 * j;
-    put<AT>((AT*)P.U + i, pf_silu(gu[0]) * gu[1]);
-}
-
 // residual of the last row of every segment -> decode slot buffer x[slot]
 __global__ void k_pf_gather_last(PfArgs P) {
     const int seg = blockIdx.y, i = blockIdx.x * PWG + threadIdx.x;
@@ -622,7 +611,7 @@ static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
     if ((rc = alloc((void**)&c->pfX, n * hp.dim * 4)) || (rc = alloc(&c->pfXn, n * hp.dim * wb)) ||
         (rc = alloc((void**)&c->pfQKV, n * c->maxRowsA * 4)) || (rc = alloc(&c->pfA, n * c->maxAd * wb)) ||
         (rc = alloc(&c->pfE, n * std::max(hp.pleDim, 8) * wb)) || (rc = alloc((void**)&c->pfH1, n * hp.dim * 4)) ||
-        (rc = alloc((void**)&c->pfGU, n * 2 * hp.ffnDim * 4)) || (rc = alloc(&c->pfU, n * hp.ffnDim * wb)) ||
+        (rc = alloc(&c->pfU, n * hp.ffnDim * wb)) ||
         (rc = alloc((void**)&c->pfMeta, (3 * n + 4 * (size_t)hp.maxSeqs + 2 * (size_t)nblk) * 4)))
         return rc;
     c->pfRows = rows;
@@ -676,7 +665,7 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     P.segStart = d_seg; P.segLen = d_seg + hp.maxSeqs; P.segSeq = d_seg + 2 * hp.maxSeqs; P.segPos0 = d_seg + 3 * hp.maxSeqs;
     P.blkSeg = d_blk; P.blkQ0 = d_blk + c->pfBlkCap;
     P.X = c->pfX; P.Xn = c->pfXn; P.QKV = c->pfQKV; P.qkvLd = c->maxRowsA; P.Amix = c->pfA; P.aLd = c->maxAd;
-    P.Eple = c->pfE; P.H1 = c->pfH1; P.GU = c->pfGU; P.U = c->pfU;
+    P.Eple = c->pfE; P.H1 = c->pfH1; P.U = c->pfU;
     const int d_ = hp.dim, F = hp.ffnDim, dt = hp.weightDtype;
 #define GEMM(A, lda, B, ldb, C, ldc, R, ldr, M, N, K)                                                       \
     do {                                                                                                    \
@@ -716,11 +705,9 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
         }
         PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (float*)P.Xn, n, d_),
                        hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (bf16_t*)P.Xn, n, d_));
-        GEMM(P.Xn, d_, L.W13, d_, P.GU, 2 * F, nullptr, 0, n, 2 * F, d_);
-        {
-            const size_t total = (size_t)n * F;
-            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_silu_mul<float>), dim3((unsigned)((total + PWG - 1) / PWG)), dim3(PWG), 0, st, P),
-                           hipLaunchKernelGGL((k_pf_silu_mul<bf16_t>), dim3((unsigned)((total + PWG - 1) / PWG)), dim3(PWG), 0, st, P));
+        { // gate/up projection with SiLU(gate) * up in the epilogue (inference.cu:262-281): U comes out in the GEMM input type
+            hipError_t e_ = mlh_gemm_tn_epi(st, dt, 1, P.Xn, d_, L.W13, d_, P.U, F, nullptr, 0, n, 2 * F, d_);
+            if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; }
         }
         GEMM(P.U, F, L.W2, F, P.X, d_, P.H1, d_, n, d_, F);
     }

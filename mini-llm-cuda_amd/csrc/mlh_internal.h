@@ -129,7 +129,7 @@ struct mlh_ctx {
     int pfRows = 0, pfBlkCap = 0;
     int prefillMode = 0; // 0: GEMM path when the shape allows and the call is long enough; 1: token by token
     std::vector<void*> pfAllocs;
-    float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr, *pfGU = nullptr;
+    float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
     void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
     int* pfMeta = nullptr;
 
@@ -154,6 +154,10 @@ int mlh_init_kernels(mlh_ctx* c);
 // kernels_gemm.hip
 hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, const void* B, int ldb, float* C, int ldc,
                        const float* R, int ldr, int M, int N, int K);
+// epi 0: as above.  epi 1 (SwiGLU): columns 2j / 2j+1 of the product are gate / up of unit j and
+// C is [M, N/2] in the operand type: C[m, j] = silu(gate) * up.
+hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                           const float* R, int ldr, int M, int N, int K);
 
 // kernels_prefill.hip
 bool mlh_prefill_gemm_supported(const mlh_ctx* c);
