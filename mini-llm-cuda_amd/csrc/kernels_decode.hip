@@ -927,6 +927,7 @@ static int launch_mix(mlh_ctx* c, const StepArgs& a, const LayerDev& L) {
 
 // Enqueues one decode step on the context's stream (no synchronisation).
 int mlh_launch_step(mlh_ctx* c, int nseq, const int* tokPtr, bool lmHead) {
+    if (lmHead && !c->profEvents && mlh_batch_step_applicable(c, nseq)) return mlh_launch_batch_step(c, nseq, tokPtr);
     StepArgs a;
     mlh_fill_args(c, a, nseq, tokPtr);
     hipStream_t st = c->stream;

@@ -318,6 +318,84 @@ static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int ld
     return hipGetLastError();
 }
 
+// ----------------------------------------------------------------------------
+// Skinny variant for M <= 64 (batched decode: one row per sequence).  The weight matrix is the big
+// operand and is read exactly once: a workgroup owns 32 weight rows, its four waves split K between
+// them in 128-byte chunks and multiply straight out of global memory -- the MFMA operand layout
+// (lane = row, 16 bytes of K) is also a reasonable load pattern: the four 16-byte loads of a lane
+// cover 64 contiguous bytes of its row.  The product is formed transposed, D[n, m] = B . A^T, so a
+// lane ends up with four consecutive n for one m: 16-byte stores into C[m, n..n+3].  The four partial
+// sums meet in LDS and are added in a fixed order.
+// ----------------------------------------------------------------------------
+template <typename T, int MB, int EPI>
+__global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
+                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K) {
+    __shared__ float red[4][MB][16][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n0 = blockIdx.x * 32, n32 = lane & 31, half = lane >> 5;
+    const int nchunks = (int)(((size_t)K * sizeof(T)) / GKB);
+    const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n32, N - 1) * ldb * sizeof(T) + half * 64;
+    const unsigned char* arow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+        arow[mb] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(mb * 32 + n32, M - 1) * lda * sizeof(T) + half * 64;
+    f32x16 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) acc[mb] = (f32x16)(0.f);
+    for (int c = wave; c < nchunks; c += 4) {
+        u32x4 fb[4], fa[MB][4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) fb[p] = *reinterpret_cast<const u32x4*>(brow + (size_t)c * GKB + p * 16);
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int p = 0; p < 4; p++) fa[mb][p] = *reinterpret_cast<const u32x4*>(arow[mb] + (size_t)c * GKB + p * 16);
+        // both operands put the same K elements in the same (half, position) slots, so every k meets itself
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) GemmTraits<T>::mma(fb[p], fa[mb][p], acc[mb]);
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) red[wave][mb][i][lane] = acc[mb][i];
+    __syncthreads();
+    // 2 MB x 4 groups of four accumulator elements; thread (wave, lane) takes groups 2 MB wave / 4 ...
+    for (int g = wave; g < MB * 4; g += 4) {
+        const int mb = g >> 2, i4 = g & 3;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = (red[0][mb][4 * i4 + j][lane] + red[1][mb][4 * i4 + j][lane]) + (red[2][mb][4 * i4 + j][lane] + red[3][mb][4 * i4 + j][lane]);
+        const int m = mb * 32 + n32, n = n0 + 8 * i4 + 4 * half; // accumulator element i: weight row 8 (i / 4) + 4 half + i % 4, column m
+        if (m >= M) continue;
+        if (EPI == GEMM_EPI_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2)
+                if (n + j + 1 < N) GemmTraits<T>::put((T*)Cv + (size_t)m * ldc + ((n + j) >> 1), (v[j] / (1.0f + expf(-v[j]))) * v[j + 1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (n + j < N) {
+                    float o = v[j];
+                    if (R) o += R[(size_t)m * ldr + n + j];
+                    ((float*)Cv)[(size_t)m * ldc + n + j] = o;
+                }
+        }
+    }
+}
+
+template <typename T, int MB>
+static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                                     const float* R, int ldr, int M, int N, int K) {
+    const dim3 grid((N + 31) / 32);
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K);
+    else
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K);
+    return hipGetLastError();
+}
+
 // Enqueues the GEMM on `stream`.  Returns hipSuccess, or an error when the shape is not supported.
 // epi = GEMM_EPI_PLAIN: C fp32 [M, N] (+ R).  epi = GEMM_EPI_SWIGLU: C is [M, N/2] in the operand type.
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
@@ -326,7 +404,14 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
     if (M <= 0 || N <= 0 || K <= 0 || ((size_t)K * esz) % GKB != 0 || ((size_t)lda * esz) % 16 != 0 || ((size_t)ldb * esz) % 16 != 0)
         return hipErrorInvalidValue;
     if (epi == GEMM_EPI_SWIGLU && (N & 1)) return hipErrorInvalidValue;
-    // long M: 256 x 256 tiles fed by direct-to-LDS loads; short M (batched decode, short prompts): 128 x 128 tiles
+    // M <= 64 (one row per sequence of a decode batch): weight-streaming skinny kernel; long M: 256 x 256 tiles
+    // fed by direct-to-LDS loads; in between: 128 x 128 tiles
+    if (M <= 32)
+        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
+                                       : launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+    if (M <= 64)
+        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
+                                       : launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
     if (M > 128)
         return dtype == MLH_DTYPE_BF16 ? launch_gemm_big<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
                                        : launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);

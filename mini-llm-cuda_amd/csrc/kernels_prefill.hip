@@ -600,6 +600,8 @@ static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
     for (void* p : c->pfAllocs) (void)hipFree(p);
     c->pfAllocs.clear();
     c->pfRows = 0;
+    for (int g = 0; g < 2; g++) // captured batched steps hold the old buffer addresses
+        if (c->graphExec[g]) { (void)hipGraphExecDestroy(c->graphExec[g]); c->graphExec[g] = nullptr; }
     const size_t n = (size_t)rows, wb = c->wbytes;
     auto alloc = [&](void** p, size_t bytes) -> int {
         MLH_CHECK(c, hipMalloc(p, std::max<size_t>(bytes, 16)));
@@ -719,5 +721,143 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     if (e != hipSuccess) { c->err = std::string("prefill launch: ") + hipGetErrorString(e); return -2; }
     MLH_CHECK(c, hipStreamSynchronize(st));
     for (int s = 0; s < nseg; s++) c->h_len[seqs[s]] += lens[s];
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Batched decode step (8 or more sequences, one new token each): the same row pipeline with the
+// skinny MFMA GEMM -- every weight matrix is streamed once per step whatever the batch size -- and
+// the decode path's own attention / GDN kernels, whose split-KV partials are combined here.
+// Everything stays on the device and on the stream (no allocation, no host round trip), so a
+// step can be captured into a graph like the GEMV step.
+// ----------------------------------------------------------------------------
+#define MLH_BATCH_GEMM_MIN_SEQS 8
+
+template <typename WT>
+__global__ void k_bd_embed(StepArgs a) {
+    const int slot = blockIdx.y, i = blockIdx.x * PWG + threadIdx.x;
+    if (slot == 0 && i == 0) *a.stepCounter += 1; // steps started; k_bd_finish logs into row (counter - 1)
+    if (i >= a.dim) return;
+    a.x[(size_t)slot * a.dim + i] = getw<WT>((const WT*)a.E + (size_t)a.tok[slot] * a.dim + i);
+}
+
+// Mixing output rows in the GEMM input type: attention layers combine the split-KV partials of the decode
+// attention kernel and apply the sigmoid gate (inference.cu:241-250); GDN layers convert the read-out.
+// PLE rows e = silu(gate) * P[tok] ride along.
+template <typename AT>
+__global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix, int aLd, AT* Eple) {
+    const int slot = blockIdx.x, tid = threadIdx.x;
+    const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
+    if (L.kind == MLH_KIND_ATTENTION) {
+        const int hd = a.hd;
+        for (int i = tid; i < L.ad; i += PWG) {
+            const int h = i / hd, e = i - h * hd;
+            const float* pp = a.part + (((size_t)slot * a.nsplit) * a.heads + h) * (hd + 2);
+            const size_t sstride = (size_t)a.heads * (hd + 2);
+            float M = -1.0e30f;
+            for (int s = 0; s < a.nsplit; s++) M = fmaxf(M, pp[s * sstride + hd]);
+            float num = 0.f, den = 0.f;
+            for (int s = 0; s < a.nsplit; s++) {
+                const float w = expf(pp[s * sstride + hd] - M);
+                num = fmaf(w, pp[s * sstride + e], num);
+                den = fmaf(w, pp[s * sstride + hd + 1], den);
+            }
+            float v = num / den;
+            if (a.gating) v = v * pf_sigmoid(qkv[L.offG + i]);
+            put<AT>(Amix + (size_t)slot * aLd + i, v);
+        }
+    } else {
+        for (int i = tid; i < L.ad; i += PWG) put<AT>(Amix + (size_t)slot * aLd + i, a.mix[(size_t)slot * L.ad + i]);
+    }
+    for (int j = tid; j < a.ple; j += PWG)
+        put<AT>(Eple + (size_t)slot * a.ple + j, pf_silu(qkv[L.offPle + j]) * getw<AT>((const AT*)L.pleTable + (size_t)a.tok[slot] * a.ple + j));
+}
+
+// One workgroup per slot: argmax of the slot's logits (lowest index on ties), logits copied to the
+// sequence's row, bookkeeping of k_finish (next token, id log, position).
+__global__ void __launch_bounds__(PWG) k_bd_finish(StepArgs a, const float* lg, int* tokOut) {
+    __shared__ float sv[PWG];
+    __shared__ int si[PWG];
+    const int slot = blockIdx.x, tid = threadIdx.x, seq = a.sidx[slot];
+    const float* row = lg + (size_t)slot * a.vocab;
+    float* dst = a.logits + (size_t)seq * a.vocab;
+    float v = -3.0e38f;
+    int idx = 0x7fffffff;
+    for (int i = tid; i < a.vocab; i += PWG) {
+        const float x = row[i];
+        dst[i] = x;
+        if (x > v) { v = x; idx = i; } // i ascends: ties keep the lower index
+    }
+    sv[tid] = v; si[tid] = idx;
+    __syncthreads();
+    for (int s = PWG / 2; s > 0; s >>= 1) {
+        if (tid < s && (sv[tid + s] > sv[tid] || (sv[tid + s] == sv[tid] && si[tid + s] < si[tid]))) { sv[tid] = sv[tid + s]; si[tid] = si[tid + s]; }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        int nxt = si[0];
+        if (nxt < 0 || nxt >= a.vocab) nxt = 0;
+        const int step = *a.stepCounter - 1;
+        tokOut[slot] = nxt;
+        a.nextTok[seq] = nxt;
+        if (step >= 0 && step < a.outCapacity) a.outIds[(size_t)step * a.nseq + slot] = nxt;
+        a.pos[seq] += 1;
+    }
+}
+
+bool mlh_batch_step_applicable(const mlh_ctx* c, int nseq) {
+    return c->prefillMode == 0 && nseq >= MLH_BATCH_GEMM_MIN_SEQS && nseq <= 64 && mlh_prefill_gemm_supported(c);
+}
+
+// Allocations the batched step needs; call outside graph capture.
+int mlh_prepare_batch_step(mlh_ctx* c, int nseq) {
+    if (!mlh_batch_step_applicable(c, nseq)) return 0;
+    int rc = ensure_prefill_buffers(c, std::max(nseq, 64));
+    if (rc) return rc;
+    if (!c->pfLogits) {
+        MLH_CHECK(c, hipMalloc((void**)&c->pfLogits, (size_t)64 * c->hp.vocabSize * 4));
+        c->allocs.push_back(c->pfLogits);
+    }
+    return 0;
+}
+
+int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
+    const mlh_hparams& hp = c->hp;
+    if (c->pfRows < nseq || !c->pfLogits) { c->err = "batched step buffers not prepared"; return -1; }
+    StepArgs a;
+    mlh_fill_args(c, a, nseq, tokPtr);
+    hipStream_t st = c->stream;
+    const int d_ = hp.dim, F = hp.ffnDim, dt = hp.weightDtype, n = nseq;
+    const bool bf = dt == MLH_DTYPE_BF16;
+#define GEMM(epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)                                                       \
+    do {                                                                                                         \
+        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);                   \
+        if (e_ != hipSuccess) { c->err = std::string("batched step GEMM: ") + hipGetErrorString(e_); return -2; } \
+    } while (0)
+    if (bf) hipLaunchKernelGGL((k_bd_embed<bf16_t>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);
+    else hipLaunchKernelGGL((k_bd_embed<float>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);
+    for (int t = hp.transformers - 1; t >= 0; t--) {
+        const LayerDev& L = c->layers[t];
+        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (bf16_t*)c->pfXn, n, d_);
+        else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (float*)c->pfXn, n, d_);
+        GEMM(0, c->pfXn, d_, L.Wa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
+        int rc = mlh_launch_one(c, L.kind == MLH_KIND_ATTENTION ? MLH_K_ATTN : MLH_K_GDN, t, nseq);
+        if (rc) return rc;
+        if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t>), dim3(n), dim3(PWG), 0, st, a, L, (bf16_t*)c->pfA, c->maxAd, (bf16_t*)c->pfE);
+        else hipLaunchKernelGGL((k_bd_mix<float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd, (float*)c->pfE);
+        GEMM(0, c->pfA, c->maxAd, L.Wo, L.ad, c->h1, d_, c->x, d_, n, d_, L.ad);
+        if (hp.pleDim > 0) GEMM(0, c->pfE, hp.pleDim, L.pleUp, hp.pleDim, c->h1, d_, c->h1, d_, n, d_, hp.pleDim);
+        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (bf16_t*)c->pfXn, n, d_);
+        else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (float*)c->pfXn, n, d_);
+        GEMM(1, c->pfXn, d_, L.W13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_);
+        GEMM(0, c->pfU, F, L.W2, F, c->x, d_, c->h1, d_, n, d_, F);
+    }
+    if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (bf16_t*)c->pfXn, n, d_);
+    else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (float*)c->pfXn, n, d_);
+    GEMM(0, c->pfXn, d_, c->E, d_, c->pfLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_);
+#undef GEMM
+    hipLaunchKernelGGL(k_bd_finish, dim3(n), dim3(PWG), 0, st, a, c->pfLogits, c->d_tok);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { c->err = std::string("batched step launch: ") + hipGetErrorString(e); return -2; }
     return 0;
 }

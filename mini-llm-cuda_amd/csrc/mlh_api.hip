@@ -482,6 +482,9 @@ extern "C" int mlh_prefill(mlh_ctx* c, int seq, const int32_t* ids, int n) {
 extern "C" int mlh_set_prefill_mode(mlh_ctx* c, int mode) {
     if (!c) return -1;
     if (mode != 0 && mode != 1) { c->err = "prefill mode must be 0 (auto) or 1 (token by token)"; return -1; }
+    if (mode != c->prefillMode)
+        for (int g = 0; g < 2; g++) // a captured step follows the mode it was captured under
+            if (c->graphExec[g]) { (void)hipGraphExecDestroy(c->graphExec[g]); c->graphExec[g] = nullptr; }
     c->prefillMode = mode;
     return 0;
 }
@@ -569,6 +572,7 @@ static int check_decode(mlh_ctx* c, const int32_t* ids, int nseq, int steps) {
         if (ids[s] < 0 || ids[s] >= hp.vocabSize) { c->err = "token id out of range"; return -1; }
         if (c->h_len[s] + steps > hp.maxL) { c->err = "sequence would exceed maxL"; return -1; }
     }
+    if ((rc = mlh_prepare_batch_step(c, nseq))) return rc;
     return set_identity_slots(c, nseq);
 }
 

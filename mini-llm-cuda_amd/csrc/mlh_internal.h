@@ -132,6 +132,7 @@ struct mlh_ctx {
     float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
     void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
     int* pfMeta = nullptr;
+    float* pfLogits = nullptr; // [64, vocab] logits of a batched decode step in slot order
 
     std::vector<int> h_len; // host mirror of d_pos
     int identityNseq = 0;   // d_sidx currently holds 0..identityNseq-1 (0 = unknown)
@@ -162,6 +163,9 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
 // kernels_prefill.hip
 bool mlh_prefill_gemm_supported(const mlh_ctx* c);
 int mlh_init_prefill_kernels(mlh_ctx* c);
+bool mlh_batch_step_applicable(const mlh_ctx* c, int nseq);
+int mlh_prepare_batch_step(mlh_ctx* c, int nseq);
+int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr);
 int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens);
 
 // kernels_persistent.hip

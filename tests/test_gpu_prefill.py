@@ -159,3 +159,56 @@ def test_prefill_bf16(pkg, orc, kind, plen):
     scale_err2 = float(np.max(np.abs(dev.logits(0) - want)) / np.max(np.abs(want)))
     assert scale_err2 <= BF16_RTOL
     dev.close()
+
+
+# ---- batched decode through the skinny GEMM ------------------------------------------------------
+@pytest.mark.parametrize("kind,nseq,graph", [("hybrid", 8, 0), ("hybrid_flags", 13, 1), ("attn_long", 33, 0), ("hd128", 64, 2)])
+def test_batched_decode_gemm_path(pkg, orc, kind, nseq, graph):
+    """Eight or more sequences per step take the MFMA path (skinny GEMMs + decode attention/GDN kernels):
+    ids and final logits against the float64 oracle, per sequence, with ragged prompt lengths; the same
+    run through the GEMV kernels (mode 1) must agree within the fp32 tolerance."""
+    hp = small_cfg(pkg, kind, maxSeqs=nseq)
+    model, dev, w = make(pkg, orc, hp, seed=31)
+    dev.set_graph(graph)
+    rng = np.random.default_rng(nseq)
+    lens = rng.integers(1, 90, size=nseq)
+    prompts = [pkg.random_tokens(31, s, hp.vocabSize, int(n)) for s, n in enumerate(lens)]
+    steps = 10
+    res = {}
+    for mode in (0, 1):
+        dev.reset()
+        dev.set_prefill_mode(mode)
+        dev.prefill_batch(list(range(nseq)), prompts)
+        firsts = [dev.greedy_token(s) for s in range(nseq)]
+        out = dev.decode_loop(firsts, steps)
+        res[mode] = (firsts, out.copy(), [dev.logits(s) for s in range(nseq)])
+    firsts, out, logits = res[0]
+    for s in range(0, nseq, max(1, nseq // 8)):  # a spread of sequences keeps the oracle time bounded
+        dec = orc.Decoder(w, "f64")
+        ids = [firsts[s]] + [int(t) for t in out[:, s]]
+        exact, tol = check_greedy_against_oracle(dec, prompts[s], ids, GAP_TOL, what=f"{kind} seq {s}")
+        assert exact + tol == len(ids)
+        dec.reset()
+        for t in list(prompts[s]) + ids[:-1]:
+            _, lg = dec.step(int(t))
+        assert_logits_close(logits[s], lg, FP32_RTOL, f"{kind} seq {s} final logits")
+        assert_logits_close(logits[s], res[1][2][s], FP32_RTOL, f"{kind} seq {s} gemm vs gemv")
+    dev.close()
+
+
+def test_batched_decode_gemm_path_bf16(pkg, orc):
+    """bf16 weights, 8 sequences: the MFMA step within 2e-2 (of the largest logit) of the oracle on bf16-rounded weights."""
+    hp = small_cfg(pkg, "hybrid", weightDtype=pkg.DTYPE_BF16, maxSeqs=8)
+    model, dev, w = make(pkg, orc, hp, seed=32, bf16=True)
+    prompts = [pkg.random_tokens(32, s, hp.vocabSize, 20 + 7 * s) for s in range(8)]
+    dev.prefill_batch(list(range(8)), prompts)
+    firsts = [dev.greedy_token(s) for s in range(8)]
+    out = dev.decode_loop(firsts, 6)
+    for s in (0, 3, 7):
+        dec = orc.Decoder(w, "f64")
+        ids = [firsts[s]] + [int(t) for t in out[:, s]]
+        for t in list(prompts[s]) + ids[:-1]:
+            _, lg = dec.step(int(t))
+        err = float(np.max(np.abs(dev.logits(s) - lg)) / np.max(np.abs(lg)))
+        assert err <= BF16_RTOL, (s, err)
+    dev.close()
