@@ -29,6 +29,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+MFMA_BF16_PEAK = 2.5e15  # MI355X dense bf16 MFMA, published peak (flop/s)
 PROMPT_LEN = 64
 
 
@@ -90,6 +91,93 @@ def cpu_baseline(model, hp, prompt, seconds_budget=20.0):
     }
 
 
+def matrix_params(hp):
+    """Weight-matrix elements one token multiplies on its way through the stack (LM head excluded)."""
+    d, F, total = hp.dim, hp.ffnDim, 0
+    for t in range(hp.transformers):
+        if hp.layerKinds[t] == 0:
+            total += 4 * d * d + 3 * d * F + (d * d if hp.queryGating else 0)
+        else:
+            qk, vv = hp.gdnHeads * hp.gdnDk, hp.gdnHeads * hp.gdnDv
+            total += 2 * qk * d + 2 * vv * d + 3 * d * F + 2 * hp.gdnHeads * d
+        if hp.pleDim:
+            total += 2 * hp.pleDim * d
+    return total
+
+
+def batched_decode_leg(m, steps=64):
+    """Configuration 4: 64 concurrent sequences of the hybrid architecture, prompt lengths uniform in
+    [32, 512] (seeded), greedy decode.  Returns tok/s and the fraction of the bytes-per-step roofline
+    (weights once per step + every sequence's K/V rows and GDN states)."""
+    hp = m.config(4)
+    nseq = hp.maxSeqs
+    model = m.Model.generate(hp, seed=4)
+    dev = m.Device(hp, 0)
+    dev.upload(model)
+    lens = np.random.default_rng(4).integers(32, 513, size=nseq)
+    prompts = [m.random_tokens(4, s, hp.vocabSize, int(n)) for s, n in enumerate(lens)]
+    dev.prefill_batch(list(range(nseq)), prompts)
+    firsts = [dev.greedy_token(s) for s in range(nseq)]
+    out = dev.decode_loop(firsts, 8)  # warm-up
+    dev.synchronize()
+    t0 = time.perf_counter()
+    out = dev.decode_loop([int(t) for t in out[-1]], steps)
+    dev.synchronize()
+    wall = time.perf_counter() - t0
+    wb = 2 if hp.weightDtype == m.DTYPE_BF16 else 4
+    weights = decode_bytes_per_token(hp, 0, wb) - sum(
+        (2 * hp.dim * 4 if hp.layerKinds[t] == 0 else 2 * hp.gdnHeads * hp.gdnDk * hp.gdnDv * 4) for t in range(hp.transformers))
+    per_seq = [decode_bytes_per_token(hp, int(n) + 8 + steps // 2, wb) - weights for n in lens]
+    step_bytes = weights + float(np.sum(per_seq))
+    dev.close()
+    return {"workload": "config 4: 64 sequences, prompts uniform in [32, 512], hybrid 3 GDN : 1 attention + PLE, fp32",
+            "steps": steps, "ms_per_step": wall / steps * 1e3, "tok_s": nseq * steps / wall,
+            "bytes_per_step": step_bytes, "achieved_GBps": step_bytes / (wall / steps) / 1e9,
+            "frac_of_hbm_peak": step_bytes / (wall / steps) / 1e9 / HBM_PEAK_GBPS,
+            "last_ids": [int(x) for x in out[-1, :4]]}
+
+
+def prefill_leg(m, reps=2):
+    """Configuration 5: 8 prompts of 2048 uniform-random tokens through the bf16 model in one pass.
+    MFMA utilisation = algorithmic flops (projections + causal attention, LM head on the last position
+    only) / time / the published dense bf16 peak; the GEMM kernel alone is also timed on the layer's
+    gate/up shape."""
+    hp = m.config(5)
+    nseq, plen = hp.maxSeqs, 2048
+    model = m.Model.generate(hp, seed=5)
+    dev = m.Device(hp, 0)
+    dev.upload(model)
+    prompts = [m.random_tokens(5, s, hp.vocabSize, plen) for s in range(nseq)]
+    best = None
+    for _ in range(reps + 1):  # the first pass allocates the work buffers
+        dev.reset()
+        dev.synchronize()
+        t0 = time.perf_counter()
+        dev.prefill_batch(list(range(nseq)), prompts)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    tokens = nseq * plen
+    n_attn = sum(1 for t in range(hp.transformers) if hp.layerKinds[t] == 0)
+    flops = 2.0 * tokens * matrix_params(hp) + n_attn * nseq * (4.0 * plen * plen * hp.dim) / 2 + 2.0 * nseq * hp.vocabSize * hp.dim
+    firsts = [dev.greedy_token(s) for s in range(nseq)]
+    t0 = time.perf_counter()
+    dev.decode_loop(firsts, 32)
+    dec = (time.perf_counter() - t0) / 32
+    dev.close()
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((4096, hp.dim), dtype=np.float32)
+    b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
+    _, us = m.selftest_gemm(a, b, None, bf16=True, iters=20)
+    gemm_tflops = 2.0 * 4096 * 2 * hp.ffnDim * hp.dim / us / 1e6
+    return {"workload": "config 5: 8 x 2048-token prompts, d2048 x 24 layers (3 GDN : 1 attention), 16 heads x 128, "
+                        "ffn 5632, vocab 32000, PLE 64, bf16 weights, fp32 accumulation",
+            "tokens": tokens, "ms": best * 1e3, "tok_s": tokens / best, "algo_tflop": flops / 1e12,
+            "achieved_TFLOPs": flops / best / 1e12, "mfma_frac_of_bf16_peak": flops / best / MFMA_BF16_PEAK,
+            "gemm_kernel": {"shape": [4096, 2 * hp.ffnDim, hp.dim], "avg_us": us, "TFLOPs": gemm_tflops,
+                            "frac_of_bf16_peak": gemm_tflops * 1e12 / MFMA_BF16_PEAK},
+            "decode_after_prefill": {"sequences": nseq, "ms_per_step": dec * 1e3, "tok_s": nseq / dec}}
+
+
 def timed_decode(dev, prompt, K, W, persistent, maxL):
     """W untimed warm-up steps, then exactly K timed steps with the device idle on both sides.
     Returns (wall seconds, HIP-event milliseconds of a second identical run, ids)."""
@@ -121,6 +209,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
     ap.add_argument("--path", choices=["persistent", "kernels"], default="kernels",
                     help="decode path reported as `value`")
+    ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
     ap.add_argument("--only-path", action="store_true", help="time only the chosen path (for profiler runs)")
     ap.add_argument("--graph-steps", type=int, default=0,
                     help="kernels path: decode steps per hipGraph replay; 0 = plain launches (use 0 under rocprofv3)")
@@ -213,6 +302,15 @@ def main():
         except Exception as e:  # the baseline is reported, never required
             cpu = {"value": None, "unit": "tok/s", "cores": 0, "kind": "port", "sample": f"failed: {e!r}"}
 
+    dev.close()
+    extras = {}
+    if not args.no_extras and not args.only_path:
+        for name, leg in (("batched_decode", batched_decode_leg), ("prefill", prefill_leg)):
+            try:
+                extras[name] = leg(m)
+            except Exception as e:  # reported alongside, never required for the headline line
+                extras[name] = {"failed": repr(e)}
+
     line = {
         "metric": "decode tok/s @ batch 1 (config 2) + % HBM roofline",
         "value": chosen["tok_s"],
@@ -241,8 +339,8 @@ def main():
         "cpu_baseline": cpu,
         "last_ids": [int(x) for x in ids[-4:]],
     }
+    line.update(extras)
     print(json.dumps(line))
-    dev.close()
     return 0
 
 

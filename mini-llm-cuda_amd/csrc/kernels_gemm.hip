@@ -14,6 +14,8 @@
 // 16-byte reads), the next slice's global loads fly while the current one is multiplied.
 #include <string.h>
 
+#include <algorithm>
+
 #include "mlh_internal.h"
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -320,20 +322,40 @@ static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int ld
 
 // ----------------------------------------------------------------------------
 // Skinny variant for M <= 64 (batched decode: one row per sequence).  The weight matrix is the big
-// operand and is read exactly once: a workgroup owns 32 weight rows, its four waves split K between
-// them in 128-byte chunks and multiply straight out of global memory -- the MFMA operand layout
-// (lane = row, 16 bytes of K) is also a reasonable load pattern: the four 16-byte loads of a lane
-// cover 64 contiguous bytes of its row.  The product is formed transposed, D[n, m] = B . A^T, so a
-// lane ends up with four consecutive n for one m: 16-byte stores into C[m, n..n+3].  The four partial
-// sums meet in LDS and are added in a fixed order.
+// operand and is read exactly once: a workgroup owns 32 weight rows and (with split-K) one slice of
+// K, its four waves take 128-byte chunks of that slice in turn and multiply straight out of global
+// memory -- the MFMA operand layout (lane = row, 16 bytes of K) is also a reasonable load pattern:
+// the four 16-byte loads of a lane cover 64 contiguous bytes of its row.  The next chunk's loads are
+// issued before the current chunk is multiplied.  The product is formed transposed, D[n, m] = B . A^T,
+// so a lane ends up with four consecutive n for one m.  The four waves' partial sums meet in LDS and
+// are added in a fixed order.
+//
+// Split-K over workgroups (matrices with few rows would otherwise occupy a fraction of the CUs):
+// every workgroup writes its partial tile to a workspace and bumps the tile's counter; whichever
+// arrives last adds the partials in slice order -- the result does not depend on arrival order --
+// applies the epilogue and resets the counter.  Partials and counters move with agent-scope atomics
+// (memory-side), which is all the ordering this needs: no cache write-back or invalidate.
 // ----------------------------------------------------------------------------
+__device__ __forceinline__ float g_ald(const float* p) {
+    return __uint_as_float(__hip_atomic_load(reinterpret_cast<const unsigned*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+__device__ __forceinline__ void g_ast(float* p, float v) {
+    __hip_atomic_store(reinterpret_cast<unsigned*>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+#define GSK_COUNTERS 1024 // tiles a split-K launch may have (N <= 32768)
+
 template <typename T, int MB, int EPI>
 __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
-                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K) {
+                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
+                                                          unsigned* counters, float* partials) {
     __shared__ float red[4][MB][16][64];
+    __shared__ int lastFlag;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = blockIdx.x * 32, n32 = lane & 31, half = lane >> 5;
+    const int ks = gridDim.y, kslice = blockIdx.y;
     const int nchunks = (int)(((size_t)K * sizeof(T)) / GKB);
+    const int cbeg = (int)((long)nchunks * kslice / ks), cend = (int)((long)nchunks * (kslice + 1) / ks);
     const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n32, N - 1) * ldb * sizeof(T) + half * 64;
     const unsigned char* arow[MB];
 #pragma unroll
@@ -342,31 +364,73 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
     f32x16 acc[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; mb++) acc[mb] = (f32x16)(0.f);
-    for (int c = wave; c < nchunks; c += 4) {
-        u32x4 fb[4], fa[MB][4];
+    u32x4 fb[2][4], fa[2][MB][4];
+    auto load = [&](int c, int buf) {
 #pragma unroll
-        for (int p = 0; p < 4; p++) fb[p] = *reinterpret_cast<const u32x4*>(brow + (size_t)c * GKB + p * 16);
+        for (int p = 0; p < 4; p++) fb[buf][p] = *reinterpret_cast<const u32x4*>(brow + (size_t)c * GKB + p * 16);
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int p = 0; p < 4; p++) fa[mb][p] = *reinterpret_cast<const u32x4*>(arow[mb] + (size_t)c * GKB + p * 16);
+            for (int p = 0; p < 4; p++) fa[buf][mb][p] = *reinterpret_cast<const u32x4*>(arow[mb] + (size_t)c * GKB + p * 16);
+    };
+    auto mul = [&](int buf) {
         // both operands put the same K elements in the same (half, position) slots, so every k meets itself
 #pragma unroll
         for (int p = 0; p < 4; p++)
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) GemmTraits<T>::mma(fb[p], fa[mb][p], acc[mb]);
+            for (int mb = 0; mb < MB; mb++) GemmTraits<T>::mma(fb[buf][p], fa[buf][mb][p], acc[mb]);
+    };
+    int c = cbeg + wave;
+    if (c < cend) load(c, 0);
+    for (; c < cend; c += 8) { // two chunks per trip so the buffers are addressed statically
+        if (c + 4 < cend) load(c + 4, 1);
+        mul(0);
+        if (c + 4 < cend) {
+            if (c + 8 < cend) load(c + 8, 0);
+            mul(1);
+        }
     }
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
         for (int i = 0; i < 16; i++) red[wave][mb][i][lane] = acc[mb][i];
     __syncthreads();
-    // 2 MB x 4 groups of four accumulator elements; thread (wave, lane) takes groups 2 MB wave / 4 ...
+    // the workgroup's tile: MB x 4 groups of four accumulator elements per lane, wave w takes groups w, w + 4
+    const size_t tileFloats = (size_t)MB * 16 * 64;
+    float* myPart = partials + ((size_t)blockIdx.x * ks + kslice) * tileFloats;
+    if (ks > 1) {
+        for (int g = wave; g < MB * 4; g += 4) {
+            const int mb = g >> 2, i4 = g & 3;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int i = 4 * i4 + j;
+                g_ast(myPart + ((size_t)mb * 16 + i) * 64 + lane, (red[0][mb][i][lane] + red[1][mb][i][lane]) + (red[2][mb][i][lane] + red[3][mb][i][lane]));
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the stores above have been acknowledged ...
+        __syncthreads();                                        // ... for every wave of the workgroup
+        if (tid == 0) {
+            const unsigned prev = __hip_atomic_fetch_add(counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lastFlag = prev == (unsigned)(ks - 1);
+            if (lastFlag) __hip_atomic_store(counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!lastFlag) return;
+    }
     for (int g = wave; g < MB * 4; g += 4) {
         const int mb = g >> 2, i4 = g & 3;
         float v[4];
 #pragma unroll
-        for (int j = 0; j < 4; j++) v[j] = (red[0][mb][4 * i4 + j][lane] + red[1][mb][4 * i4 + j][lane]) + (red[2][mb][4 * i4 + j][lane] + red[3][mb][4 * i4 + j][lane]);
+        for (int j = 0; j < 4; j++) {
+            const int i = 4 * i4 + j;
+            if (ks > 1) {
+                float sum = 0.f;
+                for (int q = 0; q < ks; q++) sum += g_ald(partials + ((size_t)blockIdx.x * ks + q) * tileFloats + ((size_t)mb * 16 + i) * 64 + lane);
+                v[j] = sum;
+            } else {
+                v[j] = (red[0][mb][i][lane] + red[1][mb][i][lane]) + (red[2][mb][i][lane] + red[3][mb][i][lane]);
+            }
+        }
         const int m = mb * 32 + n32, n = n0 + 8 * i4 + 4 * half; // accumulator element i: weight row 8 (i / 4) + 4 half + i % 4, column m
         if (m >= M) continue;
         if (EPI == GEMM_EPI_SWIGLU) {
@@ -385,21 +449,37 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
     }
 }
 
+// Workspace for split-K: GSK_COUNTERS zeroed counters, then the partial tiles.
+size_t mlh_gemm_workspace_bytes(void) { return (size_t)GSK_COUNTERS * 4 + (size_t)256 * 8 * 2 * 16 * 64 * 4; }
+
 template <typename T, int MB>
 static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                                     const float* R, int ldr, int M, int N, int K) {
-    const dim3 grid((N + 31) / 32);
+                                     const float* R, int ldr, int M, int N, int K, void* ws) {
+    const int nblocks = (N + 31) / 32;
+    const int nchunks = (int)(((size_t)K * sizeof(T)) / GKB);
+    int ks = 1;
+    // The exchange costs about three memory round trips (~5 us): only worth it when a wave would otherwise
+    // grind through many chunks on a handful of CUs (few rows, long K).
+    if (ws && nblocks <= 32 && nchunks >= 32) { // aim at ~256 workgroups, every wave with at least one chunk, workspace bounds respected
+        ks = std::min(std::min(8, 256 / nblocks), std::max(1, nchunks / 4));
+        if (nblocks > GSK_COUNTERS || (size_t)nblocks * ks > 256 * 8) ks = 1;
+    }
+    const dim3 grid(nblocks, ks);
+    unsigned* counters = (unsigned*)ws;
+    float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
     if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K);
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials);
     else
-        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K);
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials);
     return hipGetLastError();
 }
 
 // Enqueues the GEMM on `stream`.  Returns hipSuccess, or an error when the shape is not supported.
 // epi = GEMM_EPI_PLAIN: C fp32 [M, N] (+ R).  epi = GEMM_EPI_SWIGLU: C is [M, N/2] in the operand type.
+// ws: optional zero-initialised workspace of mlh_gemm_workspace_bytes() (enables split-K for M <= 64); launches that
+// share a workspace must be ordered on one stream.
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                           const float* R, int ldr, int M, int N, int K) {
+                           const float* R, int ldr, int M, int N, int K, void* ws) {
     const size_t esz = dtype == MLH_DTYPE_BF16 ? 2 : 4;
     if (M <= 0 || N <= 0 || K <= 0 || ((size_t)K * esz) % GKB != 0 || ((size_t)lda * esz) % 16 != 0 || ((size_t)ldb * esz) % 16 != 0)
         return hipErrorInvalidValue;
@@ -407,11 +487,11 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
     // M <= 64 (one row per sequence of a decode batch): weight-streaming skinny kernel; long M: 256 x 256 tiles
     // fed by direct-to-LDS loads; in between: 128 x 128 tiles
     if (M <= 32)
-        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
-                                       : launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws)
+                                       : launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws);
     if (M <= 64)
-        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
-                                       : launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws)
+                                       : launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws);
     if (M > 128)
         return dtype == MLH_DTYPE_BF16 ? launch_gemm_big<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
                                        : launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
@@ -421,7 +501,7 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
 
 hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, const void* B, int ldb, float* C, int ldc,
                        const float* R, int ldr, int M, int N, int K) {
-    return mlh_gemm_tn_epi(stream, dtype, GEMM_EPI_PLAIN, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+    return mlh_gemm_tn_epi(stream, dtype, GEMM_EPI_PLAIN, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, nullptr);
 }
 
 static void host_to_bf16(const float* src, bf16_t* dst, size_t n) {
@@ -441,7 +521,7 @@ extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A,
     if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return -1;
     if (mlh_device_count() <= 0) return -1;
     const size_t esz = dtype == MLH_DTYPE_BF16 ? 2 : 4;
-    void *dA = nullptr, *dB = nullptr;
+    void *dA = nullptr, *dB = nullptr, *dW = nullptr;
     float *dC = nullptr, *dR = nullptr;
     int rc = 0;
     std::vector<bf16_t> ha, hb;
@@ -458,12 +538,14 @@ extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A,
     if (R) { ST(hipMalloc((void**)&dR, (size_t)M * N * 4)); ST(hipMemcpy(dR, R, (size_t)M * N * 4, hipMemcpyHostToDevice)); }
     ST(hipMemcpy(dA, srcA, (size_t)M * K * esz, hipMemcpyHostToDevice));
     ST(hipMemcpy(dB, srcB, (size_t)N * K * esz, hipMemcpyHostToDevice));
-    ST(mlh_gemm_tn(nullptr, dtype, dA, K, dB, K, dC, N, dR, N, M, N, K));
+    ST(hipMalloc(&dW, mlh_gemm_workspace_bytes()));
+    ST(hipMemset(dW, 0, mlh_gemm_workspace_bytes()));
+    ST(mlh_gemm_tn_epi(nullptr, dtype, GEMM_EPI_PLAIN, dA, K, dB, K, dC, N, dR, N, M, N, K, dW));
     ST(hipDeviceSynchronize());
     if (iters > 0 && avgUs) {
         ST(hipEventCreate(&e0)); ST(hipEventCreate(&e1));
         ST(hipEventRecord(e0, nullptr));
-        for (int i = 0; i < iters; i++) ST(mlh_gemm_tn(nullptr, dtype, dA, K, dB, K, dC, N, dR, N, M, N, K));
+        for (int i = 0; i < iters; i++) ST(mlh_gemm_tn_epi(nullptr, dtype, GEMM_EPI_PLAIN, dA, K, dB, K, dC, N, dR, N, M, N, K, dW));
         ST(hipEventRecord(e1, nullptr));
         ST(hipEventSynchronize(e1));
         float ms = 0.f;
@@ -475,6 +557,6 @@ extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A,
 done:
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);
-    (void)hipFree(dA); (void)hipFree(dB); (void)hipFree(dC); (void)hipFree(dR);
+    (void)hipFree(dA); (void)hipFree(dB); (void)hipFree(dC); (void)hipFree(dR); (void)hipFree(dW);
     return rc;
 }

@@ -708,7 +708,7 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
         PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (float*)P.Xn, n, d_),
                        hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (bf16_t*)P.Xn, n, d_));
         { // gate/up projection with SiLU(gate) * up in the epilogue (inference.cu:262-281): U comes out in the GEMM input type
-            hipError_t e_ = mlh_gemm_tn_epi(st, dt, 1, P.Xn, d_, L.W13, d_, P.U, F, nullptr, 0, n, 2 * F, d_);
+            hipError_t e_ = mlh_gemm_tn_epi(st, dt, 1, P.Xn, d_, L.W13, d_, P.U, F, nullptr, 0, n, 2 * F, d_, nullptr);
             if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; }
         }
         GEMM(P.U, F, L.W2, F, P.X, d_, P.H1, d_, n, d_, F);
@@ -814,6 +814,11 @@ int mlh_prepare_batch_step(mlh_ctx* c, int nseq) {
     if (!mlh_batch_step_applicable(c, nseq)) return 0;
     int rc = ensure_prefill_buffers(c, std::max(nseq, 64));
     if (rc) return rc;
+    if (!c->gemmWs) {
+        MLH_CHECK(c, hipMalloc(&c->gemmWs, mlh_gemm_workspace_bytes()));
+        c->allocs.push_back(c->gemmWs);
+        MLH_CHECK(c, hipMemset(c->gemmWs, 0, mlh_gemm_workspace_bytes()));
+    }
     if (!c->pfLogits) {
         MLH_CHECK(c, hipMalloc((void**)&c->pfLogits, (size_t)64 * c->hp.vocabSize * 4));
         c->allocs.push_back(c->pfLogits);
@@ -831,7 +836,7 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
     const bool bf = dt == MLH_DTYPE_BF16;
 #define GEMM(epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)                                                       \
     do {                                                                                                         \
-        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);                   \
+        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, c->gemmWs);                   \
         if (e_ != hipSuccess) { c->err = std::string("batched step GEMM: ") + hipGetErrorString(e_); return -2; } \
     } while (0)
     if (bf) hipLaunchKernelGGL((k_bd_embed<bf16_t>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);

@@ -132,6 +132,7 @@ struct mlh_ctx {
     float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
     void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
     int* pfMeta = nullptr;
+    void* gemmWs = nullptr;    // split-K workspace of the skinny GEMM
     float* pfLogits = nullptr; // [64, vocab] logits of a batched decode step in slot order
 
     std::vector<int> h_len; // host mirror of d_pos
@@ -157,8 +158,11 @@ hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, co
                        const float* R, int ldr, int M, int N, int K);
 // epi 0: as above.  epi 1 (SwiGLU): columns 2j / 2j+1 of the product are gate / up of unit j and
 // C is [M, N/2] in the operand type: C[m, j] = silu(gate) * up.
+// ws: zero-initialised workspace of mlh_gemm_workspace_bytes() or null; with it, M <= 64 products of matrices
+// with few rows are split along K over workgroups (deterministically reduced).
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                           const float* R, int ldr, int M, int N, int K);
+                           const float* R, int ldr, int M, int N, int K, void* ws);
+size_t mlh_gemm_workspace_bytes(void);
 
 // kernels_prefill.hip
 bool mlh_prefill_gemm_supported(const mlh_ctx* c);

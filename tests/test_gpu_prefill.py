@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 # ---- the GEMM by itself -------------------------------------------------------------------------
 @pytest.mark.parametrize("m,n,k", [(128, 128, 32), (1, 1, 32), (17, 300, 96), (130, 257, 704), (64, 1160, 256),
-                                   (300, 128, 2048), (257, 4096, 256)])
+                                   (300, 128, 2048), (257, 4096, 256), (40, 768, 2048), (64, 100, 1024)])
 def test_gemm_fp32(pkg, m, n, k):
     """C = A.B^T (+R) on the fp32 MFMA path against float64 NumPy; ragged M and N, K a multiple of 32."""
     rng = np.random.default_rng(m * 1000 + n + k)
@@ -24,13 +24,15 @@ def test_gemm_fp32(pkg, m, n, k):
     r = rng.standard_normal((m, n), dtype=np.float32)
     for res in (None, r):
         c, _ = pkg.selftest_gemm(a, b, res)
+        c2, _ = pkg.selftest_gemm(a, b, res, iters=3)  # repeated launches on one workspace: split-K counters reset themselves
+        assert np.array_equal(c, c2)
         want = a.astype(np.float64) @ b.astype(np.float64).T + (0 if res is None else res)
         err = np.max(np.abs(c - want))
         # fp32 products summed in fp32: error grows like sqrt(k) * eps * |a||b|
         assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 1, 64), (17, 300, 128), (130, 257, 704), (300, 128, 2048)])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 1, 64), (17, 300, 128), (130, 257, 704), (300, 128, 2048), (8, 2048, 5632), (33, 96, 512)])
 def test_gemm_bf16(pkg, orc, m, n, k):
     """bf16 operands (already representable, so the product is exact in fp32) with fp32 accumulation."""
     rng = np.random.default_rng(m * 1000 + n + k + 1)
