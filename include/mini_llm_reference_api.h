@@ -36,6 +36,11 @@ void initializeRandomWeights(float range);
 /* inference.h:3-4.  runInference(L) consumes seqTokenIndices[0..L) and leaves the
  * last position's logits/probabilities readable through mllDeviceContext(). */
 int runInference(int L);
+/* The same forward over all L positions from scratch, with the contents of
+ * vocabScores_postSoftmax_DEVICE (network_globals.h:172-174: [vocabSize x L], position i at
+ * i * vocabSize) copied to hostProbs and the sequence loss of processSequence
+ * (training_orchestrator.cu:289-359) to meanLoss; either may be null.  0 = success. */
+int runInferenceAllPositions(int L, float* hostProbs, float* meanLoss);
 void getPreComputedRopeTheta(float* preComputedRopeTheta, int maxL_);
 
 /* main.cu:45 (declared extern in inference_orchestrator.cu:26) */

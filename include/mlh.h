@@ -131,6 +131,15 @@ int mlh_prefill(mlh_ctx* ctx, int seq, const int32_t* ids, int n);
  * (inference.cu:511-573), GDN layers run their recurrence over the segment. */
 int mlh_prefill_batch(mlh_ctx* ctx, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens);
 
+/* Teacher-forced forward: appends n tokens to seq like mlh_prefill and returns what
+ * runInference(L) leaves on the device for ALL L columns: logits_out and probs_out are
+ * [n, vocabSize] (position-major, the reference's column-major [V x L] buffers
+ * vocabScores_DEVICE / vocabScores_postSoftmax_DEVICE, inference.cu:723-749); either may be
+ * null.  mean_nll (may be null) receives the mean over positions 0..n-2 of
+ * -log max(p(ids[i+1] | ids[0..i]), 1e-4), the sequence loss processSequence prints
+ * (training_orchestrator.cu:289-359, clamp at :343-347).  Allocates its own staging buffers per call. */
+int mlh_forward_full(mlh_ctx* ctx, int seq, const int32_t* ids, int n, float* logits_out, float* probs_out, float* mean_nll);
+
 /* 0 (default): GEMM prefill when the call has 16 or more tokens and dim, ffnDim,
  * pleDim and the mixing widths are multiples of 32 (fp32) / 64 (bf16);
  * 1: always token by token through the decode kernels. */

@@ -81,6 +81,7 @@ _sigs_dev = {
     "mlh_prefill": (c_int, [c_void_p, c_int, c_void_p, c_int]),
     "mlh_prefill_batch": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p]),
     "mlh_set_prefill_mode": (c_int, [c_void_p, c_int]),
+    "mlh_forward_full": (c_int, [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, _P(c_float)]),
     "mlh_decode_step": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "mlh_decode_loop": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "mlh_greedy_token": (c_int, [c_void_p, c_int, _P(c_int32)]),
@@ -276,6 +277,16 @@ class Device:
         lens = np.array([len(p) for p in prompts], dtype=np.int32)
         ids = np.ascontiguousarray(np.concatenate([np.asarray(p, dtype=np.int32) for p in prompts]), dtype=np.int32)
         self._check(dev.mlh_prefill_batch(self._h, sq.size, sq.ctypes.data, ids.ctypes.data, lens.ctypes.data))
+
+    def forward_full(self, seq, ids, want_probs=True):
+        """Teacher-forced forward over ids appended to seq: (logits [n, V], probs [n, V] or None, mean NLL)."""
+        a = np.ascontiguousarray(ids, dtype=np.int32)
+        lg = np.empty((a.size, self.hp.vocabSize), dtype=np.float32)
+        pr = np.empty_like(lg) if want_probs else None
+        nll = c_float(0)
+        self._check(dev.mlh_forward_full(self._h, seq, a.ctypes.data, a.size, lg.ctypes.data,
+                                         pr.ctypes.data if pr is not None else None, byref(nll)))
+        return lg, pr, float(nll.value)
 
     def set_prefill_mode(self, mode):
         self._check(dev.mlh_set_prefill_mode(self._h, int(mode)))

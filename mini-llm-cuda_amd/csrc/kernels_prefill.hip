@@ -572,6 +572,43 @@ __global__ void __launch_bounds__(PWG) k_pf_finish(PfArgs P, int nparts, int* to
     }
 }
 
+// Row-wise softmax over the vocabulary (inference.cu:293-362) and the cross-entropy of the next token:
+// probs[row] = softmax(logits[row]); nll[row] = -log max(probs[row][target[row]], 1e-4), the clamp of
+// training_orchestrator.cu:343-347 (target < 0: none).
+__global__ void __launch_bounds__(PWG) k_pf_softmax_rows(const float* logits, float* probs, const int* target, float* nll, int V) {
+    __shared__ float red[PWG / 64];
+    const int row = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const float* lg = logits + (size_t)row * V;
+    float m = -3.0e38f;
+    for (int i = tid; i < V; i += PWG) m = fmaxf(m, lg[i]);
+    m = pf_wave_max(m);
+    if (lane == 0) red[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.f;
+    for (int i = tid; i < V; i += PWG) sum += expf(lg[i] - m);
+    sum = pf_wave_sum(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    sum = (red[0] + red[1]) + (red[2] + red[3]);
+    if (probs) {
+        float* pr = probs + (size_t)row * V;
+        for (int i = tid; i < V; i += PWG) pr[i] = expf(lg[i] - m) / sum;
+    }
+    if (nll && tid == 0) {
+        const int t = target[row];
+        nll[row] = t >= 0 ? -logf(fmaxf(expf(lg[t] - m) / sum, 0.0001f)) : 0.f;
+    }
+}
+
+int mlh_launch_softmax_rows(mlh_ctx* c, const float* logits, float* probs, const int* target, float* nll, int rows) {
+    hipLaunchKernelGGL(k_pf_softmax_rows, dim3(rows), dim3(PWG), 0, c->stream, logits, probs, target, nll, c->hp.vocabSize);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { c->err = std::string("softmax launch: ") + hipGetErrorString(e); return -2; }
+    return 0;
+}
+
 // ----------------------------------------------------------------------------
 // host side
 // ----------------------------------------------------------------------------
@@ -624,7 +661,8 @@ static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
 #define PF_DISPATCH_WT(c, expr_f32, expr_bf16) do { if ((c)->hp.weightDtype == MLH_DTYPE_BF16) { expr_bf16; } else { expr_f32; } } while (0)
 
 // Appends lens[s] tokens to sequence seqs[s] for every segment s (token ids concatenated in `ids`).
-int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens) {
+// allLogits: null, or a device buffer [rows, vocab] that receives the logits of every position.
+int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens, float* allLogits) {
     const mlh_hparams& hp = c->hp;
     int n = 0;
     for (int s = 0; s < nseg; s++) n += lens[s];
@@ -714,6 +752,12 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
         GEMM(P.U, F, L.W2, F, P.X, d_, P.H1, d_, n, d_, F);
     }
 #undef GEMM
+    if (allLogits) { // final RMSNorm + tied LM head for every row (inference.cu:705-743 computes all L columns)
+        PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, c->gF, (float*)P.Xn, n, d_),
+                       hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, c->gF, (bf16_t*)P.Xn, n, d_));
+        hipError_t e_ = mlh_gemm_tn(st, dt, P.Xn, d_, c->E, d_, allLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_);
+        if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; }
+    }
     hipLaunchKernelGGL(k_pf_gather_last, dim3(cdiv(d_, PWG), nseg), dim3(PWG), 0, st, P);
     if ((rc = mlh_launch_one(c, MLH_K_LMHEAD, 0, nseg))) return rc;
     hipLaunchKernelGGL(k_pf_finish, dim3(1), dim3(PWG), 0, st, P, c->amaxParts, c->d_tok);

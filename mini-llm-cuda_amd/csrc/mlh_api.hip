@@ -466,7 +466,7 @@ extern "C" int mlh_prefill_batch(mlh_ctx* c, int nseg, const int32_t* seqs, cons
     for (long i = 0; i < total; i++)
         if (ids[i] < 0 || ids[i] >= hp.vocabSize) { c->err = "token id out of range"; return -1; }
     if (c->prefillMode == 0 && total >= MLH_PREFILL_GEMM_MIN_ROWS && mlh_prefill_gemm_supported(c))
-        return mlh_run_prefill_gemm(c, nseg, seqs, ids, lens);
+        return mlh_run_prefill_gemm(c, nseg, seqs, ids, lens, nullptr);
     long off = 0;
     for (int s = 0; s < nseg; s++) {
         if ((rc = prefill_token_by_token(c, seqs[s], ids + off, lens[s]))) return rc;
@@ -477,6 +477,60 @@ extern "C" int mlh_prefill_batch(mlh_ctx* c, int nseg, const int32_t* seqs, cons
 
 extern "C" int mlh_prefill(mlh_ctx* c, int seq, const int32_t* ids, int n) {
     return mlh_prefill_batch(c, 1, &seq, ids, &n);
+}
+
+// Teacher-forced forward over n tokens appended to `seq`: what runInference(L) leaves in vocabScores_DEVICE and
+// vocabScores_postSoftmax_DEVICE for all L columns (inference.cu:723-749), plus the mean next-token cross-entropy.
+extern "C" int mlh_forward_full(mlh_ctx* c, int seq, const int32_t* ids, int n, float* logitsOut, float* probsOut, float* meanNll) {
+    int rc = check_ready(c);
+    if (rc) return rc;
+    const mlh_hparams& hp = c->hp;
+    const size_t V = hp.vocabSize;
+    if (seq < 0 || seq >= hp.maxSeqs) { c->err = "sequence index out of range"; return -1; }
+    if (!ids || n <= 0) { c->err = "empty input"; return -1; }
+    if (c->h_len[seq] + n > hp.maxL) { c->err = "input does not fit in maxL"; return -1; }
+    for (int i = 0; i < n; i++)
+        if (ids[i] < 0 || ids[i] >= hp.vocabSize) { c->err = "token id out of range"; return -1; }
+    float *dLogits = nullptr, *dProbs = nullptr, *dNll = nullptr;
+    int* dTarget = nullptr;
+    std::vector<int> target(n, -1);
+    for (int i = 0; i + 1 < n; i++) target[i] = ids[i + 1];
+    std::vector<float> nll(n, 0.f);
+    hipError_t e = hipMalloc((void**)&dLogits, (size_t)n * V * 4);
+    if (e == hipSuccess && probsOut) e = hipMalloc((void**)&dProbs, (size_t)n * V * 4);
+    if (e == hipSuccess) e = hipMalloc((void**)&dNll, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMalloc((void**)&dTarget, (size_t)n * 4);
+    if (e == hipSuccess) e = hipMemcpy(dTarget, target.data(), (size_t)n * 4, hipMemcpyHostToDevice);
+    if (e != hipSuccess) { c->err = std::string("forward_full buffers: ") + hipGetErrorString(e); rc = -2; }
+    if (rc == 0) {
+        if (c->prefillMode == 0 && n >= MLH_PREFILL_GEMM_MIN_ROWS && mlh_prefill_gemm_supported(c)) {
+            rc = mlh_run_prefill_gemm(c, 1, &seq, ids, &n, dLogits);
+        } else { // token by token through the decode kernels, LM head at every position
+            rc = set_slots(c, &seq, 1);
+            if (rc == 0 && hipMemcpyAsync(c->d_prompt, ids, (size_t)n * 4, hipMemcpyHostToDevice, c->stream) != hipSuccess) rc = -2;
+            for (int i = 0; i < n && rc == 0; i++) {
+                rc = mlh_launch_step(c, 1, c->d_prompt + i, true);
+                if (rc == 0 && hipMemcpyAsync(dLogits + (size_t)i * V, c->logits + (size_t)seq * V, V * 4, hipMemcpyDeviceToDevice, c->stream) != hipSuccess) rc = -2;
+            }
+            if (rc == 0) { if (hipStreamSynchronize(c->stream) != hipSuccess) rc = -2; else c->h_len[seq] += n; }
+            if (rc == -2 && c->err.empty()) c->err = "forward_full: HIP call failed";
+        }
+    }
+    if (rc == 0) rc = mlh_launch_softmax_rows(c, dLogits, dProbs, dTarget, dNll, n);
+    if (rc == 0) {
+        e = hipStreamSynchronize(c->stream);
+        if (e == hipSuccess && logitsOut) e = hipMemcpy(logitsOut, dLogits, (size_t)n * V * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && probsOut) e = hipMemcpy(probsOut, dProbs, (size_t)n * V * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess) e = hipMemcpy(nll.data(), dNll, (size_t)n * 4, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) { c->err = std::string("forward_full read-back: ") + hipGetErrorString(e); rc = -2; }
+    }
+    (void)hipFree(dLogits); (void)hipFree(dProbs); (void)hipFree(dNll); (void)hipFree(dTarget);
+    if (rc == 0 && meanNll) {
+        double s = 0;
+        for (int i = 0; i + 1 < n; i++) s += nll[i];
+        *meanNll = n > 1 ? (float)(s / (n - 1)) : 0.f;
+    }
+    return rc;
 }
 
 extern "C" int mlh_set_prefill_mode(mlh_ctx* c, int mode) {

@@ -170,7 +170,8 @@ int mlh_init_prefill_kernels(mlh_ctx* c);
 bool mlh_batch_step_applicable(const mlh_ctx* c, int nseq);
 int mlh_prepare_batch_step(mlh_ctx* c, int nseq);
 int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr);
-int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens);
+int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_t* ids, const int32_t* lens, float* allLogits);
+int mlh_launch_softmax_rows(mlh_ctx* c, const float* logits, float* probs, const int* target, float* nll, int rows);
 
 // kernels_persistent.hip
 bool mlh_persistent_supported(const mlh_ctx* c);

@@ -167,6 +167,22 @@ int runInference(int L) {
     return 0;
 }
 
+// runInference(L) as the training/verification callers use it (training_orchestrator.cu:289-359): all L
+// positions from scratch, probabilities of every position copied out in the layout of
+// vocabScores_postSoftmax_DEVICE (position i at hostProbs[i * vocabSize ...]).  hostProbs and meanLoss may be null.
+int runInferenceAllPositions(int L, float* hostProbs, float* meanLoss) {
+    const mlh_hparams& hp = current_hp();
+    if (!g_ctx || !seqTokenIndices || L <= 0 || L > hp.maxL) return 1;
+    if (mlh_reset(g_ctx, 0)) return 1;
+    g_cached.clear();
+    if (mlh_forward_full(g_ctx, 0, seqTokenIndices, L, nullptr, hostProbs, meanLoss)) {
+        printf("Error: %s\n", mlh_last_error(g_ctx));
+        return 1;
+    }
+    g_cached.assign(seqTokenIndices, seqTokenIndices + L);
+    return 0;
+}
+
 int loadStoryContext(const char* storiesPath, int storyIndex, int percentage) {
     const mlh_hparams& hp = current_hp();
     if (!seqTokenIndices) { printf("Error: allocateMemory has not been called.\n"); return 0; }

@@ -54,6 +54,7 @@ def test_reference_named_surface_is_exported_with_cxx_linkage(pkg):
     dem = exported_demangled(os.path.join(pkg.LIB_DIR, "libminillm.so"))
     for sig in ("allocateMemory(bool)", "loadVocab(char const*)", "vocabGetToken(int)", "vocabLookup(char const*)",
                 "loadModel(char const*)", "initializeRandomWeights(float)", "runInference(int)",
+                "runInferenceAllPositions(int, float*, float*)",
                 "getPreComputedRopeTheta(float*, int)", "loadStoryContext(char const*, int, int)",
                 "runInferenceLoop(char const*, int, int, bool, bool)", "seqTokenIndices"):
         assert sig in dem, f"{sig} not exported"

@@ -214,3 +214,55 @@ def test_batched_decode_gemm_path_bf16(pkg, orc):
         err = float(np.max(np.abs(dev.logits(s) - lg)) / np.max(np.abs(lg)))
         assert err <= BF16_RTOL, (s, err)
     dev.close()
+
+
+# ---- teacher-forced full-sequence forward ----------------------------------------------------------
+@pytest.mark.parametrize("kind,n,mode", [("attn_flags", 60, 0), ("hybrid", 97, 0), ("hybrid_flags", 40, 1), ("attn", 9, 0)])
+def test_forward_full_all_positions(pkg, orc, kind, n, mode):
+    """Logits and probabilities of EVERY position (what the reference's runInference(L) leaves in its
+    [V x L] buffers) and the mean next-token loss against the float64 oracle's full recompute."""
+    hp = small_cfg(pkg, kind)
+    model, dev, w = make(pkg, orc, hp, seed=41)
+    ids = pkg.random_tokens(41, 0, hp.vocabSize, n)
+    ref = orc.forward_full(w, ids, "f64", last_only=False, want_probs=True)
+    dev.set_prefill_mode(mode)
+    lg, pr, nll = dev.forward_full(0, ids)
+    assert dev.seq_len(0) == n
+    for i in range(n):
+        assert_logits_close(lg[i], ref["logits"][i], FP32_RTOL, f"{kind} position {i}")
+    assert np.max(np.abs(pr - ref["probs"])) <= 1e-6 + FP32_RTOL * np.max(ref["probs"])
+    assert np.allclose(pr.sum(axis=1), 1.0, atol=1e-5)
+    p_next = np.maximum(ref["probs"][np.arange(n - 1), ids[1:]], 1e-4)  # the reference's clamp
+    assert abs(nll - float(np.mean(-np.log(p_next)))) <= 1e-4
+    # the cache is filled as by a prefill: decoding continues from it
+    assert_logits_close(dev.logits(0), ref["logits"][-1], FP32_RTOL, "last position")
+    tok = dev.greedy_token(0)
+    nxt = int(dev.decode_step([tok])[0])
+    dec = orc.Decoder(w, "f64")
+    check_greedy_against_oracle(dec, ids, [tok, nxt], GAP_TOL, what=kind)
+    dev.close()
+
+
+def test_reference_default_architecture(pkg, orc):
+    """The shape the reference ships compiled in (network_meta.h:3-20: dim 768, 6 heads x 128, ffn 3072,
+    16 layers, vocab 20160, QK-norm and query gating on) with its uniform +-0.02 initialisation
+    (random_weights.cu:15-25; own PRNG, cuRAND's stream is not reproducible here): prefill + greedy
+    decode against the float64 oracle."""
+    hp = pkg.reference_defaults()
+    hp.maxL = 128
+    model = pkg.Model.new(hp)
+    model.init_uniform(9, 0.02)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    w = orc.Weights.from_model(model)
+    prompt = pkg.random_tokens(9, 0, hp.vocabSize, 24)
+    dev.prefill(0, prompt)
+    ids = [dev.greedy_token(0)]
+    logits = [dev.logits(0)]
+    for _ in range(5):
+        ids.append(int(dev.decode_step([ids[-1]])[0]))
+        logits.append(dev.logits(0))
+    dec = orc.Decoder(w, "f64")
+    exact, tol = check_greedy_against_oracle(dec, prompt, ids, GAP_TOL, logits, FP32_RTOL, "reference defaults")
+    assert exact + tol == len(ids)
+    dev.close()
