@@ -210,6 +210,8 @@ def main():
     ap.add_argument("--path", choices=["persistent", "kernels"], default="kernels",
                     help="decode path reported as `value`")
     ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
+    ap.add_argument("--leg", choices=["all", "batched", "prefill"], default="all",
+                    help="profiler runs: run only the batched-decode or the prefill leg and print its JSON object")
     ap.add_argument("--only-path", action="store_true", help="time only the chosen path (for profiler runs)")
     ap.add_argument("--graph-steps", type=int, default=0,
                     help="kernels path: decode steps per hipGraph replay; 0 = plain launches (use 0 under rocprofv3)")
@@ -220,6 +222,9 @@ def main():
         return 2
 
     m = entry.load_package()
+    if args.leg != "all":
+        print(json.dumps({args.leg: batched_decode_leg(m) if args.leg == "batched" else prefill_leg(m, reps=1)}))
+        return 0
     hp = m.config(2)
     K, W = max(1, args.steps), max(0, args.warmup)
     if PROMPT_LEN + K > hp.maxL:

@@ -166,9 +166,9 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 // flight while slice s is multiplied, and one barrier per slice separates the stages.
 //
 // A direct load puts lane i's 16 bytes at (wave-uniform base) + 16 i, so rows cannot be padded.  The
-// 8 pieces of a 128-byte row are stored permuted instead: slot j of row r holds piece j ^ ((r >> 1) & 7)
-// -- the lane picks which piece it fetches, not where it lands.  Sixteen consecutive rows reading the
-// same piece then touch sixteen different 16-byte bank groups.
+// 8 pieces of a 128-byte row are stored permuted instead: slot j of row r holds piece j ^ (r & 7)
+// -- the lane picks which piece it fetches, not where it lands.  Eight consecutive rows reading the
+// same piece then touch eight different 16-byte bank groups (one full 128-byte LDS beat).
 // ----------------------------------------------------------------------------
 #define GB_T 256
 #define GB_STAGE (2 * GB_T * GKB) // bytes per stage: A rows then B rows
@@ -192,7 +192,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
 #pragma unroll
     for (int q = 0; q < 8; q++) {
         const int r = wave * 64 + q * 8 + (lane >> 3);
-        const int pc = (lane & 7) ^ ((r >> 1) & 7);
+        const int pc = (lane & 7) ^ (r & 7);
         srcA[q] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(m0 + r, M - 1) * ldaB + pc * 16;
         srcB[q] = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + r, N - 1) * ldbB + pc * 16;
     }
@@ -212,8 +212,8 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
         for (int j = 0; j < 4; j++) acc[i][j] = (f32x16)(0.f);
 
     const int half = lane >> 5, lrow = lane & 31;
-    // row offsets and swizzle keys of this lane's operand rows: rows wm*128 + 32 b + lrow; (row >> 1) & 7 does not depend on b
-    const int keyA = ((wm * 128 + lrow) >> 1) & 7, keyB = ((wn * 128 + lrow) >> 1) & 7;
+    // row offsets and swizzle keys of this lane's operand rows: rows wm*128 + 32 b + lrow; row & 7 does not depend on b
+    const int keyA = (wm * 128 + lrow) & 7, keyB = (wn * 128 + lrow) & 7;
     const int offA = (wm * 128 + lrow) * GKB, offB = GB_T * GKB + (wn * 128 + lrow) * GKB;
 
     issue(0, 0);
