@@ -167,7 +167,7 @@ def prefill_leg(m, reps=2):
     rng = np.random.default_rng(5)
     a = rng.standard_normal((4096, hp.dim), dtype=np.float32)
     b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
-    _, us = m.selftest_gemm(a, b, None, bf16=True, iters=20)
+    _, us = m.selftest_gemm(a, b, None, f16=True, iters=20)  # the operand type the bf16 model's MFMA path multiplies
     gemm_tflops = 2.0 * 4096 * 2 * hp.ffnDim * hp.dim / us / 1e6
     return {"workload": "config 5: 8 x 2048-token prompts, d2048 x 24 layers (3 GDN : 1 attention), 16 heads x 128, "
                         "ffn 5632, vocab 32000, PLE 64, bf16 weights, fp32 accumulation",

@@ -408,7 +408,7 @@ class Vocab:
             pass
 
 
-def selftest_gemm(a, b, r=None, bf16=False, iters=0):
+def selftest_gemm(a, b, r=None, bf16=False, iters=0, f16=False):
     """C = a . b^T (+ r) through the device GEMM kernel; returns (C, mean microseconds or None)."""
     a = np.ascontiguousarray(a, dtype=np.float32)
     b = np.ascontiguousarray(b, dtype=np.float32)
@@ -418,7 +418,7 @@ def selftest_gemm(a, b, r=None, bf16=False, iters=0):
         r = np.ascontiguousarray(r, dtype=np.float32)
     c = np.empty((m, n), dtype=np.float32)
     us = c_double()
-    rc = dev.mlh_selftest_gemm(DTYPE_BF16 if bf16 else DTYPE_F32, m, n, k, a.ctypes.data, b.ctypes.data,
+    rc = dev.mlh_selftest_gemm(2 if f16 else (DTYPE_BF16 if bf16 else DTYPE_F32), m, n, k, a.ctypes.data, b.ctypes.data,
                                r.ctypes.data if r is not None else None, c.ctypes.data, iters, byref(us))
     if rc != 0:
         raise MlhError(f"GEMM self-test failed ({rc}): unsupported shape or no device")

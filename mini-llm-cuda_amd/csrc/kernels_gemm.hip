@@ -21,6 +21,7 @@
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 #define GKB 128           // bytes of K per row and slice
@@ -49,6 +50,16 @@ template <> struct GemmTraits<bf16_t> {
     }
 };
 
+template <> struct GemmTraits<f16_t> {
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x16& c) {
+        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void put(f16_t* p, float v) { // saturating: an overflow must not become inf
+        const _Float16 h = (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f);
+        p->bits = __builtin_bit_cast(uint16_t, h);
+    }
+};
+
 // Workgroups that run at the same time on one XCD (ids congruent mod 8 go to the same XCD and share its
 // L2) get tiles that are neighbours: every XCD takes a contiguous eighth of the tile sequence, and
 // the sequence walks panels of four N tiles top to bottom, so ~32 resident workgroups cover about
@@ -72,7 +83,7 @@ __device__ __forceinline__ void gemm_tile_of(int id, int tilesM, int tilesN, int
 // BM x BN 32x32 blocks per wave, waves arranged 2 x 2: the workgroup tile is 64 BM x 64 BN.
 template <typename T, int BM, int BN, int EPI>
 __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
-                                                      void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN) {
+                                                      void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN, float alpha) {
     constexpr int TM = 64 * BM, TN = 64 * BN;
     constexpr int PA = TM / 32, PB = TN / 32; // 16-byte pieces per thread and slice
     extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
@@ -147,7 +158,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int row = m0 + wm * 32 * BM + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
-                float v = acc[bm][bn][i];
+                float v = acc[bm][bn][i] * alpha;
                 if (EPI == GEMM_EPI_SWIGLU) {
                     const float o = __shfl_xor(v, 1, 64); // the up value sits in the odd neighbour lane
                     if (!(lane & 1) && row < M && col < N) GemmTraits<T>::put((T*)Cv + (size_t)row * ldc + (col >> 1), (v / (1.0f + expf(-v))) * o);
@@ -175,7 +186,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 
 template <typename T, int EPI>
 __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
-                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN) {
+                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN, float alpha) {
     extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -265,7 +276,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int row = m0 + wm * 128 + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
-                float v = acc[bm][bn][i];
+                float v = acc[bm][bn][i] * alpha;
                 if (EPI == GEMM_EPI_SWIGLU) {
                     const float o = __shfl_xor(v, 1, 64);
                     if (!(lane & 1) && row < M && col < N) GemmTraits<T>::put((T*)Cv + (size_t)row * ldc + (col >> 1), (v / (1.0f + expf(-v))) * o);
@@ -279,7 +290,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
 
 template <typename T>
 static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                                  const float* R, int ldr, int M, int N, int K) {
+                                  const float* R, int ldr, int M, int N, int K, float alpha) {
     const int tilesM = (M + GB_T - 1) / GB_T, tilesN = (N + GB_T - 1) / GB_T;
     const unsigned grid = (unsigned)(((tilesM * tilesN + 7) / 8) * 8);
     const size_t lds = 2 * GB_STAGE;
@@ -291,15 +302,15 @@ static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, in
         attr = true;
     }
     if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
     else
-        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
     return hipGetLastError();
 }
 
 template <typename T, int BM, int BN>
 static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                              const float* R, int ldr, int M, int N, int K) {
+                              const float* R, int ldr, int M, int N, int K, float alpha) {
     constexpr int TM = 64 * BM, TN = 64 * BN;
     const int tilesM = (M + TM - 1) / TM, tilesN = (N + TN - 1) / TN;
     const int total = tilesM * tilesN;
@@ -314,9 +325,9 @@ static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int ld
         attr[epi] = true;
     }
     if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_tn<T, BM, BN, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+        hipLaunchKernelGGL((k_gemm_tn<T, BM, BN, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
     else
-        hipLaunchKernelGGL((k_gemm_tn<T, BM, BN, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN);
+        hipLaunchKernelGGL((k_gemm_tn<T, BM, BN, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
     return hipGetLastError();
 }
 
@@ -348,7 +359,7 @@ __device__ __forceinline__ void g_ast(float* p, float v) {
 template <typename T, int MB, int EPI>
 __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
                                                           void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
-                                                          unsigned* counters, float* partials) {
+                                                          unsigned* counters, float* partials, float alpha) {
     __shared__ float red[4][MB][16][64];
     __shared__ int lastFlag;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -431,6 +442,8 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
                 v[j] = (red[0][mb][i][lane] + red[1][mb][i][lane]) + (red[2][mb][i][lane] + red[3][mb][i][lane]);
             }
         }
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] *= alpha;
         const int m = mb * 32 + n32, n = n0 + 8 * i4 + 4 * half; // accumulator element i: weight row 8 (i / 4) + 4 half + i % 4, column m
         if (m >= M) continue;
         if (EPI == GEMM_EPI_SWIGLU) {
@@ -454,7 +467,7 @@ size_t mlh_gemm_workspace_bytes(void) { return (size_t)GSK_COUNTERS * 4 + (size_
 
 template <typename T, int MB>
 static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                                     const float* R, int ldr, int M, int N, int K, void* ws) {
+                                     const float* R, int ldr, int M, int N, int K, void* ws, float alpha) {
     const int nblocks = (N + 31) / 32;
     const int nchunks = (int)(((size_t)K * sizeof(T)) / GKB);
     int ks = 1;
@@ -468,9 +481,9 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
     unsigned* counters = (unsigned*)ws;
     float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
     if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials);
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
     else
-        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials);
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
     return hipGetLastError();
 }
 
@@ -479,29 +492,36 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
 // ws: optional zero-initialised workspace of mlh_gemm_workspace_bytes() (enables split-K for M <= 64); launches that
 // share a workspace must be ordered on one stream.
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                           const float* R, int ldr, int M, int N, int K, void* ws) {
-    const size_t esz = dtype == MLH_DTYPE_BF16 ? 2 : 4;
+                           const float* R, int ldr, int M, int N, int K, void* ws, float alpha) {
+    const size_t esz = dtype == MLH_DTYPE_F32 ? 4 : 2;
     if (M <= 0 || N <= 0 || K <= 0 || ((size_t)K * esz) % GKB != 0 || ((size_t)lda * esz) % 16 != 0 || ((size_t)ldb * esz) % 16 != 0)
         return hipErrorInvalidValue;
     if (epi == GEMM_EPI_SWIGLU && (N & 1)) return hipErrorInvalidValue;
     // M <= 64 (one row per sequence of a decode batch): weight-streaming skinny kernel; long M: 256 x 256 tiles
     // fed by direct-to-LDS loads; in between: 128 x 128 tiles
+#define GEMM_BY_TYPE(call_f32, call_bf16, call_f16) \
+    return dtype == MLH_DTYPE_BF16 ? (call_bf16) : dtype == MLH_GEMM_F16 ? (call_f16) : (call_f32)
     if (M <= 32)
-        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws)
-                                       : launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws);
+        GEMM_BY_TYPE((launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
+                     (launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
+                     (launch_gemm_skinny<f16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)));
     if (M <= 64)
-        return dtype == MLH_DTYPE_BF16 ? launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws)
-                                       : launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws);
+        GEMM_BY_TYPE((launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
+                     (launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
+                     (launch_gemm_skinny<f16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)));
     if (M > 128)
-        return dtype == MLH_DTYPE_BF16 ? launch_gemm_big<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
-                                       : launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
-    return dtype == MLH_DTYPE_BF16 ? launch_gemm<bf16_t, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)
-                                   : launch_gemm<float, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);
+        GEMM_BY_TYPE((launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
+                     (launch_gemm_big<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
+                     (launch_gemm_big<f16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)));
+    GEMM_BY_TYPE((launch_gemm<float, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
+                 (launch_gemm<bf16_t, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
+                 (launch_gemm<f16_t, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)));
+#undef GEMM_BY_TYPE
 }
 
 hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, const void* B, int ldb, float* C, int ldc,
                        const float* R, int ldr, int M, int N, int K) {
-    return mlh_gemm_tn_epi(stream, dtype, GEMM_EPI_PLAIN, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, nullptr);
+    return mlh_gemm_tn_epi(stream, dtype, GEMM_EPI_PLAIN, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, nullptr, 1.0f);
 }
 
 static void host_to_bf16(const float* src, bf16_t* dst, size_t n) {
@@ -514,13 +534,20 @@ static void host_to_bf16(const float* src, bf16_t* dst, size_t n) {
     }
 }
 
+static void host_to_f16(const float* src, f16_t* dst, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        const _Float16 h = (_Float16)src[i];
+        memcpy(&dst[i].bits, &h, 2);
+    }
+}
+
 // Stand-alone check and timing of the GEMM kernel: host fp32 inputs (rounded to bf16 first when
 // dtype says so), result back on the host, mean launch time over `iters` launches from HIP events.
 extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A, const float* B, const float* R, float* C,
                                  int iters, double* avgUs) {
     if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return -1;
     if (mlh_device_count() <= 0) return -1;
-    const size_t esz = dtype == MLH_DTYPE_BF16 ? 2 : 4;
+    const size_t esz = dtype == MLH_DTYPE_F32 ? 4 : 2;
     void *dA = nullptr, *dB = nullptr, *dW = nullptr;
     float *dC = nullptr, *dR = nullptr;
     int rc = 0;
@@ -529,6 +556,10 @@ extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A,
     if (dtype == MLH_DTYPE_BF16) {
         ha.resize((size_t)M * K); hb.resize((size_t)N * K);
         host_to_bf16(A, ha.data(), ha.size()); host_to_bf16(B, hb.data(), hb.size());
+        srcA = ha.data(); srcB = hb.data();
+    } else if (dtype == MLH_GEMM_F16) {
+        ha.resize((size_t)M * K); hb.resize((size_t)N * K);
+        host_to_f16(A, (f16_t*)ha.data(), ha.size()); host_to_f16(B, (f16_t*)hb.data(), hb.size());
         srcA = ha.data(); srcB = hb.data();
     }
     hipEvent_t e0 = nullptr, e1 = nullptr;

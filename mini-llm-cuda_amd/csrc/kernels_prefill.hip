@@ -57,7 +57,7 @@ __device__ __forceinline__ float pf_wave_max(float v) {
 __device__ __forceinline__ float pf_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); } // inference.cu:248
 __device__ __forceinline__ float pf_silu(float v) { return v / (1.0f + expf(-v)); }       // inference.cu:270
 
-// store a float as the GEMM input type (fp32, or bf16 with round-to-nearest-even)
+// store a float as the GEMM input type (fp32; IEEE half for bf16 models, whose MFMA path runs in fp16; bf16)
 template <typename AT> __device__ __forceinline__ void put(AT* p, float v);
 template <> __device__ __forceinline__ void put<float>(float* p, float v) { *p = v; }
 template <> __device__ __forceinline__ void put<bf16_t>(bf16_t* p, float v) {
@@ -65,6 +65,10 @@ template <> __device__ __forceinline__ void put<bf16_t>(bf16_t* p, float v) {
     if ((u & 0x7fffffffu) > 0x7f800000u) u |= 0x00400000u;
     else u += 0x7fffu + ((u >> 16) & 1u);
     *p = (bf16_t)(u >> 16);
+}
+template <> __device__ __forceinline__ void put<f16_t>(f16_t* p, float v) { // saturating: an overflow must not become inf
+    const _Float16 h = (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f);
+    p->bits = __builtin_bit_cast(uint16_t, h);
 }
 template <typename WT> __device__ __forceinline__ float getw(const WT* p);
 template <> __device__ __forceinline__ float getw<float>(const float* p) { return *p; }
@@ -233,7 +237,7 @@ __global__ void __launch_bounds__(PWG) k_pf_attn(PfArgs P, LayerDev L) {
 }
 
 // ----------------------------------------------------------------------------
-// bf16 MFMA causal attention (bf16-weight models).  A workgroup owns one head and 128 consecutive
+// fp16 MFMA causal attention (bf16-weight models; their MFMA path computes in IEEE half, see the host section).  A workgroup owns one head and 128 consecutive
 // queries of one segment, a wave 32 of them.  Per 64-key page:
 //   S^T[key, query] = K . Q^T      (A = K tile from LDS, B = Q^T held in registers)
 //   online softmax down the key axis -- with the transposed product every lane owns ONE query column
@@ -243,20 +247,18 @@ __global__ void __launch_bounds__(PWG) k_pf_attn(PfArgs P, LayerDev L) {
 // The contraction index of the second product may be permuted freely as long as A and B agree: slot
 // (half, e) of 16-key step t is the key the accumulator layout puts there, and the V tile is written
 // to LDS transposed in exactly that order, so P never leaves its registers.
-// K and V come from the fp32 pages and are rounded to bf16 on the way into LDS; scores, softmax
+// K and V come from the fp32 pages and are rounded to fp16 on the way into LDS; scores, softmax
 // statistics and the output accumulate in fp32.
 // ----------------------------------------------------------------------------
 #define PF_MQB 128
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ uint32_t bf16_bits(float v) {
-    uint32_t u = __float_as_uint(v);
-    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) { // two floats -> two IEEE halves (round to nearest even)
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
 }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return bf16_bits(lo) | (bf16_bits(hi) << 16); }
 
 // position of key k (0..63) of a page along the permuted contraction axis of O^T += V^T . P^T
 __device__ __forceinline__ int pv_slot(int k) {
@@ -267,7 +269,7 @@ __device__ __forceinline__ int pv_slot(int k) {
 
 template <int HD>
 __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
-    constexpr int KP = HD + 8;   // K tile row pitch (bf16 elements): 16-byte reads, rows 4 banks apart
+    constexpr int KP = HD + 8;   // K tile row pitch (16-bit elements): 16-byte reads, rows 4 banks apart
     constexpr int VP = 64 + 8;   // V^T row pitch
     constexpr int KS = HD / 16;  // 16-wide contraction steps of K . Q^T
     constexpr int MB = HD / 32;  // 32-row blocks of O^T
@@ -285,15 +287,15 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
     const int maxPos = pos0 + min(q0 + PF_MQB, len) - 1;
     const bool waveActive = q0 + wave * 32 < len;
 
-    // Q^T operand: for step s the lane holds q[16 s + 8 half .. +7] of its query
+    // Q^T operand (fp16): for step s the lane holds q[16 s + 8 half .. +7] of its query
     u32x4 qop[KS];
     {
         const float* q = P.QKV + (size_t)qrow * P.qkvLd + h * HD + 8 * half;
 #pragma unroll
         for (int s = 0; s < KS; s++) {
             const f32x4 lo = *reinterpret_cast<const f32x4*>(q + 16 * s), hi = *reinterpret_cast<const f32x4*>(q + 16 * s + 4);
-            qop[s].x = pack_bf16(lo.x, lo.y); qop[s].y = pack_bf16(lo.z, lo.w);
-            qop[s].z = pack_bf16(hi.x, hi.y); qop[s].w = pack_bf16(hi.z, hi.w);
+            qop[s].x = pack_f16(lo.x, lo.y); qop[s].y = pack_f16(lo.z, lo.w);
+            qop[s].z = pack_f16(hi.x, hi.y); qop[s].w = pack_f16(hi.z, hi.w);
         }
     }
     f32x16 oacc[MB];
@@ -315,7 +317,7 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
             const int r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
             f32x4 kk = (f32x4)(0.f);
             if (j0 + r <= maxPos) kk = *reinterpret_cast<const f32x4*>(L.K + base + (size_t)r * a.dim + c4);
-            u32x2 w; w.x = pack_bf16(kk.x, kk.y); w.y = pack_bf16(kk.z, kk.w);
+            u32x2 w; w.x = pack_f16(kk.x, kk.y); w.y = pack_f16(kk.z, kk.w);
             *reinterpret_cast<u32x2*>(Kt + r * KP + c4) = w;
         }
         // ---- V tile: transposed, keys in contraction-slot order; a lane carries two keys that are neighbours there ----
@@ -326,10 +328,10 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
             if (j0 + k <= maxPos) v0 = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)k * a.dim + c4);
             if (j0 + k + 1 <= maxPos) v1 = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)(k + 1) * a.dim + c4);
             const int slot = pv_slot(k); // even, and pv_slot(k + 1) == slot + 1
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 0) * VP + slot) = pack_bf16(v0.x, v1.x);
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 1) * VP + slot) = pack_bf16(v0.y, v1.y);
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 2) * VP + slot) = pack_bf16(v0.z, v1.z);
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 3) * VP + slot) = pack_bf16(v0.w, v1.w);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 0) * VP + slot) = pack_f16(v0.x, v1.x);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 1) * VP + slot) = pack_f16(v0.y, v1.y);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 2) * VP + slot) = pack_f16(v0.z, v1.z);
+            *reinterpret_cast<uint32_t*>(Vt + (c4 + 3) * VP + slot) = pack_f16(v0.w, v1.w);
         }
         __syncthreads();
         if (!waveActive || j0 > waveMaxPos) continue; // wave-uniform; the barriers above are still reached by every wave
@@ -342,7 +344,7 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
 #pragma unroll
             for (int s = 0; s < KS; s++) {
                 const u32x4 kop = *reinterpret_cast<const u32x4*>(Kt + (32 * b + n32) * KP + 16 * s + 8 * half);
-                sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kop), __builtin_bit_cast(bf16x8, qop[s]), sacc[b], 0, 0, 0);
+                sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kop), __builtin_bit_cast(f16x8, qop[s]), sacc[b], 0, 0, 0);
             }
         }
         // ---- scale, causal mask, online softmax down the key axis ----
@@ -380,12 +382,12 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
         for (int st = 0; st < 4; st++) {
             const int b = st >> 1, e0 = 8 * (st & 1);
             u32x4 pop;
-            pop.x = pack_bf16(sacc[b][e0 + 0], sacc[b][e0 + 1]); pop.y = pack_bf16(sacc[b][e0 + 2], sacc[b][e0 + 3]);
-            pop.z = pack_bf16(sacc[b][e0 + 4], sacc[b][e0 + 5]); pop.w = pack_bf16(sacc[b][e0 + 6], sacc[b][e0 + 7]);
+            pop.x = pack_f16(sacc[b][e0 + 0], sacc[b][e0 + 1]); pop.y = pack_f16(sacc[b][e0 + 2], sacc[b][e0 + 3]);
+            pop.z = pack_f16(sacc[b][e0 + 4], sacc[b][e0 + 5]); pop.w = pack_f16(sacc[b][e0 + 6], sacc[b][e0 + 7]);
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) {
                 const u32x4 vop = *reinterpret_cast<const u32x4*>(Vt + (32 * mb + n32) * VP + 16 * st + 8 * half);
-                oacc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vop), __builtin_bit_cast(bf16x8, pop), oacc[mb], 0, 0, 0);
+                oacc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, vop), __builtin_bit_cast(f16x8, pop), oacc[mb], 0, 0, 0);
             }
         }
     }
@@ -403,7 +405,7 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
                 const f32x4 gt = *reinterpret_cast<const f32x4*>(P.QKV + row * P.qkvLd + L.offG + dcol);
                 o.x *= pf_sigmoid(gt.x); o.y *= pf_sigmoid(gt.y); o.z *= pf_sigmoid(gt.z); o.w *= pf_sigmoid(gt.w);
             }
-            u32x2 w; w.x = pack_bf16(o.x, o.y); w.y = pack_bf16(o.z, o.w);
+            u32x2 w; w.x = pack_f16(o.x, o.y); w.y = pack_f16(o.z, o.w);
             *reinterpret_cast<u32x2*>((bf16_t*)P.Amix + row * P.aLd + dcol) = w;
         }
 }
@@ -524,12 +526,12 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
 }
 
 // e[row][j] = silu(ple gate output) * P[tok][j]
-template <typename WT>
+template <typename WT, typename AT>
 __global__ void k_pf_ple(PfArgs P, LayerDev L) {
     const int row = blockIdx.x, j = threadIdx.x;
     if (j >= P.a.ple) return;
     const float g = P.QKV[(size_t)row * P.qkvLd + L.offPle + j];
-    put<WT>((WT*)P.Eple + (size_t)row * P.a.ple + j, pf_silu(g) * getw<WT>((const WT*)L.pleTable + (size_t)P.ids[row] * P.a.ple + j));
+    put<AT>((AT*)P.Eple + (size_t)row * P.a.ple + j, pf_silu(g) * getw<WT>((const WT*)L.pleTable + (size_t)P.ids[row] * P.a.ple + j));
 }
 
 // residual of the last row of every segment -> decode slot buffer x[slot]
@@ -623,6 +625,78 @@ bool mlh_prefill_gemm_supported(const mlh_ctx* c) {
     return true;
 }
 
+// ---- fp16 operands of the MFMA path for bf16 models ----
+// A bf16 value has 8 significand bits, an IEEE half 11: scaled by a power of two that brings the
+// matrix's largest magnitude just under the half range, every weight down to 2^-29 of that maximum
+// converts exactly, so the MFMA path multiplies the very bf16-rounded weights the GEMV path reads --
+// but against activations that keep 11 significand bits instead of 8.  (Accumulation is fp32 either way.)
+__global__ void k_absmax_bf16(const bf16_t* __restrict__ w, size_t n, unsigned* out) {
+    unsigned m = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) m = max(m, (unsigned)(w[i] & 0x7fffu));
+    for (int o = 32; o > 0; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o, 64));
+    if ((threadIdx.x & 63) == 0 && m) atomicMax(out, m);
+}
+__global__ void k_bf16_to_f16(const bf16_t* __restrict__ w, f16_t* __restrict__ out, size_t n, float scale, unsigned* inexact) {
+    unsigned bad = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const float v = __uint_as_float(((uint32_t)w[i]) << 16) * scale;
+        const _Float16 h = (_Float16)v;
+        out[i].bits = __builtin_bit_cast(uint16_t, h);
+        bad += ((float)h != v);
+    }
+    if (bad) atomicAdd(inexact, bad);
+}
+
+static int build_mirror(mlh_ctx* c, const void* src, size_t n, const void** dst, float* alpha, unsigned* d_scratch) {
+    void* buf = nullptr;
+    MLH_CHECK(c, hipMalloc(&buf, n * 2));
+    c->mirrorAllocs.push_back(buf);
+    MLH_CHECK(c, hipMemsetAsync(d_scratch, 0, 8, c->stream));
+    hipLaunchKernelGGL(k_absmax_bf16, dim3(1024), dim3(256), 0, c->stream, (const bf16_t*)src, n, d_scratch);
+    unsigned h[2] = {0, 0};
+    MLH_CHECK(c, hipMemcpyAsync(h, d_scratch, 4, hipMemcpyDeviceToHost, c->stream));
+    MLH_CHECK(c, hipStreamSynchronize(c->stream));
+    // largest magnitude = bf16 bits h[0]; its exponent e (unbiased): scale 2^(14 - e) puts it in [2^14, 2^15)
+    const int e = (int)((h[0] >> 7) & 0xff) - 127;
+    const int k = h[0] ? 14 - e : 0;
+    const float scale = ldexpf(1.0f, k);
+    hipLaunchKernelGGL(k_bf16_to_f16, dim3(1024), dim3(256), 0, c->stream, (const bf16_t*)src, (f16_t*)buf, n, scale, d_scratch + 1);
+    MLH_CHECK(c, hipMemcpyAsync(h, d_scratch, 8, hipMemcpyDeviceToHost, c->stream));
+    MLH_CHECK(c, hipStreamSynchronize(c->stream));
+    c->f16Inexact += h[1];
+    *dst = buf;
+    *alpha = ldexpf(1.0f, -k);
+    return 0;
+}
+
+int mlh_build_gemm_operands(mlh_ctx* c) {
+    const mlh_hparams& hp = c->hp;
+    const bool mirror = hp.weightDtype == MLH_DTYPE_BF16 && mlh_prefill_gemm_supported(c);
+    c->gemmDtype = mirror ? MLH_GEMM_F16 : hp.weightDtype;
+    c->f16Inexact = 0;
+    for (void* p : c->mirrorAllocs) (void)hipFree(p); // a repeated finalize rebuilds them
+    c->mirrorAllocs.clear();
+    unsigned* d_scratch = nullptr;
+    if (mirror) { MLH_CHECK(c, hipMalloc((void**)&d_scratch, 8)); }
+    int rc = 0;
+    for (LayerDev& L : c->layers) {
+        L.WaG = L.Wa; L.WoG = L.Wo; L.W13G = L.W13; L.W2G = L.W2; L.pleUpG = L.pleUp;
+        L.sWa = L.sWo = L.sW13 = L.sW2 = L.sPle = 1.0f;
+        if (!mirror) continue;
+        const size_t d = hp.dim, F = hp.ffnDim;
+        if ((rc = build_mirror(c, L.Wa, (size_t)L.rowsA * d, &L.WaG, &L.sWa, d_scratch)) ||
+            (rc = build_mirror(c, L.Wo, d * L.ad, &L.WoG, &L.sWo, d_scratch)) ||
+            (rc = build_mirror(c, L.W13, 2 * F * d, &L.W13G, &L.sW13, d_scratch)) ||
+            (rc = build_mirror(c, L.W2, d * F, &L.W2G, &L.sW2, d_scratch)))
+            break;
+        if (hp.pleDim > 0 && (rc = build_mirror(c, L.pleUp, d * hp.pleDim, &L.pleUpG, &L.sPle, d_scratch))) break;
+    }
+    c->EG = c->E; c->sE = 1.0f;
+    if (rc == 0 && mirror) rc = build_mirror(c, c->E, (size_t)hp.vocabSize * hp.dim, &c->EG, &c->sE, d_scratch);
+    if (d_scratch) (void)hipFree(d_scratch);
+    return rc;
+}
+
 // The headDim-128 attention tiles exceed the 64 KB a launch may use without opting in.
 int mlh_init_prefill_kernels(mlh_ctx* c) {
     const int lds = (2 * 64 * 132 + PF_QB * 128) * 4;
@@ -706,10 +780,10 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     P.blkSeg = d_blk; P.blkQ0 = d_blk + c->pfBlkCap;
     P.X = c->pfX; P.Xn = c->pfXn; P.QKV = c->pfQKV; P.qkvLd = c->maxRowsA; P.Amix = c->pfA; P.aLd = c->maxAd;
     P.Eple = c->pfE; P.H1 = c->pfH1; P.U = c->pfU;
-    const int d_ = hp.dim, F = hp.ffnDim, dt = hp.weightDtype;
-#define GEMM(A, lda, B, ldb, C, ldc, R, ldr, M, N, K)                                                       \
+    const int d_ = hp.dim, F = hp.ffnDim, dt = c->gemmDtype;
+#define GEMM(A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K)                                                \
     do {                                                                                                    \
-        hipError_t e_ = mlh_gemm_tn(st, dt, A, lda, B, ldb, C, ldc, R, ldr, M, N, K);                       \
+        hipError_t e_ = mlh_gemm_tn_epi(st, dt, 0, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, nullptr, alpha); \
         if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; } \
     } while (0)
 
@@ -718,8 +792,8 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     for (int t = hp.transformers - 1; t >= 0; t--) { // file block 0 is the top (inference.cu:384-385)
         const LayerDev& L = c->layers[t];
         PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, L.g1, (float*)P.Xn, n, d_),
-                       hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, L.g1, (bf16_t*)P.Xn, n, d_));
-        GEMM(P.Xn, d_, L.Wa, d_, P.QKV, P.qkvLd, nullptr, 0, n, L.rowsA, d_);
+                       hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, L.g1, (f16_t*)P.Xn, n, d_));
+        GEMM(P.Xn, d_, L.WaG, L.sWa, d_, P.QKV, P.qkvLd, nullptr, 0, n, L.rowsA, d_);
         if (L.kind == MLH_KIND_ATTENTION) {
             if (hp.headDim == 64) {
                 hipLaunchKernelGGL((k_pf_qk_rope_kv<64>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
@@ -732,30 +806,30 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
             }
         } else if (hp.gdnDk == 64) {
             PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<64, float>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_gdn<64, bf16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
+                           hipLaunchKernelGGL((k_pf_gdn<64, f16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
         } else {
             PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<128, float>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_gdn<128, bf16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
+                           hipLaunchKernelGGL((k_pf_gdn<128, f16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
         }
-        GEMM(P.Amix, P.aLd, L.Wo, L.ad, P.H1, d_, P.X, d_, n, d_, L.ad);
+        GEMM(P.Amix, P.aLd, L.WoG, L.sWo, L.ad, P.H1, d_, P.X, d_, n, d_, L.ad);
         if (hp.pleDim > 0) {
-            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_ple<float>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_ple<bf16_t>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L));
-            GEMM(P.Eple, hp.pleDim, L.pleUp, hp.pleDim, P.H1, d_, P.H1, d_, n, d_, hp.pleDim);
+            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_ple<float, float>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L),
+                           hipLaunchKernelGGL((k_pf_ple<bf16_t, f16_t>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L));
+            GEMM(P.Eple, hp.pleDim, L.pleUpG, L.sPle, hp.pleDim, P.H1, d_, P.H1, d_, n, d_, hp.pleDim);
         }
         PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (float*)P.Xn, n, d_),
-                       hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (bf16_t*)P.Xn, n, d_));
+                       hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (f16_t*)P.Xn, n, d_));
         { // gate/up projection with SiLU(gate) * up in the epilogue (inference.cu:262-281): U comes out in the GEMM input type
-            hipError_t e_ = mlh_gemm_tn_epi(st, dt, 1, P.Xn, d_, L.W13, d_, P.U, F, nullptr, 0, n, 2 * F, d_, nullptr);
+            hipError_t e_ = mlh_gemm_tn_epi(st, dt, 1, P.Xn, d_, L.W13G, d_, P.U, F, nullptr, 0, n, 2 * F, d_, nullptr, L.sW13);
             if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; }
         }
-        GEMM(P.U, F, L.W2, F, P.X, d_, P.H1, d_, n, d_, F);
+        GEMM(P.U, F, L.W2G, L.sW2, F, P.X, d_, P.H1, d_, n, d_, F);
     }
 #undef GEMM
     if (allLogits) { // final RMSNorm + tied LM head for every row (inference.cu:705-743 computes all L columns)
         PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, c->gF, (float*)P.Xn, n, d_),
-                       hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, c->gF, (bf16_t*)P.Xn, n, d_));
-        hipError_t e_ = mlh_gemm_tn(st, dt, P.Xn, d_, c->E, d_, allLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_);
+                       hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.X, c->gF, (f16_t*)P.Xn, n, d_));
+        hipError_t e_ = mlh_gemm_tn_epi(st, dt, 0, P.Xn, d_, c->EG, d_, allLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_, nullptr, c->sE);
         if (e_ != hipSuccess) { c->err = std::string("prefill GEMM: ") + hipGetErrorString(e_); return -2; }
     }
     hipLaunchKernelGGL(k_pf_gather_last, dim3(cdiv(d_, PWG), nseg), dim3(PWG), 0, st, P);
@@ -788,7 +862,7 @@ __global__ void k_bd_embed(StepArgs a) {
 // Mixing output rows in the GEMM input type: attention layers combine the split-KV partials of the decode
 // attention kernel and apply the sigmoid gate (inference.cu:241-250); GDN layers convert the read-out.
 // PLE rows e = silu(gate) * P[tok] ride along.
-template <typename AT>
+template <typename WT, typename AT>
 __global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix, int aLd, AT* Eple) {
     const int slot = blockIdx.x, tid = threadIdx.x;
     const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
@@ -814,7 +888,7 @@ __global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix
         for (int i = tid; i < L.ad; i += PWG) put<AT>(Amix + (size_t)slot * aLd + i, a.mix[(size_t)slot * L.ad + i]);
     }
     for (int j = tid; j < a.ple; j += PWG)
-        put<AT>(Eple + (size_t)slot * a.ple + j, pf_silu(qkv[L.offPle + j]) * getw<AT>((const AT*)L.pleTable + (size_t)a.tok[slot] * a.ple + j));
+        put<AT>(Eple + (size_t)slot * a.ple + j, pf_silu(qkv[L.offPle + j]) * getw<WT>((const WT*)L.pleTable + (size_t)a.tok[slot] * a.ple + j));
 }
 
 // One workgroup per slot: argmax of the slot's logits (lowest index on ties), logits copied to the
@@ -876,34 +950,34 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
     StepArgs a;
     mlh_fill_args(c, a, nseq, tokPtr);
     hipStream_t st = c->stream;
-    const int d_ = hp.dim, F = hp.ffnDim, dt = hp.weightDtype, n = nseq;
-    const bool bf = dt == MLH_DTYPE_BF16;
-#define GEMM(epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K)                                                       \
+    const int d_ = hp.dim, F = hp.ffnDim, dt = c->gemmDtype, n = nseq;
+    const bool bf = hp.weightDtype == MLH_DTYPE_BF16;
+#define GEMM(epi, A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K)                                                \
     do {                                                                                                         \
-        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, c->gemmWs);                   \
+        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, c->gemmWs, alpha);  \
         if (e_ != hipSuccess) { c->err = std::string("batched step GEMM: ") + hipGetErrorString(e_); return -2; } \
     } while (0)
     if (bf) hipLaunchKernelGGL((k_bd_embed<bf16_t>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);
     else hipLaunchKernelGGL((k_bd_embed<float>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);
     for (int t = hp.transformers - 1; t >= 0; t--) {
         const LayerDev& L = c->layers[t];
-        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (bf16_t*)c->pfXn, n, d_);
+        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (f16_t*)c->pfXn, n, d_);
         else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (float*)c->pfXn, n, d_);
-        GEMM(0, c->pfXn, d_, L.Wa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
+        GEMM(0, c->pfXn, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
         int rc = mlh_launch_one(c, L.kind == MLH_KIND_ATTENTION ? MLH_K_ATTN : MLH_K_GDN, t, nseq);
         if (rc) return rc;
-        if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t>), dim3(n), dim3(PWG), 0, st, a, L, (bf16_t*)c->pfA, c->maxAd, (bf16_t*)c->pfE);
-        else hipLaunchKernelGGL((k_bd_mix<float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd, (float*)c->pfE);
-        GEMM(0, c->pfA, c->maxAd, L.Wo, L.ad, c->h1, d_, c->x, d_, n, d_, L.ad);
-        if (hp.pleDim > 0) GEMM(0, c->pfE, hp.pleDim, L.pleUp, hp.pleDim, c->h1, d_, c->h1, d_, n, d_, hp.pleDim);
-        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (bf16_t*)c->pfXn, n, d_);
+        if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd, (f16_t*)c->pfE);
+        else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd, (float*)c->pfE);
+        GEMM(0, c->pfA, c->maxAd, L.WoG, L.sWo, L.ad, c->h1, d_, c->x, d_, n, d_, L.ad);
+        if (hp.pleDim > 0) GEMM(0, c->pfE, hp.pleDim, L.pleUpG, L.sPle, hp.pleDim, c->h1, d_, c->h1, d_, n, d_, hp.pleDim);
+        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (f16_t*)c->pfXn, n, d_);
         else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (float*)c->pfXn, n, d_);
-        GEMM(1, c->pfXn, d_, L.W13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_);
-        GEMM(0, c->pfU, F, L.W2, F, c->x, d_, c->h1, d_, n, d_, F);
+        GEMM(1, c->pfXn, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_);
+        GEMM(0, c->pfU, F, L.W2G, L.sW2, F, c->x, d_, c->h1, d_, n, d_, F);
     }
-    if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<bf16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (bf16_t*)c->pfXn, n, d_);
+    if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (f16_t*)c->pfXn, n, d_);
     else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (float*)c->pfXn, n, d_);
-    GEMM(0, c->pfXn, d_, c->E, d_, c->pfLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_);
+    GEMM(0, c->pfXn, d_, c->EG, c->sE, d_, c->pfLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_);
 #undef GEMM
     hipLaunchKernelGGL(k_bd_finish, dim3(n), dim3(PWG), 0, st, a, c->pfLogits, c->d_tok);
     hipError_t e = hipGetLastError();

@@ -79,6 +79,7 @@ extern "C" void mlh_destroy(mlh_ctx* c) {
     for (int i = 0; i < 2; i++) if (c->graphExec[i]) (void)hipGraphExecDestroy(c->graphExec[i]);
     for (void* p : c->allocs) (void)hipFree(p);
     for (void* p : c->pfAllocs) (void)hipFree(p);
+    for (void* p : c->mirrorAllocs) (void)hipFree(p);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
 }
@@ -358,6 +359,7 @@ extern "C" int mlh_finalize(mlh_ctx* c) {
     (void)hipSetDevice(c->device);
     int rc = mlh_init_kernels(c);
     if (rc == 0) rc = mlh_init_prefill_kernels(c);
+    if (rc == 0) rc = mlh_build_gemm_operands(c);
     if (rc) return rc;
     MLH_CHECK(c, hipMemcpy(c->d_layers, c->layers.data(), c->layers.size() * sizeof(LayerDev), hipMemcpyHostToDevice));
     MLH_CHECK(c, hipDeviceSynchronize());

@@ -14,6 +14,9 @@
 #define MLH_WAVE 64
 
 typedef uint16_t bf16_t;
+// IEEE half, as the MFMA path stores weights and activations of bf16 models (see MLH_GEMM_F16)
+struct f16_t { uint16_t bits; };
+#define MLH_GEMM_F16 2 // GEMM operand type code beside MLH_DTYPE_F32 / MLH_DTYPE_BF16
 
 // Device-side description of one transformer block.
 struct LayerDev {
@@ -35,6 +38,10 @@ struct LayerDev {
     int kind;
     int rowsA, offK, offV, offG, offPle, offGa, offGb;
     int ad;               // width of the mixing output fed to Wo
+    // What the MFMA path multiplies: the matrices themselves for fp32 models; for bf16 models IEEE-half
+    // mirrors scaled by a power of two (exact), with the inverse scale applied to the product.
+    const void *WaG, *WoG, *W13G, *W2G, *pleUpG;
+    float sWa, sWo, sW13, sW2, sPle;
 };
 
 // Arguments shared by all kernels of a decode step.
@@ -132,6 +139,11 @@ struct mlh_ctx {
     float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
     void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
     int* pfMeta = nullptr;
+    const void* EG = nullptr;  // LM-head matrix as the MFMA path reads it (see LayerDev::WaG)
+    float sE = 1.0f;
+    int gemmDtype = MLH_DTYPE_F32; // operand type of the MFMA path: MLH_DTYPE_F32 or MLH_GEMM_F16
+    std::vector<void*> mirrorAllocs;
+    long f16Inexact = 0;       // bf16 weights that had no exact scaled-half representation (reported at finalize)
     void* gemmWs = nullptr;    // split-K workspace of the skinny GEMM
     float* pfLogits = nullptr; // [64, vocab] logits of a batched decode step in slot order
 
@@ -160,13 +172,15 @@ hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, co
 // C is [M, N/2] in the operand type: C[m, j] = silu(gate) * up.
 // ws: zero-initialised workspace of mlh_gemm_workspace_bytes() or null; with it, M <= 64 products of matrices
 // with few rows are split along K over workgroups (deterministically reduced).
+// alpha scales the product before the epilogue (the power of two an fp16 weight mirror was scaled by, inverted).
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                           const float* R, int ldr, int M, int N, int K, void* ws);
+                           const float* R, int ldr, int M, int N, int K, void* ws, float alpha = 1.0f);
 size_t mlh_gemm_workspace_bytes(void);
 
 // kernels_prefill.hip
 bool mlh_prefill_gemm_supported(const mlh_ctx* c);
 int mlh_init_prefill_kernels(mlh_ctx* c);
+int mlh_build_gemm_operands(mlh_ctx* c); // at finalize: fp16 mirrors for bf16 models
 bool mlh_batch_step_applicable(const mlh_ctx* c, int nseq);
 int mlh_prepare_batch_step(mlh_ctx* c, int nseq);
 int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr);

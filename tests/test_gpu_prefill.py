@@ -46,6 +46,17 @@ def test_gemm_bf16(pkg, orc, m, n, k):
         assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
 
 
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 5632), (130, 257, 704), (300, 4096, 2048)])
+def test_gemm_f16(pkg, m, n, k):
+    """IEEE-half operands (what the MFMA path of bf16 models multiplies) with fp32 accumulation."""
+    rng = np.random.default_rng(m + n + k)
+    a = rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).astype(np.float32)
+    b = rng.standard_normal((n, k), dtype=np.float32).astype(np.float16).astype(np.float32)
+    c, _ = pkg.selftest_gemm(a, b, None, f16=True)
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    assert np.max(np.abs(c - want)) <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5
+
+
 def test_gemm_rejects_bad_k(pkg):
     a = np.zeros((4, 40), dtype=np.float32)
     with pytest.raises(RuntimeError):
@@ -141,8 +152,9 @@ def test_prefill_paged(pkg, orc):
 
 @pytest.mark.parametrize("kind,plen", [("attn_flags", 90), ("hybrid", 100), ("hd128", 199), ("attn_long", 333)])
 def test_prefill_bf16(pkg, orc, kind, plen):
-    """bf16 weights: GEMM prefill (bf16 GEMM inputs) within 2e-2 of the float64 oracle on bf16-rounded
-    weights, and of the token-by-token path (fp32 activations)."""
+    """bf16 weights: the MFMA prefill multiplies exact fp16 mirrors of the bf16-rounded weights with
+    activations rounded to fp16: within 2e-2 (stated) and 4e-3 (asserted) of the float64 oracle on the
+    bf16-rounded weights, relative to the largest logit; likewise the token-by-token path (fp32 activations)."""
     hp = small_cfg(pkg, kind, weightDtype=pkg.DTYPE_BF16)
     model, dev, w = make(pkg, orc, hp, seed=25, bf16=True)
     prompt = pkg.random_tokens(25, 0, hp.vocabSize, plen)
@@ -154,7 +166,7 @@ def test_prefill_bf16(pkg, orc, kind, plen):
     worst = float(np.max(np.abs(got - want) / den))
     scale_err = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
     print(f"{kind}: bf16 prefill worst rel {worst:.3e}, max|diff|/max|logit| {scale_err:.3e}")
-    assert scale_err <= BF16_RTOL
+    assert scale_err <= 4e-3 <= BF16_RTOL
     dev.reset()
     dev.set_prefill_mode(1)
     dev.prefill(0, prompt)
