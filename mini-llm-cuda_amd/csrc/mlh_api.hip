@@ -196,6 +196,9 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         (rc = dev_alloc(c, &c->pamaxVal, (size_t)c->numCUs)) || (rc = dev_alloc(c, &c->pamaxIdx, (size_t)c->numCUs)) ||
         (rc = dev_alloc(c, &c->kvPart, (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2))))
         return bail(rc);
+    c->taggedWords = (size_t)2 * d + c->maxRowsA + (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2) + c->maxAd + F + 2 * (size_t)c->numCUs + 64;
+    if ((rc = dev_alloc(c, &c->tagged, c->taggedWords)))
+        return bail(rc);
     if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1)))) return bail(rc);
     c->copyBytes = (size_t)256 << 20;
     char *cs, *cd;
@@ -574,11 +577,14 @@ static void dump_persistent_timing(mlh_ctx* c) {
     const int n = 16 * c->hp.transformers;
     std::vector<unsigned long long> t(n);
     if (hipMemcpy(t.data(), c->d_timing, (size_t)n * 8, hipMemcpyDeviceToHost) != hipSuccess) return;
-    static const char* names[15] = {"A.norm", "A.rows", "A->B sync", "B.mix", "B->C sync", "C.prologue", "C.rows", "C->D sync",
+    const char* names[15] = {"A.norm", "A.rows", "A->B sync", "B.mix", "B->C sync", "C.prologue", "C.rows", "C->D sync",
                                     "D.norm", "D.rows", "D->E sync", "E.load", "E.rows", "E->A sync", "x.load"};
     double tot[15] = {0};
     for (int l = 0; l < c->hp.transformers; l++)
         for (int k = 0; k < 15; k++) tot[k] += (double)(t[l * 16 + k + 1] - t[l * 16 + k]) / 100.0; // 100 MHz clock
+    static const char* tnames[15] = {"x.wait", "A.norm", "A.rows", "B.mix", "C.wait", "C.rows", "h1.wait", "D.norm", "D.rows",
+                                     "u.wait", "E.rows", "-", "-", "-", "-"};
+    if (c->usePersistent == 2) for (int k = 0; k < 15; k++) names[k] = tnames[k];
     fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
     double sum = 0;
     for (int k = 0; k < 15; k++) { fprintf(stderr, " %s=%.2f", names[k], tot[k] / c->hp.transformers); sum += tot[k] / c->hp.transformers; }
@@ -752,7 +758,8 @@ extern "C" int mlh_set_graph(mlh_ctx* c, int stepsPerGraph) {
 
 extern "C" int mlh_set_persistent(mlh_ctx* c, int enabled) {
     if (!c) return -1;
-    c->usePersistent = enabled != 0;
+    if (enabled < 0 || enabled > 2) { c->err = "persistent mode must be 0, 1 or 2"; return -1; }
+    c->usePersistent = enabled;
     return 0;
 }
 

@@ -121,7 +121,9 @@ struct mlh_ctx {
     // persistent batch-1 decode kernel
     int numCUs = 0;
     bool coopLaunch = false;
-    bool usePersistent = false;
+    int usePersistent = 0;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange
+    unsigned long long* tagged = nullptr; // (value, tag) exchange words of mode 2
+    size_t taggedWords = 0;
     LayerDev* d_layers = nullptr;  // device copy of `layers`
     unsigned* d_sync = nullptr;    // barrier words + abort flag
     float* pamaxVal = nullptr;     // [numCUs]

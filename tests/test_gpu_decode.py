@@ -49,7 +49,7 @@ def make(pkg, orc, hp, seed, bf16=False):
     return model, dev, w
 
 
-@pytest.mark.parametrize("persistent", [1, 0], ids=["persistent", "kernels"])
+@pytest.mark.parametrize("persistent", [2, 1, 0], ids=["tagged", "persistent", "kernels"])
 @pytest.mark.parametrize("kind,plen,steps", [("attn", 16, 40), ("attn_flags", 16, 40), ("hybrid", 16, 40),
                                              ("hybrid_flags", 16, 40), ("hd128", 16, 40), ("attn_long", 300, 12)])
 def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
@@ -72,7 +72,7 @@ def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
     dev.close()
 
 
-@pytest.mark.parametrize("persistent", [1, 0], ids=["persistent", "kernels"])
+@pytest.mark.parametrize("persistent", [2, 1, 0], ids=["tagged", "persistent", "kernels"])
 def test_config1_golden_horizon(pkg, orc, persistent):
     """Configuration 1 at full size: 16-token prompt, 128 greedy steps on the device loop, checked
     against the oracle and against the committed golden ids."""
