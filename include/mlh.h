@@ -170,15 +170,17 @@ int mlh_read_logits(mlh_ctx* ctx, int seq, float* out);
 /* Softmax of those logits (vocabScores_postSoftmax_DEVICE, inference.cu:745-749). */
 int mlh_read_probs(mlh_ctx* ctx, int seq, float* out);
 
-/* How decode steps are issued: 0 = plain kernel launches; k >= 1 = replays of a captured
- * hipGraph that covers k consecutive decode steps (default 1; at most 64). */
+/* How the kernel-sequence decode step is issued: 0 = plain kernel launches (default); k >= 1 = replays
+ * of a captured hipGraph that covers k consecutive decode steps (at most 64). */
 int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
 
-/* Batch-1 decode (nseq = 1) runs, when enabled (default off) and the shape allows it, as ONE
- * cooperative launch of a persistent kernel that decodes all requested steps: the ~60 dependent
- * phases of a token are separated by grid barriers instead of kernel launches.  Disabled, or for
- * nseq > 1, the step is a sequence of kernels issued as mlh_set_graph says. */
-int mlh_set_persistent(mlh_ctx* ctx, int enabled);
+/* Batch-1 decode (nseq = 1): mode 1 (default) runs, when the shape allows it, as ONE launch of a
+ * persistent kernel (one workgroup per compute unit) that decodes all requested steps: the ~60
+ * dependent phases of a token are separated by grid barriers instead of kernel launches.  Mode 2 is
+ * the same kernel without barriers (consumers spin on tagged data words).  Both need every compute
+ * unit free; their waits are bounded, and a call whose wait expired returns -3 with a message.
+ * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says. */
+int mlh_set_persistent(mlh_ctx* ctx, int mode);
 
 int mlh_synchronize(mlh_ctx* ctx);
 

@@ -121,7 +121,7 @@ struct mlh_ctx {
     // persistent batch-1 decode kernel
     int numCUs = 0;
     bool coopLaunch = false;
-    int usePersistent = 0;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange
+    int usePersistent = 1;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange
     unsigned long long* tagged = nullptr; // (value, tag) exchange words of mode 2
     size_t taggedWords = 0;
     LayerDev* d_layers = nullptr;  // device copy of `layers`
