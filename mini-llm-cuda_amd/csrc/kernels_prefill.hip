@@ -82,17 +82,24 @@ __global__ void k_pf_embed(PfArgs P) {
     P.X[(size_t)row * P.a.dim + i] = getw<WT>((const WT*)P.a.E + (size_t)P.ids[row] * P.a.dim + i);
 }
 
-// inference.cu:24-50 + 83-95, one wave per row
+// inference.cu:24-50 + 83-95, one wave per row (d is a multiple of 8 on this path: 16-byte loads)
 template <typename AT>
 __global__ void __launch_bounds__(PWG) k_pf_rmsnorm(const float* __restrict__ X, const float* __restrict__ gamma, AT* out, int n, int d) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (row >= n) return;
     const float* x = X + (size_t)row * d;
     float s = 0.f;
-    for (int i = lane; i < d; i += 64) s = fmaf(x[i], x[i], s);
+    for (int i = lane * 4; i < d; i += 256) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(x + i);
+        s = fmaf(v.x, v.x, s); s = fmaf(v.y, v.y, s); s = fmaf(v.z, v.z, s); s = fmaf(v.w, v.w, s);
+    }
     s = pf_wave_sum(s);
     const float r = sqrtf(s / (float)d + 1e-8f);
-    for (int i = lane; i < d; i += 64) put<AT>(out + (size_t)row * d + i, gamma[i] * (x[i] / r));
+    for (int i = lane * 4; i < d; i += 256) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(x + i), g = *reinterpret_cast<const f32x4*>(gamma + i);
+        AT* o = out + (size_t)row * d + i;
+        put<AT>(o, g.x * (v.x / r)); put<AT>(o + 1, g.y * (v.y / r)); put<AT>(o + 2, g.z * (v.z / r)); put<AT>(o + 3, g.w * (v.w / r));
+    }
 }
 
 // Per (head, row): per-head RMSNorm of q and k (inference.cu:52-81, 97-111), RoPE on adjacent pairs at the
