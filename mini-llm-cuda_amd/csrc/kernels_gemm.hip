@@ -171,8 +171,8 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 }
 
 // ----------------------------------------------------------------------------
-// Large-tile variant for long M (prefill): 256 x 256 output tile per workgroup, each of the 2 x 2
-// waves owning 128 x 128 (sixteen 32x32 accumulators).  K slices of 128 bytes per row go from global
+// Large-tile variant for long M (prefill): 256 x 256 output tile per 512-thread workgroup, each of the
+// 2 x 4 waves owning 128 x 64 (eight 32x32 accumulators).  K slices of 128 bytes per row go from global
 // memory straight into LDS (no register staging), two stages deep: the loads of slice s+1 are in
 // flight while slice s is multiplied, and one barrier per slice separates the stages.
 //
@@ -184,12 +184,15 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 #define GB_T 256
 #define GB_STAGE (2 * GB_T * GKB) // bytes per stage: A rows then B rows
 
+#define GB_THREADS 512 // 8 waves: 2 along M x 4 along N, each 128 x 64 (two waves per SIMD keep LDS and MFMA busy in turn)
+#define GB_BN 2        // 32-wide column blocks per wave
+
 template <typename T, int EPI>
-__global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
-                                                          void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN, float alpha) {
+__global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
+                                                            void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN, float alpha) {
     extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave >> 2, wn = wave & 3;
     int tm, tn;
     gemm_tile_of(blockIdx.x, tilesM, tilesN, tm, tn);
     if (tm < 0) return;
@@ -197,35 +200,35 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
     const int nslices = (int)(((size_t)K * sizeof(T)) / GKB);
     const size_t ldaB = (size_t)lda * sizeof(T), ldbB = (size_t)ldb * sizeof(T);
 
-    // this wave fills rows [64 wave, 64 wave + 64) of A and of B, eight rows per load instruction
-    const unsigned char* srcA[8];
-    const unsigned char* srcB[8];
+    // this wave fills rows [32 wave, 32 wave + 32) of A and of B, eight rows per load instruction
+    const unsigned char* srcA[4];
+    const unsigned char* srcB[4];
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        const int r = wave * 64 + q * 8 + (lane >> 3);
+    for (int q = 0; q < 4; q++) {
+        const int r = wave * 32 + q * 8 + (lane >> 3);
         const int pc = (lane & 7) ^ (r & 7);
         srcA[q] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(m0 + r, M - 1) * ldaB + pc * 16;
         srcB[q] = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + r, N - 1) * ldbB + pc * 16;
     }
     auto issue = [&](int s, int stage) {
-        unsigned char* dst = gsm + stage * GB_STAGE + wave * 64 * GKB;
+        unsigned char* dst = gsm + stage * GB_STAGE + wave * 32 * GKB;
 #pragma unroll
-        for (int q = 0; q < 8; q++) {
+        for (int q = 0; q < 4; q++) {
             __builtin_amdgcn_global_load_lds(srcA[q] + (size_t)s * GKB, dst + q * 8 * GKB, 16, 0, 0);
             __builtin_amdgcn_global_load_lds(srcB[q] + (size_t)s * GKB, dst + GB_T * GKB + q * 8 * GKB, 16, 0, 0);
         }
     };
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][GB_BN];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = (f32x16)(0.f);
+        for (int j = 0; j < GB_BN; j++) acc[i][j] = (f32x16)(0.f);
 
     const int half = lane >> 5, lrow = lane & 31;
-    // row offsets and swizzle keys of this lane's operand rows: rows wm*128 + 32 b + lrow; row & 7 does not depend on b
-    const int keyA = (wm * 128 + lrow) & 7, keyB = (wn * 128 + lrow) & 7;
-    const int offA = (wm * 128 + lrow) * GKB, offB = GB_T * GKB + (wn * 128 + lrow) * GKB;
+    // row offsets and swizzle keys of this lane's operand rows (row & 7 does not depend on the 32-row block)
+    const int keyA = (wm * 128 + lrow) & 7, keyB = (wn * 32 * GB_BN + lrow) & 7;
+    const int offA = (wm * 128 + lrow) * GKB, offB = GB_T * GKB + (wn * 32 * GB_BN + lrow) * GKB;
 
     issue(0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -235,14 +238,13 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
         if (s + 1 < nslices) issue(s + 1, stage ^ 1);
         const unsigned char* base = gsm + stage * GB_STAGE;
         // operand fragments one 16-wide step ahead of the MFMAs that use them
-        u32x4 fa[2][4], fb[2][4];
+        u32x4 fa[2][4], fb[2][GB_BN];
         auto frags = [&](int jj, int buf) {
             const int pa = ((2 * jj + half) ^ keyA) * 16, pb = ((2 * jj + half) ^ keyB) * 16;
 #pragma unroll
-            for (int b = 0; b < 4; b++) {
-                fa[buf][b] = *reinterpret_cast<const u32x4*>(base + offA + b * 32 * GKB + pa);
-                fb[buf][b] = *reinterpret_cast<const u32x4*>(base + offB + b * 32 * GKB + pb);
-            }
+            for (int b = 0; b < 4; b++) fa[buf][b] = *reinterpret_cast<const u32x4*>(base + offA + b * 32 * GKB + pa);
+#pragma unroll
+            for (int b = 0; b < GB_BN; b++) fb[buf][b] = *reinterpret_cast<const u32x4*>(base + offB + b * 32 * GKB + pb);
         };
         frags(0, 0);
 #pragma unroll
@@ -254,14 +256,14 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
 #pragma unroll
             for (int bm = 0; bm < 2; bm++)
 #pragma unroll
-                for (int bn = 0; bn < 4; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
+                for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
             __builtin_amdgcn_sched_barrier(0);
             if (jj < 3) frags(jj + 1, (jj + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int bm = 2; bm < 4; bm++)
 #pragma unroll
-                for (int bn = 0; bn < 4; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
+                for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
         }
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // slice s+1 has landed
@@ -271,8 +273,8 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn_big(const T* __restrict__ 
 #pragma unroll
     for (int bm = 0; bm < 4; bm++)
 #pragma unroll
-        for (int bn = 0; bn < 4; bn++) {
-            const int col = n0 + wn * 128 + bn * 32 + lrow;
+        for (int bn = 0; bn < GB_BN; bn++) {
+            const int col = n0 + wn * 32 * GB_BN + bn * 32 + lrow;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
                 const int row = m0 + wm * 128 + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
@@ -302,9 +304,9 @@ static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, in
         attr = true;
     }
     if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
+        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GB_THREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
     else
-        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_PLAIN>), dim3(grid), dim3(GTHREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
+        hipLaunchKernelGGL((k_gemm_tn_big<T, GEMM_EPI_PLAIN>), dim3(grid), dim3(GB_THREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
     return hipGetLastError();
 }
 
