@@ -420,21 +420,30 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
 // Gated-delta-net prefill.  The rows of a head's state evolve independently of each other
 //   S[r,:] <- alpha S[r,:] + beta (v_r - alpha u_r) k^T,  u_r = S[r,:].k,   o_r = S_new[r,:].q
 // (the decode kernel's update, regrouped; k, q L2-normalised), so one workgroup carries PF_GR rows of
-// one head of one segment in registers across the whole segment: 8 lanes per row, each with DK/8
-// columns.  Sixteen tokens of q, k, v and gate inputs are staged in LDS at a time, the next sixteen
+// one head of one segment in registers across the whole segment: 4 lanes per row, each with DK/4
+// columns.  The decay is kept out of the element loop: the registers hold S / a for a running scalar a
+// (the product of the alphas since the last renormalisation), so a token costs three FMAs per element
+// -- S.k, S.q and the rank-1 update -- instead of four.  Sixteen tokens of q, k, v and gate inputs are staged in LDS at a time, the next sixteen
 // being loaded into registers meanwhile.  With p = S_old[r,:].q the read-out needs no second pass:
 // o_r = (alpha p + w (k.q)) / |q|,  w = beta (v_r - alpha u_r) / |k|.
 #define PF_GC 16
-#define PF_GR 32
+#define PF_GR 64
+// Workgroup barrier that orders LDS traffic only: __syncthreads() also waits for every outstanding global
+// load (loads and stores share one counter), which would put the next chunk's prefetch on the critical path.
+__device__ __forceinline__ void pf_lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+template <int CTRL> __device__ __forceinline__ float quad_swap(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
 template <int DK, typename AT>
 __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
     constexpr int DV = DK, TPR = PWG / PF_GR, CPT = DK / TPR;
+    static_assert(TPR == 4, "the row sum below is a quad reduction");
     constexpr int NQK = PF_GC * DK / 4 / PWG; // f32x4 loads per thread for each of q and k
     __shared__ __attribute__((aligned(16))) float qs[PF_GC][DK];
     __shared__ __attribute__((aligned(16))) float ks[PF_GC][DK];
     __shared__ float vs[PF_GC][PF_GR];
     __shared__ float zs[PF_GC][2];
-    __shared__ float gate[PF_GC][5]; // alpha, beta, 1/|q|, 1/|k|, k.q
+    __shared__ float gate[PF_GC][6]; // alpha, beta, 1/|q|, 1/|k|, k.q, 1/alpha
     const StepArgs& a = P.a;
     const int h = blockIdx.x, seg = blockIdx.y, r0 = blockIdx.z * PF_GR, tid = threadIdx.x;
     const int seq = P.segSeq[seg], len = P.segLen[seg], row0 = P.segStart[seg];
@@ -446,8 +455,9 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(Srow + c);
         S[c] = v.x; S[c + 1] = v.y; S[c + 2] = v.z; S[c + 3] = v.w;
     }
+    float ascale = 1.0f, ainv = 1.0f; // S (true state) = ascale * S[] (registers); ainv = 1 / ascale
     f32x4 qreg[NQK], kreg[NQK];
-    float vreg[2], zreg = 0.f;
+    float vreg[PF_GC * PF_GR / PWG], zreg = 0.f;
     auto fetch = [&](int t0) {
         const int last = len - 1 - t0; // >= 0
 #pragma unroll
@@ -458,7 +468,7 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
             kreg[it] = *reinterpret_cast<const f32x4*>(qkv + L.offK + h * DK + e4);
         }
 #pragma unroll
-        for (int it = 0; it < 2; it++) {
+        for (int it = 0; it < PF_GC * PF_GR / PWG; it++) {
             const int i = it * PWG + tid, c = i / PF_GR, e = i % PF_GR;
             vreg[it] = P.QKV[(size_t)(row0 + t0 + min(c, last)) * P.qkvLd + L.offV + h * DV + r0 + e];
         }
@@ -470,7 +480,7 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
     fetch(0);
     for (int t0 = 0; t0 < len; t0 += PF_GC) {
         const int nt = min(PF_GC, len - t0);
-        __syncthreads(); // the previous chunk has been consumed
+        pf_lds_barrier(); // the previous chunk has been consumed
 #pragma unroll
         for (int it = 0; it < NQK; it++) {
             const int i = it * PWG + tid, c = i / (DK / 4), e4 = (i % (DK / 4)) * 4;
@@ -478,12 +488,12 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
             *reinterpret_cast<f32x4*>(&ks[c][e4]) = kreg[it];
         }
 #pragma unroll
-        for (int it = 0; it < 2; it++) {
+        for (int it = 0; it < PF_GC * PF_GR / PWG; it++) {
             const int i = it * PWG + tid;
             vs[i / PF_GR][i % PF_GR] = vreg[it];
         }
         if (tid < 2 * PF_GC) zs[tid >> 1][tid & 1] = zreg;
-        __syncthreads();
+        pf_lds_barrier();
         if (t0 + PF_GC < len) fetch(t0 + PF_GC); // in flight during this chunk's arithmetic
         { // per token: |q|, |k|, k.q and the gates -- 16 threads per token
             const int c = tid >> 4, sub = tid & 15;
@@ -497,34 +507,48 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
             if (sub == 0) {
                 const float za = zs[c][0] + L.gdnBa[h], zb = zs[c][1] + L.gdnBb[h];
                 const float rq = 1.0f / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
-                gate[c][0] = expf(-(fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
+                const float sp = fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)));
+                gate[c][0] = expf(-sp);
+                gate[c][5] = expf(sp);
                 gate[c][1] = pf_sigmoid(zb);
                 gate[c][2] = rq; gate[c][3] = rk; gate[c][4] = kq * rq * rk; // k.q of the normalised vectors
             }
         }
-        __syncthreads();
+        pf_lds_barrier();
+#pragma unroll 4
         for (int c = 0; c < nt; c++) {
             const float alpha = gate[c][0], beta = gate[c][1], rq = gate[c][2], rk = gate[c][3], kqn = gate[c][4];
             float kk[CPT];
-            float u = 0.f, p = 0.f;
+            float ua[4] = {0.f, 0.f, 0.f, 0.f}, pa[4] = {0.f, 0.f, 0.f, 0.f}; // four independent chains each
 #pragma unroll
             for (int e = 0; e < CPT; e += 4) {
                 const f32x4 k4 = *reinterpret_cast<const f32x4*>(&ks[c][c0 + e]);
                 const f32x4 q4 = *reinterpret_cast<const f32x4*>(&qs[c][c0 + e]);
                 kk[e] = k4.x; kk[e + 1] = k4.y; kk[e + 2] = k4.z; kk[e + 3] = k4.w;
-                u = fmaf(S[e], k4.x, u); u = fmaf(S[e + 1], k4.y, u); u = fmaf(S[e + 2], k4.z, u); u = fmaf(S[e + 3], k4.w, u);
-                p = fmaf(S[e], q4.x, p); p = fmaf(S[e + 1], q4.y, p); p = fmaf(S[e + 2], q4.z, p); p = fmaf(S[e + 3], q4.w, p);
+                ua[0] = fmaf(S[e], k4.x, ua[0]); ua[1] = fmaf(S[e + 1], k4.y, ua[1]); ua[2] = fmaf(S[e + 2], k4.z, ua[2]); ua[3] = fmaf(S[e + 3], k4.w, ua[3]);
+                pa[0] = fmaf(S[e], q4.x, pa[0]); pa[1] = fmaf(S[e + 1], q4.y, pa[1]); pa[2] = fmaf(S[e + 2], q4.z, pa[2]); pa[3] = fmaf(S[e + 3], q4.w, pa[3]);
             }
-#pragma unroll
-            for (int o = TPR / 2; o > 0; o >>= 1) { u += __shfl_xor(u, o, 64); p += __shfl_xor(p, o, 64); }
-            u *= rk; p *= rq;                                  // against the normalised k and q
+            float u = (ua[0] + ua[1]) + (ua[2] + ua[3]), p = (pa[0] + pa[1]) + (pa[2] + pa[3]);
+            // sum over the 4 lanes of a row: quad permutes in the VALU (a cross-lane shuffle through LDS costs
+            // ~100 cycles each, and this is the serial path from one token to the next)
+            u += quad_swap<0xB1>(u); p += quad_swap<0xB1>(p);   // lanes 0<->1, 2<->3
+            u += quad_swap<0x4E>(u); p += quad_swap<0x4E>(p);   // lanes 0<->2, 1<->3
+            u *= rk * ascale; p *= rq * ascale;                // against the normalised k and q, with the decay put back
             const float wn = beta * (vs[c][r] - alpha * u);    // coefficient of the normalised k
-            const float w = wn * rk;
+            ascale *= alpha; ainv *= gate[c][5];               // gate[c][5] = 1 / alpha
+            if (ascale < 1.0e-12f) {                           // workgroup-uniform (one head): fold the decay into the registers
 #pragma unroll
-            for (int e = 0; e < CPT; e++) S[e] = fmaf(w, kk[e], alpha * S[e]);
+                for (int e = 0; e < CPT; e++) S[e] *= ascale;
+                ascale = 1.0f; ainv = 1.0f;
+            }
+            const float w = wn * rk * ainv;
+#pragma unroll
+            for (int e = 0; e < CPT; e++) S[e] = fmaf(w, kk[e], S[e]);
             if (cg == 0) put<AT>((AT*)P.Amix + (size_t)(row0 + t0 + c) * P.aLd + h * DV + r0 + r, alpha * p + wn * kqn);
         }
     }
+#pragma unroll
+    for (int e = 0; e < CPT; e++) S[e] *= ascale;
 #pragma unroll
     for (int c = 0; c < CPT; c += 4) {
         f32x4 v; v.x = S[c]; v.y = S[c + 1]; v.z = S[c + 2]; v.w = S[c + 3];
