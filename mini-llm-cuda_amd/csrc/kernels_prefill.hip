@@ -435,7 +435,7 @@ template <int CTRL> __device__ __forceinline__ float quad_swap(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
 }
 template <int DK, typename AT>
-__global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
+__global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L, int skipFrom) {
     constexpr int DV = DK, TPR = PWG / PF_GR, CPT = DK / TPR;
     static_assert(TPR == 4, "the row sum below is a quad reduction");
     constexpr int NQK = PF_GC * DK / 4 / PWG; // f32x4 loads per thread for each of q and k
@@ -447,6 +447,7 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
     const StepArgs& a = P.a;
     const int h = blockIdx.x, seg = blockIdx.y, r0 = blockIdx.z * PF_GR, tid = threadIdx.x;
     const int seq = P.segSeq[seg], len = P.segLen[seg], row0 = P.segStart[seg];
+    if (len >= skipFrom) return; // taken by the chunk-parallel kernels
     const int r = tid / TPR, cg = tid % TPR, c0 = cg * CPT;
     float* Srow = L.S + (((size_t)seq * a.gdnHeads + h) * DV + r0 + r) * DK + c0;
     float S[CPT];
@@ -554,6 +555,324 @@ __global__ void __launch_bounds__(PWG) k_pf_gdn(PfArgs P, LayerDev L) {
         f32x4 v; v.x = S[c]; v.y = S[c + 1]; v.z = S[c + 2]; v.w = S[c + 3];
         *reinterpret_cast<f32x4*>(Srow + c) = v;
     }
+}
+
+// ----------------------------------------------------------------------------
+// Chunk-parallel gated-delta-net prefill on the MFMA units (bf16 models, segments of 64 tokens or more).
+//
+// Over a chunk of C = 64 tokens starting from state S0, with g_t = sum_{j<=t} log(alpha_j):
+//   S_t = e^{g_t} S0 + sum_{i<=t} e^{g_t - g_i} w_i k_i^T,      w_t = beta_t (v_t - alpha_t S_{t-1} k_t)
+// (k, q L2-normalised).  Substituting S_{t-1} gives a unit-lower-triangular system for the w_t:
+//   (I + A) W^T = beta (.) V - diag(beta e^{g}) K S0^T,   A[t,i] = beta_t e^{g_t - g_i} (k_i . k_t), i < t
+// so W^T = Vt - Kt S0^T with Vt = (I+A)^{-1} (beta (.) V) and Kt = (I+A)^{-1} diag(beta e^{g}) K, both free
+// of S0.  The outputs and the next state are then plain products:
+//   O   = diag(e^{g}) Q S0^T + M W^T,      M[t,i] = e^{g_t - g_i} (k_i . q_t), i <= t
+//   S_C = e^{g_C} S0 + W Kh,               Kh[i,:] = e^{g_C - g_i} k_i
+// k_gdn_prep builds Vt, Kt, diag(e^g) Q, M, Kh for every chunk of every head in parallel (forward
+// substitution, 64 steps, one column per thread); k_gdn_scan walks the chunks of one head of one
+// segment in order with the state -- transposed, S^T[dk, dv] -- in MFMA accumulators, 56 MFMAs per
+// chunk and wave.  Operands are IEEE half, accumulation and the state fp32.  Every contraction index
+// (dk in Kt S0^T and Q S0^T, the chunk's token index in M W^T and Kh^T W^T) is stored in the order
+// the accumulator layout holds it (slot_of below), so S0^T and W^T are used as MFMA B operands straight
+// from the accumulator registers, without a transpose through LDS.
+// ----------------------------------------------------------------------------
+#define GD_C 64
+// accumulator element i of lane (n, half) of a 32x32 tile is row 8(i/4) + 4 half + i%4; a 16-wide MFMA step
+// st takes elements 8 st .. 8 st + 7 of both halves.  slot_of(x) = position of row x of a (multi-tile)
+// contraction axis in that order: tile x/32, then step, half, element.
+__host__ __device__ __forceinline__ int slot_of(int x) {
+    const int x32 = x & 31;
+    const int i = 4 * (x32 >> 3) + (x32 & 3), hh = (x32 >> 2) & 1;
+    return (x & ~31) + 16 * (i >> 3) + 8 * hh + (i & 7);
+}
+template <int DK> struct GdLayout { // one chunk's operand image (bytes), rows padded by 16 bytes against LDS bank conflicts
+    static constexpr int KP = (DK + 8) * 2, TP = (GD_C + 8) * 2; // row pitches of [*, DK] and [*, 64] half matrices
+    static constexpr int oKt = 0, oQh = oKt + GD_C * KP, oM = oQh + GD_C * KP, oKhT = oM + GD_C * TP;
+    static constexpr int image = oKhT + DK * TP;                  // 62464 (DK 128), 36864 (DK 64): multiples of 1024
+    static constexpr int oVt = image;                             // fp32 [64, DV], read straight from global
+    static constexpr int total = image + GD_C * DK * 4;
+};
+__device__ __forceinline__ uint16_t f16_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
+
+template <int DK>
+__global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const int* __restrict__ chunkSeg, const int* __restrict__ chunkT0,
+                                                      unsigned char* __restrict__ ws, float* __restrict__ gCexp) {
+    constexpr int DV = DK, NT = 2 * DK;
+    typedef GdLayout<DK> Lay;
+    extern __shared__ __attribute__((aligned(16))) unsigned char pls[];
+    float* Am = reinterpret_cast<float*>(pls);            // [64][64]
+    float* gs = Am + GD_C * GD_C;                         // g[64], beta[64], sp[64], 1/|k|[64], 1/|q|[64], partial sums [4][64]
+    uint16_t* k16 = reinterpret_cast<uint16_t*>(gs + 9 * GD_C); // [64][DK + 8] normalised k, half
+    uint16_t* q16 = k16 + GD_C * (DK + 8);
+    const StepArgs& a = P.a;
+    const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int seg = chunkSeg[chunk], t0 = chunkT0[chunk];
+    const int nv = min(GD_C, P.segLen[seg] - t0), row0 = P.segStart[seg] + t0;
+    unsigned char* img = ws + ((size_t)chunk * a.gdnHeads + h) * Lay::total;
+    float* g = gs; float* beta = gs + GD_C; float* sp = gs + 2 * GD_C; float* rk = gs + 3 * GD_C; float* rq = gs + 4 * GD_C;
+    float* part = gs + 5 * GD_C;
+
+    // Thread (sel, cidx) keeps column cidx of q (sel 0: threads [0, DK)) or k (sel 1: threads [DK, 2 DK)) for the 64
+    // tokens of the chunk in registers (tokens past the segment end: zero).
+    const int sel = tid / DK, cidx = tid % DK;
+    float colv[GD_C];
+    {
+        const float* src = P.QKV + (size_t)row0 * P.qkvLd + (sel ? L.offK : 0) + h * DK + cidx;
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) colv[t] = t < nv ? src[(size_t)t * P.qkvLd] : 0.f;
+    }
+    if (tid < GD_C) { // gates
+        const int t = tid;
+        float s_ = 0.f, b_ = 0.f;
+        if (t < nv) {
+            const float* qkv = P.QKV + (size_t)(row0 + t) * P.qkvLd;
+            const float za = qkv[L.offGa + h] + L.gdnBa[h], zb = qkv[L.offGb + h] + L.gdnBb[h];
+            s_ = fmaxf(za, 0.f) + log1pf(expf(-fabsf(za))); // -log(alpha)
+            b_ = pf_sigmoid(zb);
+        }
+        sp[t] = s_; beta[t] = b_;
+        float v = -s_; // inclusive prefix sum over the 64 tokens (one wave)
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { const float u = __shfl_up(v, o, 64); if (tid >= o) v += u; }
+        g[t] = v;
+    }
+    { // squared norms per token: reduce-scatter over the 64 lanes of a wave (lane t ends up with token t), then over waves
+        float r[GD_C];
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) r[t] = colv[t] * colv[t];
+#pragma unroll
+        for (int o = 32, n = 32; o > 0; o >>= 1, n >>= 1) {
+            const bool up = (lane & o) != 0;
+#pragma unroll
+            for (int i = 0; i < n; i++) {
+                const float keep = up ? r[i + n] : r[i], send = up ? r[i] : r[i + n];
+                r[i] = keep + __shfl_xor(send, o, 64);
+            }
+        }
+        part[wave * GD_C + lane] = r[0];
+    }
+    __syncthreads();
+    if (tid < 2 * GD_C) { // 1 / norm of q (threads 0..63) and k (64..127)
+        const int t = tid & 63, m = tid >> 6; // m 0: q, 1: k
+        constexpr int WPM = DK / 64;          // waves per matrix
+        float ss = 0.f;
+#pragma unroll
+        for (int w = 0; w < WPM; w++) ss += part[(m * WPM + w) * GD_C + t];
+        (m ? rk : rq)[t] = 1.0f / sqrtf(ss + 1e-6f);
+    }
+    __syncthreads();
+    { // normalise the register column, publish the half copy for the MFMAs
+        const float* rr = sel ? rk : rq;
+        uint16_t* d16 = sel ? k16 : q16;
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) {
+            colv[t] *= rr[t];
+            d16[t * (DK + 8) + cidx] = f16_bits(colv[t]);
+        }
+    }
+    __syncthreads();
+    { // K K^T and Q K^T on the MFMA units: 2 x 2 tiles each
+        const int n32 = lane & 31, half = lane >> 5;
+        for (int tix = wave; tix < 8; tix += NT / 64) {
+            const int which = tix >> 2, tt = (tix >> 1) & 1, ti = tix & 1;
+            const uint16_t* Aop = (which ? q16 : k16) + (32 * tt + n32) * (DK + 8) + 8 * half;
+            const uint16_t* Bop = k16 + (32 * ti + n32) * (DK + 8) + 8 * half;
+            f32x16 acc;
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[i] = 0.f;
+#pragma unroll
+            for (int s_ = 0; s_ < DK / 16; s_++)
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(Aop + 16 * s_)),
+                                                             __builtin_bit_cast(f16x8, *reinterpret_cast<const u32x4*>(Bop + 16 * s_)), acc, 0, 0, 0);
+            const int i_ = 32 * ti + n32;
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                const int t = 32 * tt + 8 * (e >> 2) + 4 * half + (e & 3);
+                const float dec = expf(g[t] - g[i_]); // <= 1 where it is used (i <= t)
+                if (which == 0) Am[t * GD_C + i_] = i_ < t ? beta[t] * dec * acc[e] : 0.f;
+                else *reinterpret_cast<uint16_t*>(img + Lay::oM + t * Lay::TP + 2 * slot_of(i_)) = f16_bits(i_ <= t ? dec * acc[e] : 0.f);
+            }
+        }
+    }
+    __syncthreads();
+    // forward substitution, one column per thread: threads [0, DV) solve beta (.) V, threads [DV, 2 DV) -- the ones
+    // that hold the k columns -- solve diag(beta e^g) K
+    float X[GD_C];
+    const int col = cidx;
+    if (tid < DV) {
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) X[t] = t < nv ? beta[t] * P.QKV[(size_t)(row0 + t) * P.qkvLd + L.offV + h * DV + col] : 0.f;
+    } else {
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) X[t] = beta[t] * expf(g[t]) * colv[t];
+    }
+#pragma unroll
+    for (int t = 1; t < GD_C; t++) {
+        float acc0 = X[t], acc1 = 0.f, acc2 = 0.f, acc3 = 0.f; // four chains: the row's dot product is on the serial path
+#pragma unroll
+        for (int i4 = 0; i4 < t; i4 += 4) {
+            const f32x4 a4 = *reinterpret_cast<const f32x4*>(Am + t * GD_C + i4); // zero at and beyond the diagonal
+            acc0 = fmaf(-a4.x, X[i4], acc0);
+            if (i4 + 1 < t) acc1 = fmaf(-a4.y, X[i4 + 1], acc1);
+            if (i4 + 2 < t) acc2 = fmaf(-a4.z, X[i4 + 2], acc2);
+            if (i4 + 3 < t) acc3 = fmaf(-a4.w, X[i4 + 3], acc3);
+        }
+        X[t] = (acc0 + acc1) + (acc2 + acc3);
+    }
+    const float gC = g[GD_C - 1];
+    const int sl = slot_of(col);
+    // Kt, diag(e^g) Q and Kh^T are assembled in LDS in the image layout (the half copies of k and q are no longer
+    // needed: the MFMAs are done) and leave as 16-byte rows; element-wise 2-byte stores to global would touch a
+    // different cache line per lane.
+    uint16_t* khs = q16 + GD_C * (DK + 8); // [DK][64 + 8]
+    if (tid < DV) { // holds the q column
+        float* Vt = reinterpret_cast<float*>(img + Lay::oVt);
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) {
+            Vt[t * DV + col] = X[t];
+            q16[t * (DK + 8) + sl] = f16_bits(expf(g[t]) * colv[t]);
+        }
+    } else { // holds the k column
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) {
+            k16[t * (DK + 8) + sl] = f16_bits(X[t]);
+            khs[col * (GD_C + 8) + slot_of(t)] = f16_bits(expf(gC - g[t]) * colv[t]); // token axis in slot order
+        }
+    }
+    __syncthreads();
+    {
+        const u32x4* s1 = reinterpret_cast<const u32x4*>(k16);
+        u32x4* d1 = reinterpret_cast<u32x4*>(img + Lay::oKt);
+        for (int i = tid; i < 2 * GD_C * Lay::KP / 16; i += NT) d1[i] = s1[i];
+        const u32x4* s2 = reinterpret_cast<const u32x4*>(khs);
+        u32x4* d2 = reinterpret_cast<u32x4*>(img + Lay::oKhT);
+        for (int i = tid; i < DK * Lay::TP / 16; i += NT) d2[i] = s2[i];
+    }
+    if (tid == 0) gCexp[(size_t)chunk * a.gdnHeads + h] = expf(gC);
+}
+
+// Copies one chunk's operand image (IMG bytes, a multiple of 1 KB) from global memory straight into LDS, 1 KB per
+// instruction, the NW waves of the workgroup taking instructions in turn.
+template <int IMG, int NW>
+__device__ __forceinline__ void gd_issue_image(const unsigned char* src, unsigned char* dst, int wave, int lane) {
+    for (int q = wave; q < IMG / 1024; q += NW) __builtin_amdgcn_global_load_lds(src + q * 1024 + lane * 16, dst + q * 1024, 16, 0, 0);
+}
+
+template <int DK>
+__global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const int* __restrict__ chunkBase, const unsigned char* __restrict__ ws,
+                                                      const float* __restrict__ gCexp) {
+    constexpr int DV = DK, NW = DV / 32, JT = DK / 32; // waves (one per 32 state columns dv), dk tiles
+    typedef GdLayout<DK> Lay;
+    extern __shared__ __attribute__((aligned(16))) unsigned char sls[]; // two operand images
+    const StepArgs& a = P.a;
+    const int h = blockIdx.x, seg = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int len = P.segLen[seg];
+    if (len < GD_C) return; // short segments take the recurrent kernel
+    const int seq = P.segSeq[seg], row0 = P.segStart[seg], nch = (len + GD_C - 1) / GD_C, cb = chunkBase[seg];
+    const int n32 = lane & 31, half = lane >> 5, dv = 32 * wave + n32;
+    float* Sg = L.S + ((size_t)seq * a.gdnHeads + h) * DV * DK;
+    f32x16 St[JT]; // S^T tile j: rows dk = 32 j + 8(i/4) + 4 half + i%4, column dv
+#pragma unroll
+    for (int j = 0; j < JT; j++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) St[j][i] = Sg[(size_t)dv * DK + 32 * j + 8 * (i >> 2) + 4 * half + (i & 3)];
+    auto image_of = [&](int c) { return ws + ((size_t)(cb + c) * a.gdnHeads + h) * Lay::total; };
+    auto issue = [&](int c, int stage) { gd_issue_image<Lay::image, NW>(image_of(c), sls + stage * Lay::image, wave, lane); };
+    f32x16 Vt[2];
+    auto load_vt = [&](int c) {
+        const float* v = reinterpret_cast<const float*>(image_of(c) + Lay::oVt);
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) Vt[tt][i] = v[(32 * tt + 8 * (i >> 2) + 4 * half + (i & 3)) * DV + dv];
+    };
+    issue(0, 0);
+    load_vt(0);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    for (int c = 0; c < nch; c++) {
+        const unsigned char* im = sls + (c & 1) * Lay::image;
+        if (c + 1 < nch) issue(c + 1, (c + 1) & 1);
+        const float gC = gCexp[(size_t)(cb + c) * a.gdnHeads + h];
+        // S0^T as B operands: step (j, st) = elements 8 st .. 8 st + 7 of tile j, rounded to half
+        u32x4 sop[JT][2];
+#pragma unroll
+        for (int j = 0; j < JT; j++)
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+                sop[j][st].x = pack_f16(St[j][8 * st + 0], St[j][8 * st + 1]); sop[j][st].y = pack_f16(St[j][8 * st + 2], St[j][8 * st + 3]);
+                sop[j][st].z = pack_f16(St[j][8 * st + 4], St[j][8 * st + 5]); sop[j][st].w = pack_f16(St[j][8 * st + 6], St[j][8 * st + 7]);
+            }
+        // X = Kt S0^T, Y = diag(e^g) Q S0^T : [64 tokens, 32 dv]
+        f32x16 X[2], Y[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) { X[tt][i] = 0.f; Y[tt][i] = 0.f; }
+            const unsigned char* kr = im + Lay::oKt + (32 * tt + n32) * Lay::KP + 16 * half;
+            const unsigned char* qr = im + Lay::oQh + (32 * tt + n32) * Lay::KP + 16 * half;
+#pragma unroll
+            for (int j = 0; j < JT; j++)
+#pragma unroll
+                for (int st = 0; st < 2; st++) {
+                    const u32x4 ka = *reinterpret_cast<const u32x4*>(kr + 32 * (2 * j + st));
+                    const u32x4 qa = *reinterpret_cast<const u32x4*>(qr + 32 * (2 * j + st));
+                    X[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ka), __builtin_bit_cast(f16x8, sop[j][st]), X[tt], 0, 0, 0);
+                    Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, qa), __builtin_bit_cast(f16x8, sop[j][st]), Y[tt], 0, 0, 0);
+                }
+        }
+        // W^T = Vt - X, as B operands (token axis in slot order by construction)
+        u32x4 wop[2][2];
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++)
+#pragma unroll
+            for (int st = 0; st < 2; st++) {
+                float w[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) w[e] = Vt[tt][8 * st + e] - X[tt][8 * st + e];
+                wop[tt][st].x = pack_f16(w[0], w[1]); wop[tt][st].y = pack_f16(w[2], w[3]);
+                wop[tt][st].z = pack_f16(w[4], w[5]); wop[tt][st].w = pack_f16(w[6], w[7]);
+            }
+        if (c + 1 < nch) load_vt(c + 1); // Vt of this chunk has been consumed
+        // O = Y + M W^T (M is lower triangular: tokens of tile 0 see only tile 0)
+#pragma unroll
+        for (int tt = 0; tt < 2; tt++) {
+            const unsigned char* mr = im + Lay::oM + (32 * tt + n32) * Lay::TP + 16 * half;
+#pragma unroll
+            for (int t2 = 0; t2 <= tt; t2++)
+#pragma unroll
+                for (int st = 0; st < 2; st++) {
+                    const u32x4 ma = *reinterpret_cast<const u32x4*>(mr + 32 * (2 * t2 + st));
+                    Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ma), __builtin_bit_cast(f16x8, wop[t2][st]), Y[tt], 0, 0, 0);
+                }
+            const int nvalid = len - (c * GD_C + 32 * tt);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int tk = 8 * (i >> 2) + 4 * half + (i & 3);
+                if (tk < nvalid) put<f16_t>((f16_t*)P.Amix + (size_t)(row0 + c * GD_C + 32 * tt + tk) * P.aLd + h * DV + dv, Y[tt][i]);
+            }
+        }
+        // S^T <- e^{g_C} S^T + Kh^T W^T
+#pragma unroll
+        for (int j = 0; j < JT; j++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) St[j][i] *= gC;
+            const unsigned char* hr = im + Lay::oKhT + (32 * j + n32) * Lay::TP + 16 * half;
+#pragma unroll
+            for (int t2 = 0; t2 < 2; t2++)
+#pragma unroll
+                for (int st = 0; st < 2; st++) {
+                    const u32x4 ha = *reinterpret_cast<const u32x4*>(hr + 32 * (2 * t2 + st));
+                    St[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ha), __builtin_bit_cast(f16x8, wop[t2][st]), St[j], 0, 0, 0);
+                }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the next chunk's image (and Vt) has landed
+        __syncthreads();                                  // ... for every wave; everyone is done with this image
+    }
+#pragma unroll
+    for (int j = 0; j < JT; j++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) Sg[(size_t)dv * DK + 32 * j + 8 * (i >> 2) + 4 * half + (i & 3)] = St[j][i];
 }
 
 // e[row][j] = silu(ple gate output) * P[tok][j]
@@ -729,7 +1048,13 @@ int mlh_build_gemm_operands(mlh_ctx* c) {
 }
 
 // The headDim-128 attention tiles exceed the 64 KB a launch may use without opting in.
+static size_t gdn_prep_lds(int dk) { return ((size_t)GD_C * GD_C + 9 * GD_C) * 4 + (size_t)2 * GD_C * (dk + 8) * 2 + (size_t)dk * (GD_C + 8) * 2; }
+
 int mlh_init_prefill_kernels(mlh_ctx* c) {
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gdn_prep<64>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)gdn_prep_lds(64)));
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gdn_prep<128>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)gdn_prep_lds(128)));
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gdn_scan<64>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GdLayout<64>::image));
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gdn_scan<128>), hipFuncAttributeMaxDynamicSharedMemorySize, 2 * GdLayout<128>::image));
     const int lds = (2 * 64 * 132 + PF_QB * 128) * 4;
     MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_pf_attn<128, float>), hipFuncAttributeMaxDynamicSharedMemorySize, lds));
     return 0;
@@ -751,15 +1076,16 @@ static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
         return 0;
     };
     int rc;
-    const int nblk = cdiv(rows, PF_QB) + hp.maxSeqs;
+    const int nblk = cdiv(rows, PF_QB) + hp.maxSeqs, nchunk = cdiv(rows, GD_C) + hp.maxSeqs;
     if ((rc = alloc((void**)&c->pfX, n * hp.dim * 4)) || (rc = alloc(&c->pfXn, n * hp.dim * wb)) ||
         (rc = alloc((void**)&c->pfQKV, n * c->maxRowsA * 4)) || (rc = alloc(&c->pfA, n * c->maxAd * wb)) ||
         (rc = alloc(&c->pfE, n * std::max(hp.pleDim, 8) * wb)) || (rc = alloc((void**)&c->pfH1, n * hp.dim * 4)) ||
         (rc = alloc(&c->pfU, n * hp.ffnDim * wb)) ||
-        (rc = alloc((void**)&c->pfMeta, (3 * n + 4 * (size_t)hp.maxSeqs + 2 * (size_t)nblk) * 4)))
+        (rc = alloc((void**)&c->pfMeta, (3 * n + 4 * (size_t)hp.maxSeqs + 2 * (size_t)nblk + 2 * (size_t)nchunk + hp.maxSeqs) * 4)))
         return rc;
     c->pfRows = rows;
     c->pfBlkCap = nblk;
+    c->pfChunkCap = nchunk;
     return 0;
 }
 
@@ -776,20 +1102,37 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     // ---- metadata ----
     const bool mfmaAttn = hp.weightDtype == MLH_DTYPE_BF16; // bf16 models: bf16 MFMA attention, 128 queries per workgroup
     const int qb = mfmaAttn ? PF_MQB : PF_QB;
-    std::vector<int> rowSeq(n), rowPos(n), segStart(nseg), segPos0(nseg), blkSeg, blkQ0;
+    std::vector<int> rowSeq(n), rowPos(n), segStart(nseg), segPos0(nseg), blkSeg, blkQ0, chunkSeg, chunkT0, chunkBase(nseg, 0);
+    bool anyGdn = false;
+    for (const LayerDev& L : c->layers) anyGdn = anyGdn || L.kind == MLH_KIND_GDN;
+    const bool gdnChunked = anyGdn && c->gemmDtype == MLH_GEMM_F16; // segments of 64 tokens or more: chunk-parallel MFMA path
     int r = 0;
     for (int s = 0; s < nseg; s++) {
         segStart[s] = r;
         segPos0[s] = c->h_len[seqs[s]];
         for (int i = 0; i < lens[s]; i++, r++) { rowSeq[r] = seqs[s]; rowPos[r] = segPos0[s] + i; }
         for (int q0 = 0; q0 < lens[s]; q0 += qb) { blkSeg.push_back(s); blkQ0.push_back(q0); }
+        chunkBase[s] = (int)chunkSeg.size();
+        if (gdnChunked && lens[s] >= GD_C)
+            for (int t0 = 0; t0 < lens[s]; t0 += GD_C) { chunkSeg.push_back(s); chunkT0.push_back(t0); }
     }
-    const int nblk = (int)blkSeg.size();
+    const int nblk = (int)blkSeg.size(), nchunk = (int)chunkSeg.size();
     if (nblk > c->pfBlkCap) { c->err = "prefill: too many attention blocks"; return -1; }
+    if (nchunk > 0) {
+        const size_t per = (size_t)hp.gdnHeads * (hp.gdnDk == 64 ? GdLayout<64>::total : GdLayout<128>::total);
+        if ((size_t)nchunk > c->pfGdnChunks) {
+            MLH_CHECK(c, hipStreamSynchronize(c->stream));
+            if (c->pfGdnWs) { (void)hipFree(c->pfGdnWs); (void)hipFree(c->pfGdnG); c->pfGdnWs = nullptr; c->pfGdnG = nullptr; c->pfGdnChunks = 0; }
+            MLH_CHECK(c, hipMalloc(&c->pfGdnWs, (size_t)nchunk * per));
+            MLH_CHECK(c, hipMalloc((void**)&c->pfGdnG, (size_t)nchunk * hp.gdnHeads * 4));
+            c->pfGdnChunks = nchunk;
+        }
+    }
     int* d = c->pfMeta;
     int* d_ids = d; int* d_rowSeq = d + n; int* d_rowPos = d + 2 * n;
     int* d_seg = d + 3 * n; // segStart, segLen, segSeq, segPos0 (maxSeqs each)
     int* d_blk = d_seg + 4 * hp.maxSeqs;
+    int* d_chunk = d_blk + 2 * c->pfBlkCap; // chunkSeg, chunkT0 (pfChunkCap each), chunkBase (maxSeqs)
     hipStream_t st = c->stream;
     MLH_CHECK(c, hipMemcpyAsync(d_ids, ids, (size_t)n * 4, hipMemcpyHostToDevice, st));
     MLH_CHECK(c, hipMemcpyAsync(d_rowSeq, rowSeq.data(), (size_t)n * 4, hipMemcpyHostToDevice, st));
@@ -800,6 +1143,12 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     MLH_CHECK(c, hipMemcpyAsync(d_seg + 3 * hp.maxSeqs, segPos0.data(), (size_t)nseg * 4, hipMemcpyHostToDevice, st));
     MLH_CHECK(c, hipMemcpyAsync(d_blk, blkSeg.data(), (size_t)nblk * 4, hipMemcpyHostToDevice, st));
     MLH_CHECK(c, hipMemcpyAsync(d_blk + c->pfBlkCap, blkQ0.data(), (size_t)nblk * 4, hipMemcpyHostToDevice, st));
+    if (nchunk > 0) {
+        if (nchunk > c->pfChunkCap) { c->err = "prefill: too many GDN chunks"; return -1; }
+        MLH_CHECK(c, hipMemcpyAsync(d_chunk, chunkSeg.data(), (size_t)nchunk * 4, hipMemcpyHostToDevice, st));
+        MLH_CHECK(c, hipMemcpyAsync(d_chunk + c->pfChunkCap, chunkT0.data(), (size_t)nchunk * 4, hipMemcpyHostToDevice, st));
+        MLH_CHECK(c, hipMemcpyAsync(d_chunk + 2 * c->pfChunkCap, chunkBase.data(), (size_t)nseg * 4, hipMemcpyHostToDevice, st));
+    }
     MLH_CHECK(c, hipMemcpyAsync(c->d_sidx, seqs, (size_t)nseg * 4, hipMemcpyHostToDevice, st));
     MLH_CHECK(c, hipStreamSynchronize(st)); // the host vectors above go out of scope
     c->identityNseq = 0;
@@ -835,12 +1184,26 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
                 if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<128>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
                 else hipLaunchKernelGGL((k_pf_attn<128, float>), dim3(hp.attnHeads, nblk), dim3(PWG), (size_t)(2 * 64 * 132 + PF_QB * 128) * 4, st, P, L);
             }
-        } else if (hp.gdnDk == 64) {
-            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<64, float>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_gdn<64, f16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
         } else {
-            PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<128, float>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L),
-                           hipLaunchKernelGGL((k_pf_gdn<128, f16_t>), dim3(hp.gdnHeads, nseg, hp.gdnDv / PF_GR), dim3(PWG), 0, st, P, L));
+            const int skipFrom = nchunk > 0 ? GD_C : 0x7fffffff;
+            const dim3 gr(hp.gdnHeads, nseg, hp.gdnDv / PF_GR);
+            if (hp.gdnDk == 64) {
+                PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<64, float>), gr, dim3(PWG), 0, st, P, L, skipFrom),
+                               hipLaunchKernelGGL((k_pf_gdn<64, f16_t>), gr, dim3(PWG), 0, st, P, L, skipFrom));
+            } else {
+                PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_gdn<128, float>), gr, dim3(PWG), 0, st, P, L, skipFrom),
+                               hipLaunchKernelGGL((k_pf_gdn<128, f16_t>), gr, dim3(PWG), 0, st, P, L, skipFrom));
+            }
+            if (nchunk > 0) {
+                const int* dcs = d_chunk; const int* dct = d_chunk + c->pfChunkCap; const int* dcb = d_chunk + 2 * c->pfChunkCap;
+                if (hp.gdnDk == 64) {
+                    hipLaunchKernelGGL((k_gdn_prep<64>), dim3(nchunk, hp.gdnHeads), dim3(128), gdn_prep_lds(64), st, P, L, dcs, dct, (unsigned char*)c->pfGdnWs, c->pfGdnG);
+                    hipLaunchKernelGGL((k_gdn_scan<64>), dim3(hp.gdnHeads, nseg), dim3(128), (size_t)2 * GdLayout<64>::image, st, P, L, dcb, (const unsigned char*)c->pfGdnWs, c->pfGdnG);
+                } else {
+                    hipLaunchKernelGGL((k_gdn_prep<128>), dim3(nchunk, hp.gdnHeads), dim3(256), gdn_prep_lds(128), st, P, L, dcs, dct, (unsigned char*)c->pfGdnWs, c->pfGdnG);
+                    hipLaunchKernelGGL((k_gdn_scan<128>), dim3(hp.gdnHeads, nseg), dim3(256), (size_t)2 * GdLayout<128>::image, st, P, L, dcb, (const unsigned char*)c->pfGdnWs, c->pfGdnG);
+                }
+            }
         }
         GEMM(P.Amix, P.aLd, L.WoG, L.sWo, L.ad, P.H1, d_, P.X, d_, n, d_, L.ad);
         if (hp.pleDim > 0) {

@@ -80,6 +80,8 @@ extern "C" void mlh_destroy(mlh_ctx* c) {
     for (void* p : c->allocs) (void)hipFree(p);
     for (void* p : c->pfAllocs) (void)hipFree(p);
     for (void* p : c->mirrorAllocs) (void)hipFree(p);
+    if (c->pfGdnWs) (void)hipFree(c->pfGdnWs);
+    if (c->pfGdnG) (void)hipFree(c->pfGdnG);
     if (c->stream) (void)hipStreamDestroy(c->stream);
     delete c;
 }

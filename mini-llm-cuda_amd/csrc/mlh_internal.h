@@ -141,6 +141,10 @@ struct mlh_ctx {
     float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
     void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
     int* pfMeta = nullptr;
+    int pfChunkCap = 0;
+    void* pfGdnWs = nullptr;   // chunk operands of the chunk-parallel GDN prefill
+    float* pfGdnG = nullptr;
+    size_t pfGdnChunks = 0;
     const void* EG = nullptr;  // LM-head matrix as the MFMA path reads it (see LayerDev::WaG)
     float sE = 1.0f;
     int gemmDtype = MLH_DTYPE_F32; // operand type of the MFMA path: MLH_DTYPE_F32 or MLH_GEMM_F16
