@@ -589,8 +589,8 @@ template <int DK> struct GdLayout { // one chunk's operand image (bytes), rows p
     static constexpr int KP = (DK + 8) * 2, TP = (GD_C + 8) * 2; // row pitches of [*, DK] and [*, 64] half matrices
     static constexpr int oKt = 0, oQh = oKt + GD_C * KP, oM = oQh + GD_C * KP, oKhT = oM + GD_C * TP;
     static constexpr int image = oKhT + DK * TP;                  // 62464 (DK 128), 36864 (DK 64): multiples of 1024
-    static constexpr int oVt = image;                             // fp32 [64, DV], read straight from global
-    static constexpr int total = image + GD_C * DK * 4;
+    static constexpr int oVt = image;                             // half [64, DV], read straight from global
+    static constexpr int total = image + GD_C * DK * 2;
 };
 __device__ __forceinline__ uint16_t f16_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 
@@ -602,7 +602,7 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     extern __shared__ __attribute__((aligned(16))) unsigned char pls[];
     float* Am = reinterpret_cast<float*>(pls);            // [64][64]
     float* gs = Am + GD_C * GD_C;                         // g[64], beta[64], sp[64], 1/|k|[64], 1/|q|[64], partial sums [4][64]
-    uint16_t* k16 = reinterpret_cast<uint16_t*>(gs + 9 * GD_C); // [64][DK + 8] normalised k, half
+    uint16_t* k16 = reinterpret_cast<uint16_t*>(gs + 12 * GD_C); // [64][DK + 8] normalised k, half
     uint16_t* q16 = k16 + GD_C * (DK + 8);
     const StepArgs& a = P.a;
     const int chunk = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -611,6 +611,8 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     unsigned char* img = ws + ((size_t)chunk * a.gdnHeads + h) * Lay::total;
     float* g = gs; float* beta = gs + GD_C; float* sp = gs + 2 * GD_C; float* rk = gs + 3 * GD_C; float* rq = gs + 4 * GD_C;
     float* part = gs + 5 * GD_C;
+    float* eg = gs + 9 * GD_C;   // e^{g_t}
+    float* egc = gs + 10 * GD_C; // e^{g_C - g_t}
 
     // Thread (sel, cidx) keeps column cidx of q (sel 0: threads [0, DK)) or k (sel 1: threads [DK, 2 DK)) for the 64
     // tokens of the chunk in registers (tokens past the segment end: zero).
@@ -659,6 +661,7 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
 #pragma unroll
         for (int w = 0; w < WPM; w++) ss += part[(m * WPM + w) * GD_C + t];
         (m ? rk : rq)[t] = 1.0f / sqrtf(ss + 1e-6f);
+        if (m == 0) { eg[t] = expf(g[t]); egc[t] = expf(g[GD_C - 1] - g[t]); }
     }
     __syncthreads();
     { // normalise the register column, publish the half copy for the MFMAs
@@ -704,7 +707,7 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
         for (int t = 0; t < GD_C; t++) X[t] = t < nv ? beta[t] * P.QKV[(size_t)(row0 + t) * P.qkvLd + L.offV + h * DV + col] : 0.f;
     } else {
 #pragma unroll
-        for (int t = 0; t < GD_C; t++) X[t] = beta[t] * expf(g[t]) * colv[t];
+        for (int t = 0; t < GD_C; t++) X[t] = beta[t] * eg[t] * colv[t];
     }
 #pragma unroll
     for (int t = 1; t < GD_C; t++) {
@@ -726,17 +729,17 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     // different cache line per lane.
     uint16_t* khs = q16 + GD_C * (DK + 8); // [DK][64 + 8]
     if (tid < DV) { // holds the q column
-        float* Vt = reinterpret_cast<float*>(img + Lay::oVt);
+        uint16_t* Vt = reinterpret_cast<uint16_t*>(img + Lay::oVt);
 #pragma unroll
         for (int t = 0; t < GD_C; t++) {
-            Vt[t * DV + col] = X[t];
-            q16[t * (DK + 8) + sl] = f16_bits(expf(g[t]) * colv[t]);
+            Vt[t * DV + col] = f16_bits(X[t]);
+            q16[t * (DK + 8) + sl] = f16_bits(eg[t] * colv[t]);
         }
     } else { // holds the k column
 #pragma unroll
         for (int t = 0; t < GD_C; t++) {
             k16[t * (DK + 8) + sl] = f16_bits(X[t]);
-            khs[col * (GD_C + 8) + slot_of(t)] = f16_bits(expf(gC - g[t]) * colv[t]); // token axis in slot order
+            khs[col * (GD_C + 8) + slot_of(t)] = f16_bits(egc[t] * colv[t]); // e^{g_C - g_t} k_t, token axis in slot order
         }
     }
     __syncthreads();
@@ -780,11 +783,11 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
     auto issue = [&](int c, int stage) { gd_issue_image<Lay::image, NW>(image_of(c), sls + stage * Lay::image, wave, lane); };
     f32x16 Vt[2];
     auto load_vt = [&](int c) {
-        const float* v = reinterpret_cast<const float*>(image_of(c) + Lay::oVt);
+        const _Float16* v = reinterpret_cast<const _Float16*>(image_of(c) + Lay::oVt);
 #pragma unroll
         for (int tt = 0; tt < 2; tt++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) Vt[tt][i] = v[(32 * tt + 8 * (i >> 2) + 4 * half + (i & 3)) * DV + dv];
+            for (int i = 0; i < 16; i++) Vt[tt][i] = (float)v[(32 * tt + 8 * (i >> 2) + 4 * half + (i & 3)) * DV + dv];
     };
     issue(0, 0);
     load_vt(0);
@@ -1048,7 +1051,7 @@ int mlh_build_gemm_operands(mlh_ctx* c) {
 }
 
 // The headDim-128 attention tiles exceed the 64 KB a launch may use without opting in.
-static size_t gdn_prep_lds(int dk) { return ((size_t)GD_C * GD_C + 9 * GD_C) * 4 + (size_t)2 * GD_C * (dk + 8) * 2 + (size_t)dk * (GD_C + 8) * 2; }
+static size_t gdn_prep_lds(int dk) { return ((size_t)GD_C * GD_C + 12 * GD_C) * 4 + (size_t)2 * GD_C * (dk + 8) * 2 + (size_t)dk * (GD_C + 8) * 2; }
 
 int mlh_init_prefill_kernels(mlh_ctx* c) {
     MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gdn_prep<64>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)gdn_prep_lds(64)));
