@@ -37,9 +37,8 @@ struct PfArgs {
     void* Xn;          // [n, dim] GEMM input (weight dtype)
     float* QKV;        // [n, qkvLd]
     int qkvLd;
-    void* Amix;        // [n, aLd] mixing output (weight dtype)
+    void* Amix;        // [n, aLd] GEMM input of the output projection: mixing output, then (at column L.ad) the PLE row
     int aLd;
-    void* Eple;        // [n, ple]
     float* H1;         // [n, dim]
     void* U;           // [n, ffn]
 };
@@ -878,13 +877,13 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
         for (int i = 0; i < 16; i++) Sg[(size_t)dv * DK + 32 * j + 8 * (i >> 2) + 4 * half + (i & 3)] = St[j][i];
 }
 
-// e[row][j] = silu(ple gate output) * P[tok][j]
+// e[row][j] = silu(ple gate output) * P[tok][j], appended to the row of the mixing output
 template <typename WT, typename AT>
 __global__ void k_pf_ple(PfArgs P, LayerDev L) {
     const int row = blockIdx.x, j = threadIdx.x;
     if (j >= P.a.ple) return;
     const float g = P.QKV[(size_t)row * P.qkvLd + L.offPle + j];
-    put<AT>((AT*)P.Eple + (size_t)row * P.a.ple + j, pf_silu(g) * getw<WT>((const WT*)L.pleTable + (size_t)P.ids[row] * P.a.ple + j));
+    put<AT>((AT*)P.Amix + (size_t)row * P.aLd + L.ad + j, pf_silu(g) * getw<WT>((const WT*)L.pleTable + (size_t)P.ids[row] * P.a.ple + j));
 }
 
 // residual of the last row of every segment -> decode slot buffer x[slot]
@@ -1032,17 +1031,26 @@ int mlh_build_gemm_operands(mlh_ctx* c) {
     unsigned* d_scratch = nullptr;
     if (mirror) { MLH_CHECK(c, hipMalloc((void**)&d_scratch, 8)); }
     int rc = 0;
+    const size_t d = hp.dim, F = hp.ffnDim, pl = hp.pleDim, wb = c->wbytes;
     for (LayerDev& L : c->layers) {
-        L.WaG = L.Wa; L.WoG = L.Wo; L.W13G = L.W13; L.W2G = L.W2; L.pleUpG = L.pleUp;
-        L.sWa = L.sWo = L.sW13 = L.sW2 = L.sPle = 1.0f;
+        L.WaG = L.Wa; L.WoG = L.Wo; L.W13G = L.W13; L.W2G = L.W2;
+        L.sWa = L.sWo = L.sW13 = L.sW2 = 1.0f;
+        const void* wo = L.Wo;
+        if (pl > 0) { // [Wo | pleUp] along K, in the storage type
+            void* cat = nullptr;
+            MLH_CHECK(c, hipMalloc(&cat, d * (L.ad + pl) * wb));
+            c->mirrorAllocs.push_back(cat);
+            MLH_CHECK(c, hipMemcpy2D(cat, (L.ad + pl) * wb, L.Wo, L.ad * wb, L.ad * wb, d, hipMemcpyDeviceToDevice));
+            MLH_CHECK(c, hipMemcpy2D((char*)cat + L.ad * wb, (L.ad + pl) * wb, L.pleUp, pl * wb, pl * wb, d, hipMemcpyDeviceToDevice));
+            wo = cat;
+            L.WoG = cat;
+        }
         if (!mirror) continue;
-        const size_t d = hp.dim, F = hp.ffnDim;
         if ((rc = build_mirror(c, L.Wa, (size_t)L.rowsA * d, &L.WaG, &L.sWa, d_scratch)) ||
-            (rc = build_mirror(c, L.Wo, d * L.ad, &L.WoG, &L.sWo, d_scratch)) ||
+            (rc = build_mirror(c, wo, d * (L.ad + pl), &L.WoG, &L.sWo, d_scratch)) ||
             (rc = build_mirror(c, L.W13, 2 * F * d, &L.W13G, &L.sW13, d_scratch)) ||
             (rc = build_mirror(c, L.W2, d * F, &L.W2G, &L.sW2, d_scratch)))
             break;
-        if (hp.pleDim > 0 && (rc = build_mirror(c, L.pleUp, d * hp.pleDim, &L.pleUpG, &L.sPle, d_scratch))) break;
     }
     c->EG = c->E; c->sE = 1.0f;
     if (rc == 0 && mirror) rc = build_mirror(c, c->E, (size_t)hp.vocabSize * hp.dim, &c->EG, &c->sE, d_scratch);
@@ -1081,8 +1089,8 @@ static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
     int rc;
     const int nblk = cdiv(rows, PF_QB) + hp.maxSeqs, nchunk = cdiv(rows, GD_C) + hp.maxSeqs;
     if ((rc = alloc((void**)&c->pfX, n * hp.dim * 4)) || (rc = alloc(&c->pfXn, n * hp.dim * wb)) ||
-        (rc = alloc((void**)&c->pfQKV, n * c->maxRowsA * 4)) || (rc = alloc(&c->pfA, n * c->maxAd * wb)) ||
-        (rc = alloc(&c->pfE, n * std::max(hp.pleDim, 8) * wb)) || (rc = alloc((void**)&c->pfH1, n * hp.dim * 4)) ||
+        (rc = alloc((void**)&c->pfQKV, n * c->maxRowsA * 4)) || (rc = alloc(&c->pfA, n * (c->maxAd + hp.pleDim) * wb)) ||
+        (rc = alloc((void**)&c->pfH1, n * hp.dim * 4)) ||
         (rc = alloc(&c->pfU, n * hp.ffnDim * wb)) ||
         (rc = alloc((void**)&c->pfMeta, (3 * n + 4 * (size_t)hp.maxSeqs + 2 * (size_t)nblk + 2 * (size_t)nchunk + hp.maxSeqs) * 4)))
         return rc;
@@ -1161,8 +1169,8 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     P.n = n; P.nseg = nseg; P.ids = d_ids; P.rowSeq = d_rowSeq; P.rowPos = d_rowPos;
     P.segStart = d_seg; P.segLen = d_seg + hp.maxSeqs; P.segSeq = d_seg + 2 * hp.maxSeqs; P.segPos0 = d_seg + 3 * hp.maxSeqs;
     P.blkSeg = d_blk; P.blkQ0 = d_blk + c->pfBlkCap;
-    P.X = c->pfX; P.Xn = c->pfXn; P.QKV = c->pfQKV; P.qkvLd = c->maxRowsA; P.Amix = c->pfA; P.aLd = c->maxAd;
-    P.Eple = c->pfE; P.H1 = c->pfH1; P.U = c->pfU;
+    P.X = c->pfX; P.Xn = c->pfXn; P.QKV = c->pfQKV; P.qkvLd = c->maxRowsA; P.Amix = c->pfA; P.aLd = c->maxAd + hp.pleDim;
+    P.H1 = c->pfH1; P.U = c->pfU;
     const int d_ = hp.dim, F = hp.ffnDim, dt = c->gemmDtype;
 #define GEMM(A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K)                                                \
     do {                                                                                                    \
@@ -1208,12 +1216,10 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
                 }
             }
         }
-        GEMM(P.Amix, P.aLd, L.WoG, L.sWo, L.ad, P.H1, d_, P.X, d_, n, d_, L.ad);
-        if (hp.pleDim > 0) {
+        if (hp.pleDim > 0)
             PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_ple<float, float>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L),
                            hipLaunchKernelGGL((k_pf_ple<bf16_t, f16_t>), dim3(n), dim3(std::max(64, hp.pleDim)), 0, st, P, L));
-            GEMM(P.Eple, hp.pleDim, L.pleUpG, L.sPle, hp.pleDim, P.H1, d_, P.H1, d_, n, d_, hp.pleDim);
-        }
+        GEMM(P.Amix, P.aLd, L.WoG, L.sWo, L.ad + hp.pleDim, P.H1, d_, P.X, d_, n, d_, L.ad + hp.pleDim); // Wo . a + pleUp . e + x
         PF_DISPATCH_WT(c, hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (float*)P.Xn, n, d_),
                        hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, P.H1, L.g2, (f16_t*)P.Xn, n, d_));
         { // gate/up projection with SiLU(gate) * up in the epilogue (inference.cu:262-281): U comes out in the GEMM input type
@@ -1258,9 +1264,9 @@ __global__ void k_bd_embed(StepArgs a) {
 
 // Mixing output rows in the GEMM input type: attention layers combine the split-KV partials of the decode
 // attention kernel and apply the sigmoid gate (inference.cu:241-250); GDN layers convert the read-out.
-// PLE rows e = silu(gate) * P[tok] ride along.
+// PLE rows e = silu(gate) * P[tok] are appended to the row (column L.ad on).
 template <typename WT, typename AT>
-__global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix, int aLd, AT* Eple) {
+__global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix, int aLd) {
     const int slot = blockIdx.x, tid = threadIdx.x;
     const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
     if (L.kind == MLH_KIND_ATTENTION) {
@@ -1285,7 +1291,7 @@ __global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix
         for (int i = tid; i < L.ad; i += PWG) put<AT>(Amix + (size_t)slot * aLd + i, a.mix[(size_t)slot * L.ad + i]);
     }
     for (int j = tid; j < a.ple; j += PWG)
-        put<AT>(Eple + (size_t)slot * a.ple + j, pf_silu(qkv[L.offPle + j]) * getw<WT>((const WT*)L.pleTable + (size_t)a.tok[slot] * a.ple + j));
+        put<AT>(Amix + (size_t)slot * aLd + L.ad + j, pf_silu(qkv[L.offPle + j]) * getw<WT>((const WT*)L.pleTable + (size_t)a.tok[slot] * a.ple + j));
 }
 
 // One workgroup per slot: argmax of the slot's logits (lowest index on ties), logits copied to the
@@ -1363,10 +1369,9 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
         GEMM(0, c->pfXn, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
         int rc = mlh_launch_one(c, L.kind == MLH_KIND_ATTENTION ? MLH_K_ATTN : MLH_K_GDN, t, nseq);
         if (rc) return rc;
-        if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd, (f16_t*)c->pfE);
-        else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd, (float*)c->pfE);
-        GEMM(0, c->pfA, c->maxAd, L.WoG, L.sWo, L.ad, c->h1, d_, c->x, d_, n, d_, L.ad);
-        if (hp.pleDim > 0) GEMM(0, c->pfE, hp.pleDim, L.pleUpG, L.sPle, hp.pleDim, c->h1, d_, c->h1, d_, n, d_, hp.pleDim);
+        if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd + hp.pleDim);
+        else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
+        GEMM(0, c->pfA, c->maxAd + hp.pleDim, L.WoG, L.sWo, L.ad + hp.pleDim, c->h1, d_, c->x, d_, n, d_, L.ad + hp.pleDim);
         if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (f16_t*)c->pfXn, n, d_);
         else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (float*)c->pfXn, n, d_);
         GEMM(1, c->pfXn, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_);

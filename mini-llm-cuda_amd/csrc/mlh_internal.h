@@ -40,8 +40,9 @@ struct LayerDev {
     int ad;               // width of the mixing output fed to Wo
     // What the MFMA path multiplies: the matrices themselves for fp32 models; for bf16 models IEEE-half
     // mirrors scaled by a power of two (exact), with the inverse scale applied to the product.
-    const void *WaG, *WoG, *W13G, *W2G, *pleUpG;
-    float sWa, sWo, sW13, sW2, sPle;
+    // WoG is [dim, ad + pleDim]: Wo with pleUp appended along K, so that h1 = [a | e] . WoG^T is one product.
+    const void *WaG, *WoG, *W13G, *W2G;
+    float sWa, sWo, sW13, sW2;
 };
 
 // Arguments shared by all kernels of a decode step.
@@ -139,7 +140,7 @@ struct mlh_ctx {
     int prefillMode = 0; // 0: GEMM path when the shape allows and the call is long enough; 1: token by token
     std::vector<void*> pfAllocs;
     float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
-    void *pfXn = nullptr, *pfA = nullptr, *pfE = nullptr, *pfU = nullptr;
+    void *pfXn = nullptr, *pfA = nullptr, *pfU = nullptr;
     int* pfMeta = nullptr;
     int pfChunkCap = 0;
     void* pfGdnWs = nullptr;   // chunk operands of the chunk-parallel GDN prefill
