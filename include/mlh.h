@@ -179,8 +179,16 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
  * dependent phases of a token are separated by grid barriers instead of kernel launches.  Mode 2 is
  * the same kernel without barriers (consumers spin on tagged data words).  Both need every compute
  * unit free; their waits are bounded, and a call whose wait expired returns -3 with a message.
- * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says. */
+ * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says.
+ * Mode 3 treats each of the eight XCDs as a tensor-parallel rank (heads and FFN units are split over the
+ * XCDs, exchanges inside an XCD go through its L2, only two per layer cross XCDs); it covers models of
+ * attention layers with head size 64 and no per-layer embeddings on a 256-unit device
+ * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise. */
 int mlh_set_persistent(mlh_ctx* ctx, int mode);
+
+/* 1 when mode 3 of mlh_set_persistent applies to this context's model and device, else 0
+ * (no counterpart in the reference: its decode loop is one kernel sequence, inference_orchestrator.cu:120-165). */
+int mlh_xcd_decode_supported(mlh_ctx* ctx);
 
 int mlh_synchronize(mlh_ctx* ctx);
 

@@ -89,6 +89,7 @@ _sigs_dev = {
     "mlh_read_probs": (c_int, [c_void_p, c_int, c_void_p]),
     "mlh_set_graph": (c_int, [c_void_p, c_int]),
     "mlh_set_persistent": (c_int, [c_void_p, c_int]),
+    "mlh_xcd_decode_supported": (c_int, [c_void_p]),
     "mlh_synchronize": (c_int, [c_void_p]),
     "mlh_time_kernel": (c_int, [c_void_p, c_int, c_int, c_int, c_int, _P(c_double), _P(c_double)]),
     "mlh_kernel_name": (c_char_p, [c_int]),
@@ -329,6 +330,9 @@ class Device:
 
     def set_persistent(self, enabled):
         self._check(dev.mlh_set_persistent(self._h, int(enabled)))
+
+    def xcd_decode_supported(self):
+        return bool(dev.mlh_xcd_decode_supported(self._h))
 
     def synchronize(self):
         self._check(dev.mlh_synchronize(self._h))

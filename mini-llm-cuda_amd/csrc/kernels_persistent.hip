@@ -23,62 +23,11 @@
 #include <stdlib.h>
 
 #include "mlh_internal.h"
+#include "persist_common.h"
 
 #define PWG 512
 #define PWAVES (PWG / MLH_WAVE)
 #define P_SPIN_LIMIT (1u << 21)
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ float ald(const float* p) {
-    return __uint_as_float(__hip_atomic_load(reinterpret_cast<const unsigned*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-}
-__device__ __forceinline__ void ast(float* p, float v) {
-    __hip_atomic_store(reinterpret_cast<unsigned*>(p), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ unsigned aldu(const unsigned* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void astu(unsigned* p, unsigned v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-
-// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
-// global load (loads and stores share one counter on this ISA), which would serialise the weight
-// prefetch with each barrier; inside this kernel threads of a workgroup exchange data through LDS only.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
-__device__ __forceinline__ float pwave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MLH_WAVE);
-    return v;
-}
-__device__ __forceinline__ float pwave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MLH_WAVE));
-    return v;
-}
-__device__ __forceinline__ float psigmoid(float v) { return 1.0f / (1.0f + expf(-v)); } // inference.cu:248
-__device__ __forceinline__ float psilu(float v) { return v / (1.0f + expf(-v)); }       // inference.cu:270
-
-// Weight element access: 16-byte vectors, fp32 (4 values) or bf16 (8 values).
-template <typename WT> struct PVec;
-template <> struct PVec<float> {
-    static constexpr int N = 4;
-    typedef f32x4 Raw;
-    static __device__ __forceinline__ Raw load(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
-    static __device__ __forceinline__ void unpack(const Raw& v, float (&o)[4]) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
-    static __device__ __forceinline__ float one(const float* p) { return *p; }
-};
-template <> struct PVec<bf16_t> {
-    static constexpr int N = 8;
-    typedef u32x4 Raw;
-    static __device__ __forceinline__ Raw load(const bf16_t* p) { return *reinterpret_cast<const u32x4*>(p); }
-    static __device__ __forceinline__ void unpack(const Raw& v, float (&o)[8]) {
-        o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
-        o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
-        o[4] = __uint_as_float(v.z << 16); o[5] = __uint_as_float(v.z & 0xffff0000u);
-        o[6] = __uint_as_float(v.w << 16); o[7] = __uint_as_float(v.w & 0xffff0000u);
-    }
-    static __device__ __forceinline__ float one(const bf16_t* p) { return __uint_as_float(((uint32_t)*p) << 16); }
-};
-
 #define PPF 8 // 16-byte chunks per lane and row held in registers across a barrier
 
 template <typename WT>

@@ -1,0 +1,971 @@
+// Batch-1 decode with every XCD of the MI355X acting as a tensor-parallel rank (gfx950, wave64).
+//
+// The chip is eight XCDs of 32 compute units, each XCD with its own L2.  An exchange between
+// workgroups of ONE XCD can go through that L2 (about 0.7 us per hop: the producer's store is written
+// through its L1, the consumer reads with non-temporal loads that do not stay in its L1); an exchange
+// ACROSS XCDs has to go through the memory side (about 2.2 us).  The barrier-per-phase decode kernel
+// pays five chip-wide exchanges per layer; this one pays two, plus five inside the XCDs:
+//
+//   XCD X owns the attention heads h = X, X+8, ... and the FFN units [X F/8, (X+1) F/8).
+//   A  RMSNorm(x) and the q|k|v|gate rows of the XCD's heads           -> inside the XCD  (inference.cu:388-465)
+//   B  attention of those heads, split over 64-key tiles               -> inside the XCD  (inference.cu:467-573)
+//   C  combine + gate, then the Wo product over the XCD's COLUMNS      -> partial h1, across XCDs
+//      (inference.cu:241-250, 582-610)
+//      every workgroup adds the eight partials of its 1/32 slice, publishes the slice inside the XCD
+//   D  RMSNorm(h1) and gate/up rows of the XCD's FFN units, SiLU*up    -> inside the XCD  (inference.cu:612-672)
+//   E  W2 product over the XCD's F/8 columns                           -> partial x, across XCDs (inference.cu:675-699)
+//   LM head rows over all workgroups, argmax across XCDs                                  (inference.cu:705-743)
+//
+// Every exchanged value is one 64-bit word (value, tag): the tag is the number of the layer pass that
+// produced it, the buffers start at zero, and a consumer reads until the tag is there, so data arrival is
+// the synchronisation and a late or stale read only costs another read.  Every exchange is all-to-all
+// within its group, so no workgroup can run more than one exchange ahead of another one of its group and
+// each buffer is rewritten a whole layer later.  Waits are bounded: an expired wait raises the abort
+// flag and every workgroup leaves.
+//
+// A workgroup is 7 worker waves and one communicator wave (two waves per SIMD: 256 registers each).  Workers never wait on global memory except
+// for their own weights: each holds the weight rows of its next two phases in registers, issued two
+// phases ahead, so that HBM latency is off the critical path (loads return in issue order on this ISA:
+// a wave that polled would see its poll answered only after its prefetches).  The communicator does all
+// the polling, the small reductions, q/k norm + RoPE and the softmax-partials combine, puts the result
+// in LDS and meets the workers at a workgroup barrier.  K/V tiles of a wave's first attention unit are
+// fetched global -> LDS directly (no registers) a whole layer ahead.
+#include <stdlib.h>
+
+#include "mlh_internal.h"
+#include "persist_common.h"
+
+#define XWORK 7                 // worker waves per workgroup
+#define XS1 4                   // full-width rows a worker keeps in its first register set
+#define XWG ((XWORK + 1) * 64)  // + the communicator wave
+#define XCDS 8
+#define XPER 32                 // workgroups per XCD: the grid is exactly XCDS * XPER
+#define XLW (XWORK * XPER)      // worker waves per XCD
+#define XNH 4                   // heads per XCD at most
+#define XAW 2                   // worker waves of a workgroup that take attention units
+#define XCH 4                   // 16-byte chunks per lane of a full-width row kept in registers
+#define XSPIN (1u << 20)
+#define XHD 64
+
+typedef unsigned long long u64;
+
+struct XcdArgs {
+    StepArgs a;
+    const LayerDev* layers;
+    int NL, steps, seq;
+    unsigned* abortFlag;
+    unsigned* tagCounter;   // tags already used by earlier launches (advanced by workgroup 0 at the end)
+    unsigned* xcdCount;     // [XCDS] zero at launch: workgroups that have arrived on each XCD
+    int maxTiles;
+    int fs;                 // FFN units per XCD
+    // exchange words: L = read inside the XCD that wrote them ([XCDS] regions), P = partials read by every XCD
+    u64* qkvL; int qkvStride;   // [XCDS][4 * XNH * 64]
+    u64* partL; int partStride; // [XCDS][XNH * maxTiles * 66]
+    u64* h1P;                   // [XCDS][d]
+    u64* h1L;                   // [XCDS][d]
+    u64* uL;                    // [XCDS][fs]
+    u64* xP;                    // [XCDS][d]
+    u64* xL;                    // [XCDS][d]
+    u64* amax;                  // [grid][2]
+    u64* timing;                // optional: communicator of workgroup 0, last step, 8 stamps per layer
+};
+
+__device__ __forceinline__ u64 xpack(float v, unsigned tag) { return ((u64)tag << 32) | __float_as_uint(v); }
+// across XCDs: write-through store, load served by the memory side
+__device__ __forceinline__ void xst(u64* p, float v, unsigned tag) { __hip_atomic_store(p, xpack(v, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ u64 xld(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// inside one XCD: the store leaves the L1 (which is write-through) for the XCD's L2; the load is non-temporal, so
+// the line is not kept in the reader's L1 and the next read fetches it from the L2 again
+__device__ __forceinline__ void lst(u64* p, float v, unsigned tag) { __hip_atomic_store(p, xpack(v, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+__device__ __forceinline__ u64 lld(const u64* p) { return __builtin_nontemporal_load(p); }
+
+// One wave fetches n tagged words into LDS, NB loads per lane in flight, reading again until every tag is there.
+template <bool CROSS, int NB>
+__device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, float* dst, const unsigned* abortFlag, bool& ok) {
+    const int lane = threadIdx.x & 63;
+    for (int base = 0; base < n; base += 64 * NB) {
+        u64 w[NB];
+        for (unsigned spins = 0;; spins++) {
+            asm volatile("" ::: "memory"); // the loads below are repeated every round
+            bool all = true;
+#pragma unroll
+            for (int k = 0; k < NB; k++) {
+                const int i = base + k * 64 + lane;
+                const u64* p = src + (i < n ? i : n - 1);
+                w[k] = CROSS ? xld(p) : lld(p);
+                all = all && (unsigned)(w[k] >> 32) == tag;
+            }
+            if (all) break;
+            if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(abortFlag))) { ok = false; break; }
+        }
+#pragma unroll
+        for (int k = 0; k < NB; k++) {
+            const int i = base + k * 64 + lane;
+            if (i < n) dst[i] = __uint_as_float((unsigned)w[k]);
+        }
+    }
+}
+
+// Sum of the eight XCDs' partials over this workgroup's slice [s0, s0 + sl) plus the residual, published inside
+// the XCD; then the whole vector is fetched from the XCD's 32 slices.  have[X'] false: that XCD contributes nothing.
+__device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int s0, int sl, unsigned tag, unsigned haveMask,
+                                                     const float* resid, float* scratch, u64* pub, float* dst,
+                                                     const unsigned* abortFlag, bool& ok) {
+    const int lane = threadIdx.x & 63;
+    const int n = XCDS * sl;
+    constexpr int NB = 8;
+    u64 w[NB];
+    for (unsigned spins = 0;; spins++) {
+        asm volatile("" ::: "memory");
+        bool all = true;
+#pragma unroll
+        for (int k = 0; k < NB; k++) {
+            const int i = k * 64 + lane;
+            const int xc = i / sl, e = i - xc * sl;
+            const bool need = i < n && ((haveMask >> xc) & 1u);
+            w[k] = need ? xld(part + (size_t)xc * d + s0 + e) : ((u64)tag << 32);
+            all = all && (unsigned)(w[k] >> 32) == tag;
+        }
+        if (all) break;
+        if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(abortFlag))) { ok = false; break; }
+    }
+#pragma unroll
+    for (int k = 0; k < NB; k++) {
+        const int i = k * 64 + lane;
+        if (i < n) scratch[i] = __uint_as_float((unsigned)w[k]);
+    }
+    __builtin_amdgcn_wave_barrier();
+    for (int e = lane; e < sl; e += 64) {
+        float s = 0.f;
+#pragma unroll
+        for (int xc = 0; xc < XCDS; xc++) s += scratch[xc * sl + e]; // fixed order: the result does not depend on timing
+        lst(pub + s0 + e, s + resid[s0 + e], tag);
+    }
+    poll_vec<false, 8>(pub, d, tag, dst, abortFlag, ok);
+}
+
+// Values that are the same in every lane of a wave, said so to the compiler: address arithmetic on them is then
+// done once per wave on the scalar unit, and loads take the form scalar base + 32-bit lane offset.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+template <typename T>
+__device__ __forceinline__ T* uni_ptr(T* p) { // p points into global memory (the layer table holds it as a generic pointer)
+    const u64 v = (u64)p;
+    const u64 u = ((u64)(unsigned)__builtin_amdgcn_readfirstlane((int)(v >> 32)) << 32) | (u64)(unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)v);
+    return (T*)(__attribute__((address_space(1))) T*)u;
+}
+
+template <typename WT, int NR> struct XRows { typename PVec<WT>::Raw r[NR * XCH]; }; // NR full-width rows
+template <typename WT> struct XPf { typename PVec<WT>::Raw r[8]; };
+template <typename WT> struct XGain { f32x4 g[XCH][PVec<WT>::N / 4]; };
+
+// weights (16 bytes) times N activations in registers
+template <typename WT>
+__device__ __forceinline__ float chunk_dot_reg(const typename PVec<WT>::Raw& w, const float (&x)[PVec<WT>::N], float acc) {
+    constexpr int N = PVec<WT>::N;
+    float f[N];
+    PVec<WT>::unpack(w, f);
+#pragma unroll
+    for (int i = 0; i < N; i++) acc = fmaf(f[i], x[i], acc);
+    return acc;
+}
+// weights (16 bytes) times N activations in LDS
+template <typename WT>
+__device__ __forceinline__ float chunk_dot_lds(const typename PVec<WT>::Raw& w, const float* xs, float acc) {
+    constexpr int N = PVec<WT>::N;
+    float f[N];
+    PVec<WT>::unpack(w, f);
+#pragma unroll
+    for (int i = 0; i < N; i += 4) {
+        const f32x4 xv = *reinterpret_cast<const f32x4*>(xs + i);
+        acc = fmaf(f[i], xv.x, acc); acc = fmaf(f[i + 1], xv.y, acc);
+        acc = fmaf(f[i + 2], xv.z, acc); acc = fmaf(f[i + 3], xv.w, acc);
+    }
+    return acc;
+}
+
+// Pins a wave-uniform pointer in scalar registers as an opaque value: without this the optimiser re-associates
+// (base + row offset) + lane offset into (base + lane offset) + row offset, hoists the per-lane part out of the loops
+// and ends up with one 64-bit vector address per load site, held in registers across the whole kernel.
+template <typename T>
+__device__ __forceinline__ const T* pin_uniform(const T* p) { // p: wave-uniform, into global memory
+    u64 v = (u64)p;
+    asm("" : "+s"(v));
+    return (const T*)(__attribute__((address_space(1))) const T*)v;
+}
+
+// 16 bytes at (wave-uniform base) + (32-bit lane offset in bytes) + constant: the addressing mode that needs no
+// 64-bit arithmetic per lane (scalar base register + one offset register + immediate).
+// (The empty statement keeps the widening of the lane offset next to the load: instruction selection works block by
+// block and only then sees that the offset is a 32-bit value.)
+template <typename WT>
+__device__ __forceinline__ typename PVec<WT>::Raw load16(const void* base, unsigned laneBytes, unsigned constBytes) {
+    asm volatile("" : "+v"(laneBytes));
+    return *reinterpret_cast<const typename PVec<WT>::Raw*>(reinterpret_cast<const char*>(base) + (size_t)laneBytes + constBytes);
+}
+__device__ __forceinline__ f32x4 load16f(const void* base, unsigned laneBytes, unsigned constBytes) {
+    asm volatile("" : "+v"(laneBytes));
+    return *reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(base) + (size_t)laneBytes + constBytes);
+}
+
+// NR full-width rows (wave-uniform indices; < 0: none) of the wave-uniform matrix W go into registers: lane l holds
+// columns (ch 64 + l) N .. + N of every row, ch < nch.  Registers of absent rows and chunks keep what they held.
+template <typename WT, int NR>
+__device__ __forceinline__ void issue_rows(typename PVec<WT>::Raw (&dst)[NR * XCH], const WT* W, size_t ld, const int (&rows)[NR], int nch) {
+    const unsigned lb = (threadIdx.x & 63u) * 16u;
+#pragma unroll
+    for (int k = 0; k < NR; k++)
+        if (rows[k] >= 0) {
+            const WT* rp = pin_uniform(W + (size_t)rows[k] * ld);
+#pragma unroll
+            for (int ch = 0; ch < XCH; ch++)
+                if (ch < nch) dst[k * XCH + ch] = load16<WT>(rp, lb, ch * 1024u);
+        }
+}
+template <typename WT>
+__device__ __forceinline__ void issue_gain(XGain<WT>& gn, const float* gain, int nch) {
+    constexpr int N = PVec<WT>::N;
+    const unsigned lb = (threadIdx.x & 63u) * (N * 4u);
+    gain = pin_uniform(gain);
+#pragma unroll
+    for (int ch = 0; ch < XCH; ch++)
+        if (ch < nch)
+#pragma unroll
+            for (int q = 0; q < N / 4; q++) gn.g[ch][q] = load16f(gain, lb, ch * 64u * N * 4u + q * 16u);
+}
+
+// xn = gain * (src / sqrt(mean(src^2) + 1e-8)) for this lane's columns (inference.cu:24-50, 83-95); every wave
+// computes the mean itself from the vector in LDS, so no workgroup reduction is needed.
+template <typename WT>
+__device__ __forceinline__ void normed_columns(const float* src, const XGain<WT>& gn, int d, int nch, float (&xn)[XCH][PVec<WT>::N]) {
+    constexpr int N = PVec<WT>::N;
+    const int c0 = (threadIdx.x & 63) * N;
+    float ss = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < XCH; ch++)
+        if (ch < nch) {
+#pragma unroll
+            for (int q = 0; q < N / 4; q++) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(src + ch * 64 * N + c0 + 4 * q);
+                xn[ch][4 * q] = v.x; xn[ch][4 * q + 1] = v.y; xn[ch][4 * q + 2] = v.z; xn[ch][4 * q + 3] = v.w;
+                ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+            }
+        }
+    ss = pwave_sum(ss);
+    const float r = sqrtf(ss / (float)d + 1e-8f);
+#pragma unroll
+    for (int ch = 0; ch < XCH; ch++)
+        if (ch < nch) {
+#pragma unroll
+            for (int q = 0; q < N / 4; q++) {
+                const f32x4 g = gn.g[ch][q];
+                xn[ch][4 * q] = g.x * (xn[ch][4 * q] / r); xn[ch][4 * q + 1] = g.y * (xn[ch][4 * q + 1] / r);
+                xn[ch][4 * q + 2] = g.z * (xn[ch][4 * q + 2] / r); xn[ch][4 * q + 3] = g.w * (xn[ch][4 * q + 3] / r);
+            }
+        }
+}
+
+template <typename WT, int NRAW>
+__device__ __forceinline__ float row_dot_reg(const typename PVec<WT>::Raw (&r)[NRAW], int which, int nch, const float (&xn)[XCH][PVec<WT>::N]) {
+    float acc = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < XCH; ch++)
+        if (ch < nch) acc = chunk_dot_reg<WT>(r[which * XCH + ch], xn[ch], acc);
+    return acc;
+}
+template <typename WT>
+__device__ __forceinline__ float row_dot_stream(const WT* W, size_t ld, int row, int nch, const float (&xn)[XCH][PVec<WT>::N]) {
+    const WT* rp = pin_uniform(W + (size_t)row * ld);
+    const unsigned lb = (threadIdx.x & 63u) * 16u;
+    float acc = 0.f;
+#pragma unroll
+    for (int ch = 0; ch < XCH; ch++)
+        if (ch < nch) acc = chunk_dot_reg<WT>(load16<WT>(rp, lb, ch * 1024u), xn[ch], acc);
+    return acc;
+}
+
+// Row of the fused first-phase matrix behind local index rho of XCD X: parts q, k, v, gate; nh heads of 64 rows each.
+__device__ __forceinline__ int rowA_of(int offK, int offV, int offG, int X, int nh, int rho) {
+    const int per = nh * XHD, p = rho / per, rem = rho - p * per, j = rem >> 6, i = rem & 63;
+    const int off = p == 0 ? 0 : p == 1 ? offK : p == 2 ? offV : offG;
+    return off + (X + XCDS * j) * XHD + i;
+}
+
+// Wo columns of the XCD's heads: a pass covers N rows per wave (64/N lanes per 64-column head segment).
+template <typename WT>
+__device__ __forceinline__ void issue_wo(XPf<WT>& pf, const WT* Wo, int ad, int X, int nh, int lw, int d) {
+    constexpr int N = PVec<WT>::N, CPS = XHD / N;
+    const unsigned lane = threadIdx.x & 63u;
+    const unsigned lb = ((lane / CPS) * (unsigned)ad + (lane % CPS) * N) * (unsigned)sizeof(WT); // row within the pass, chunk within the head segment
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+        if ((p * XLW + lw) * N < d) {
+            const WT* rp = pin_uniform(Wo + (size_t)((p * XLW + lw) * N) * ad + X * XHD);
+#pragma unroll
+            for (int j = 0; j < XNH; j++)
+                if (j < nh) pf.r[p * XNH + j] = load16<WT>(rp, lb, j * XCDS * XHD * (unsigned)sizeof(WT));
+        }
+}
+// W2 columns [X fs, (X+1) fs): rows lw, lw + XLW, ...; four rows x two chunks per lane are prefetched.
+template <typename WT>
+__device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int fs, int F, int lw, int d) {
+    constexpr int N = PVec<WT>::N;
+    const int lane = threadIdx.x & 63, CR = fs / N;
+    const unsigned lb = (threadIdx.x & 63u) * 16u;
+#pragma unroll
+    for (int k = 0; k < 4; k++)
+        if (lw + XLW * k < d) {
+            const WT* rp = pin_uniform(W2 + (size_t)(lw + XLW * k) * F + (size_t)X * fs);
+#pragma unroll
+            for (int c0 = 0; c0 < 2; c0++)
+                if (lane + 64 * c0 < CR) pf.r[k * 2 + c0] = load16<WT>(rp, lb, c0 * 1024u);
+        }
+}
+
+// K and V tile (64 rows x 64 floats each) of one head, rows below `lim`, global -> LDS without registers.  An
+// instruction moves 1 KB: lane i's 16 bytes land at base + 16 i, i.e. row 4q + i/16, slot i%16; the lane fetches the
+// piece that belongs there under the swizzle slot = piece ^ (row & 15), which makes the per-lane row reads of the
+// score loop conflict-free.  Kh, Vh: wave-uniform pointers to row 0 of the head's slice of the page.
+__device__ __forceinline__ void issue_kv_tile(const float* Kh, const float* Vh, int d, int lim, float* tK, float* tV) {
+    const unsigned lane = threadIdx.x & 63u;
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        const unsigned row = 4 * q + (lane >> 4), piece = (lane & 15) ^ (row & 15);
+        // row 4q of the tile is the wave-uniform part of the address, the lane adds (lane / 16) rows and its piece
+        const char* Kq = pin_uniform(reinterpret_cast<const char*>(Kh + (size_t)(4 * q) * d));
+        const char* Vq = pin_uniform(reinterpret_cast<const char*>(Vh + (size_t)(4 * q) * d));
+        unsigned lb = ((lane >> 4) * (unsigned)d + piece * 4u) * 4u;
+        if ((int)row < lim) {
+            asm volatile("" : "+v"(lb));
+            __builtin_amdgcn_global_load_lds(Kq + (size_t)lb, tK + q * 256, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(Vq + (size_t)lb, tV + q * 256, 16, 0, 0);
+        }
+    }
+}
+
+struct XShared {
+    float *xs, *h1s, *qkvs, *as, *us, *scratch, *bestv, *tiles;
+    int *besti, *ctl;
+    LayerDev* Ls;
+};
+
+#define X_STAMP(slot)                                                                                   \
+    do {                                                                                                \
+        if (P.timing && wg == 0 && lane == 0 && step == P.steps - 1) P.timing[(slot)] = wall_clock64(); \
+    } while (0)
+#define X_BARRIER()                  \
+    do {                             \
+        lds_barrier();               \
+        if (uni(S.ctl[0])) return;   \
+    } while (0)
+
+// ------------------------------------------------------------------------------------------------ communicator
+template <typename WT>
+__device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
+    const StepArgs& a = P.a;
+    const int d = a.dim, V = a.vocab;
+    const int lane = threadIdx.x & 63, wg = blockIdx.x;
+    const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
+    const int np = 3 + (a.gating ? 1 : 0);
+    const int RA = np * nh * XHD;
+    const int sl = d / XPER, s0 = r * sl;
+    unsigned headMask = 0; // XCDs that own at least one head
+    for (int xc = 0; xc < XCDS; xc++) headMask |= (a.heads > xc ? 1u : 0u) << xc;
+    u64* qkvL = P.qkvL + (size_t)X * P.qkvStride;
+    u64* partL = P.partL + (size_t)X * P.partStride;
+    bool ok = true;
+
+    for (int step = 0; step < P.steps; step++) {
+        const float rc = a.rope[(size_t)pos * XHD + (lane & ~1)], rsn = a.rope[(size_t)pos * XHD + (lane | 1)];
+        const int pageNew = a.pageTable[P.seq * a.pagesPerSeq + (pos >> 6)];
+        const int T = pos + 1, ntiles = (T + 63) >> 6;
+        // embedding gather (inference.cu:9-22): every workgroup keeps its own copy of the residual stream
+        for (int i = lane; i < d; i += 64) S.xs[i] = PVec<WT>::one((const WT*)a.E + (size_t)tok * d + i);
+
+        for (int t = P.NL - 1; t >= 0; t--) { // file block 0 is the top of the stack (inference.cu:384-385)
+            const LayerDev& L = S.Ls[t];
+            const unsigned lt = tagBase + (unsigned)(step * P.NL + (P.NL - 1 - t) + 1);
+            const int ts = (P.NL - 1 - t) * 16;
+            X_STAMP(ts + 0);
+            // q/k gains of this layer: issued ahead of the wait for x, whose answer comes later anyway
+            float gq[XNH], gk[XNH];
+            if (a.qkNorm)
+#pragma unroll
+                for (int j = 0; j < XNH; j++)
+                    if (j < nh) { gq[j] = uni_ptr(L.gq)[(X + XCDS * j) * XHD + lane]; gk[j] = uni_ptr(L.gk)[(X + XCDS * j) * XHD + lane]; }
+            if (t != P.NL - 1) // partial x of the layer below, all XCDs, + its residual h1
+                reduce_publish_fetch(P.xP, d, s0, sl, lt - 1, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok);
+            if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+            X_STAMP(ts + 1);
+            X_BARRIER(); // 1: x in LDS
+
+            // q | k | v | gate of the XCD's heads; per-head RMSNorm (inference.cu:52-81, 97-111), RoPE on adjacent
+            // pairs (inference.cu:113-134); workgroup 0 of the XCD appends the new K/V rows to the cache
+            poll_vec<false, 8>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok);
+            {
+                float* qs = S.qkvs;
+                float* ks = qs + nh * XHD;
+                float* vs = ks + nh * XHD;
+#pragma unroll
+                for (int j = 0; j < XNH; j++)
+                    if (j < nh) {
+                        const int h = X + XCDS * j;
+                        float q = qs[j * XHD + lane], k = ks[j * XHD + lane];
+                        if (a.qkNorm) {
+                            const float sq = pwave_sum(q * q), sk = pwave_sum(k * k);
+                            const float rq = sqrtf(sq / (float)XHD + 1e-8f), rk = sqrtf(sk / (float)XHD + 1e-8f);
+                            q = gq[j] * (q / rq);
+                            k = gk[j] * (k / rk);
+                        }
+                        const float qo = __shfl_xor(q, 1, MLH_WAVE), ko = __shfl_xor(k, 1, MLH_WAVE);
+                        if (lane & 1) { q = rsn * qo + rc * q; k = rsn * ko + rc * k; }
+                        else { q = rc * q - rsn * qo; k = rc * k - rsn * ko; }
+                        qs[j * XHD + lane] = q;
+                        ks[j * XHD + lane] = k;
+                        if (r == 0) { // write-through: read from the next step on, by whichever workgroup takes the tile
+                            const size_t o = ((size_t)pageNew * MLH_KV_PAGE + (pos & 63)) * d + h * XHD + lane;
+                            ast(uni_ptr(L.K) + o, k);
+                            ast(uni_ptr(L.V) + o, vs[j * XHD + lane]);
+                        }
+                    }
+            }
+            if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+            X_STAMP(ts + 2);
+            X_BARRIER(); // 2: q, k, v, gate in LDS
+
+            // softmax partials of the XCD's heads -> mixing output (lane = dimension), gate (inference.cu:241-250)
+            {
+                const int U = nh * ntiles;
+                const float* gs = S.qkvs + 3 * nh * XHD;
+                float M = -1.0e30f, num = 0.f, den = 0.f;
+                int cur = 0;
+                for (int u0 = 0; u0 < U; u0 += 16) {
+                    u64 wa[16], wml;
+                    for (unsigned spins = 0;; spins++) {
+                        asm volatile("" ::: "memory");
+                        bool all = true;
+#pragma unroll
+                        for (int k = 0; k < 16; k++) {
+                            const int u = u0 + k < U ? u0 + k : U - 1, j = u / ntiles, tl = u - j * ntiles;
+                            wa[k] = lld(partL + ((size_t)j * P.maxTiles + tl) * (XHD + 2) + lane);
+                            all = all && (unsigned)(wa[k] >> 32) == lt;
+                        }
+                        {   // lanes 0..15: running maxima of the 16 units, lanes 16..31: their sums
+                            const int k = lane & 15, u = u0 + k < U ? u0 + k : U - 1, j = u / ntiles, tl = u - j * ntiles;
+                            wml = lld(partL + ((size_t)j * P.maxTiles + tl) * (XHD + 2) + XHD + ((lane >> 4) & 1));
+                            all = all && (unsigned)(wml >> 32) == lt;
+                        }
+                        if (__all(all)) break;
+                        if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(P.abortFlag))) { ok = false; break; }
+                    }
+                    const float ml = __uint_as_float((unsigned)wml);
+#pragma unroll
+                    for (int k = 0; k < 16; k++) {
+                        if (u0 + k < U) {
+                            const int j = (u0 + k) / ntiles;
+                            if (j != cur) {
+                                float v = num / den;
+                                if (a.gating) v = v * psigmoid(gs[cur * XHD + lane]);
+                                S.as[cur * XHD + lane] = v;
+                                cur = j; M = -1.0e30f; num = 0.f; den = 0.f;
+                            }
+                            const float mk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ml), k));
+                            const float lk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ml), 16 + k));
+                            const float Mn = fmaxf(M, mk), corr = expf(M - Mn), w = expf(mk - Mn);
+                            num = fmaf(w, __uint_as_float((unsigned)wa[k]), num * corr);
+                            den = fmaf(w, lk, den * corr);
+                            M = Mn;
+                        }
+                    }
+                }
+                if (U > 0) {
+                    float v = num / den;
+                    if (a.gating) v = v * psigmoid(gs[cur * XHD + lane]);
+                    S.as[cur * XHD + lane] = v;
+                }
+            }
+            if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+            X_STAMP(ts + 3);
+            X_BARRIER(); // 3: mixing output of the XCD's heads in LDS
+
+            // h1 = x + sum of the XCDs' Wo partials (inference.cu:252-260)
+            reduce_publish_fetch(P.h1P, d, s0, sl, lt, headMask, S.xs, S.scratch, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok);
+            if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+            X_STAMP(ts + 4);
+            X_BARRIER(); // 4: h1 in LDS
+
+            poll_vec<false, 8>(P.uL + (size_t)X * P.fs, P.fs, lt, S.us, P.abortFlag, ok);
+            if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+            X_STAMP(ts + 5);
+            X_BARRIER(); // 5: the XCD's FFN activations in LDS
+        }
+
+        // ---------------------------------------------------------------------- LM head + argmax
+        const unsigned ltLast = tagBase + (unsigned)(step * P.NL + P.NL);
+        reduce_publish_fetch(P.xP, d, s0, sl, ltLast, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok);
+        if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+        X_BARRIER(); // final x in LDS
+        X_BARRIER(); // the workers' best logits in LDS
+        {
+            float v = lane < XWORK ? S.bestv[lane] : -3.0e38f;
+            int i = lane < XWORK ? S.besti[lane] : 0x7fffffff;
+#pragma unroll
+            for (int o = 4; o > 0; o >>= 1) {
+                const float v2 = __shfl_xor(v, o, MLH_WAVE);
+                const int i2 = __shfl_xor(i, o, MLH_WAVE);
+                if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
+            }
+            if (lane == 0) {
+                xst(P.amax + 2 * wg, v, tagBase + (unsigned)step + 1);
+                xst(P.amax + 2 * wg + 1, __uint_as_float((unsigned)i), tagBase + (unsigned)step + 1);
+            }
+            poll_vec<true, 8>(P.amax, 2 * (int)gridDim.x, tagBase + (unsigned)step + 1, S.scratch, P.abortFlag, ok);
+            v = -3.0e38f; i = 0x7fffffff;
+            for (int k = lane; k < (int)gridDim.x; k += 64) {
+                const float v2 = S.scratch[2 * k];
+                const int i2 = (int)__float_as_uint(S.scratch[2 * k + 1]);
+                if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float v2 = __shfl_xor(v, o, MLH_WAVE);
+                const int i2 = __shfl_xor(i, o, MLH_WAVE);
+                if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
+            }
+            if (i < 0 || i >= V) i = 0; // only reachable with non-finite logits
+            tok = i;
+            if (lane == 0) S.ctl[1] = tok;
+            if (wg == 0 && lane == 0) { // the append of inference_orchestrator.cu:149-151, kept on the device
+                const int sc = *a.stepCounter;
+                if (sc + step < a.outCapacity) a.outIds[sc + step] = tok;
+            }
+        }
+        if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+        pos += 1;
+        X_BARRIER(); // next token in LDS
+    }
+    if (wg == 0 && lane == 0) {
+        // every workgroup read the counter before it could contribute to the first exchange, and this point lies
+        // behind the last one
+        *P.tagCounter = tagBase + (unsigned)(P.steps * P.NL + 1);
+        *a.stepCounter += P.steps;
+        a.pos[P.seq] = pos;
+        ((int*)a.tok)[0] = tok;
+        a.nextTok[P.seq] = tok;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ workers
+template <typename WT>
+__device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
+    constexpr int N = PVec<WT>::N, CPS = XHD / N;
+    const StepArgs& a = P.a;
+    const int d = a.dim, F = a.ffn, V = a.vocab, fs = P.fs;
+    const int nch = d / (64 * N); // 16-byte chunks per lane of a full-width row
+    const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6), wg = blockIdx.x;
+    const int lw = wave * XPER + r;             // worker wave within the XCD: consecutive rows land on different workgroups
+    const int gwl = wave * (int)gridDim.x + wg; // worker wave within the grid (LM head)
+    const int TWL = XWORK * (int)gridDim.x;
+    const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
+    const int np = 3 + (a.gating ? 1 : 0);
+    const int RA = np * nh * XHD;
+    u64* qkvL = P.qkvL + (size_t)X * P.qkvStride;
+    u64* partL = P.partL + (size_t)X * P.partStride;
+    float* tK = S.tiles + (wave < XAW ? wave : 0) * 8192;
+    float* tV = tK + 4096;
+    const int aslot = wave * XPER + r; // attention unit slot of this wave (waves below XAW only)
+    const WT* E = (const WT*)a.E;
+
+    XRows<WT, XS1> s1; // rows of phases A / D / LM head
+    XPf<WT> s2;      // rows of phases C / E / LM head
+    XGain<WT> gn;
+    // first-phase rows lw, lw + XLW, ... of layer Lx and its first gain vector
+    auto issueA = [&](const LayerDev& Lx) {
+        const int offK = uni(Lx.offK), offV = uni(Lx.offV), offG = uni(Lx.offG);
+        int rows[XS1];
+#pragma unroll
+        for (int k = 0; k < XS1; k++) rows[k] = lw + XLW * k < RA ? rowA_of(offK, offV, offG, X, nh, lw + XLW * k) : -1;
+        issue_rows<WT, XS1>(s1.r, uni_ptr((const WT*)Lx.Wa), d, rows, nch);
+        issue_gain<WT>(gn, uni_ptr(Lx.g1), nch);
+    };
+    // first K/V tile of this wave in layer Lx when the sequence holds npos rows
+    auto issueKV = [&](const LayerDev& Lx, int npos) {
+        const int nt = (npos + 64) >> 6;
+        if (aslot < nh * nt) {
+            const int j = aslot % nh, tl = aslot / nh;
+            const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + tl]);
+            const size_t base = ((size_t)page * MLH_KV_PAGE) * d + (X + XCDS * j) * XHD;
+            issue_kv_tile(uni_ptr((const float*)Lx.K) + base, uni_ptr((const float*)Lx.V) + base, d, npos - tl * 64, tK, tV);
+        }
+    };
+    {
+        const LayerDev& L0 = S.Ls[P.NL - 1];
+        issueA(L0);
+        issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, lw, d);
+        if (wave < XAW) issueKV(L0, pos);
+    }
+
+    for (int step = 0; step < P.steps; step++) {
+        const int T = pos + 1, ntiles = (T + 63) >> 6, newTile = pos >> 6;
+        for (int t = P.NL - 1; t >= 0; t--) {
+            const LayerDev& L = S.Ls[t];
+            const unsigned lt = tagBase + (unsigned)(step * P.NL + (P.NL - 1 - t) + 1);
+            const bool lastLayer = t == 0;
+            const LayerDev& Ln = S.Ls[lastLayer ? P.NL - 1 : t - 1];
+            X_BARRIER(); // 1
+            // ------------------------------------------------------------------ phase A
+            {
+                float xn[XCH][N];
+                normed_columns<WT>(S.xs, gn, d, nch, xn);
+#pragma unroll
+                for (int k = 0; k < XS1; k++) {
+                    const int rho = lw + XLW * k;
+                    if (rho < RA) {
+                        const float acc = pwave_sum(row_dot_reg<WT>(s1.r, k, nch, xn));
+                        if (lane == 0) lst(qkvL + rho, acc, lt);
+                    }
+                }
+                if (lw + XS1 * XLW < RA) {
+                    const int offK = uni(L.offK), offV = uni(L.offV), offG = uni(L.offG);
+                    const WT* Wa = uni_ptr((const WT*)L.Wa);
+                    for (int rho = lw + XS1 * XLW; rho < RA; rho += XLW) {
+                        const float acc = pwave_sum(row_dot_stream<WT>(Wa, d, rowA_of(offK, offV, offG, X, nh, rho), nch, xn));
+                        if (lane == 0) lst(qkvL + rho, acc, lt);
+                    }
+                }
+            }
+            X_BARRIER(); // 2
+            // ------------------------------------------------------------------ phase B
+            if (wave < XAW) {
+                const int U = nh * ntiles;
+                const float* qsAll = S.qkvs;
+                const float* ksAll = qsAll + nh * XHD;
+                const float* vsAll = ksAll + nh * XHD;
+                for (int u = aslot; u < U; u += XAW * XPER) {
+                    const int j = u % nh, tl = u / nh, j0 = tl << 6;
+                    if (u != aslot) { // tiles beyond the first one were not fetched ahead
+                        const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + tl]);
+                        const size_t base = ((size_t)page * MLH_KV_PAGE) * d + (X + XCDS * j) * XHD;
+                        issue_kv_tile(uni_ptr((const float*)L.K) + base, uni_ptr((const float*)L.V) + base, d, pos - j0, tK, tV);
+                    }
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the tile has landed in LDS
+                    const int nv = T - j0 < 64 ? T - j0 : 64;       // keys of this tile, the new one included
+                    if (tl == newTile && lane < 16) {                // this step's row comes from LDS, not from the cache
+                        const int rn = pos - j0;
+                        *reinterpret_cast<f32x4*>(tK + rn * 64 + ((lane ^ (rn & 15)) << 2)) = *reinterpret_cast<const f32x4*>(ksAll + j * XHD + lane * 4);
+                        *reinterpret_cast<f32x4*>(tV + rn * 64 + ((lane ^ (rn & 15)) << 2)) = *reinterpret_cast<const f32x4*>(vsAll + j * XHD + lane * 4);
+                    }
+                    __builtin_amdgcn_wave_barrier();
+                    float s = 0.f;
+                    {
+                        const float* kr = tK + lane * 64;
+                        const float* qs = qsAll + j * XHD;
+#pragma unroll 4
+                        for (int p = 0; p < 16; p++) {
+                            const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + ((p ^ (lane & 15)) << 2));
+                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qs + p * 4);
+                            s = fmaf(kk.x, qq.x, s); s = fmaf(kk.y, qq.y, s); s = fmaf(kk.z, qq.z, s); s = fmaf(kk.w, qq.w, s);
+                        }
+                    }
+                    const bool valid = lane < nv;
+                    s = valid ? s / sqrtf((float)XHD) : -1.0e30f; // inference.cu:154
+                    const float m = pwave_max(s);
+                    const float e = valid ? expf(s - m) : 0.f;
+                    const float l = pwave_sum(e);
+                    float acc = 0.f;
+                    const float* vcol = tV + (lane & 3);
+                    const int pc = lane >> 2;
+                    if (nv == 64) {
+#pragma unroll 8
+                        for (int jj = 0; jj < 64; jj++) {
+                            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj));
+                            acc = fmaf(pj, vcol[jj * 64 + ((pc ^ (jj & 15)) << 2)], acc);
+                        }
+                    } else {
+                        for (int jj = 0; jj < nv; jj++) { // rows from nv on hold whatever the tile held before
+                            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj));
+                            acc = fmaf(pj, vcol[jj * 64 + ((pc ^ (jj & 15)) << 2)], acc);
+                        }
+                    }
+                    u64* out = partL + ((size_t)j * P.maxTiles + tl) * (XHD + 2);
+                    lst(out + lane, acc, lt);
+                    if (lane == 0) { lst(out + XHD, m, lt); lst(out + XHD + 1, l, lt); }
+                    __builtin_amdgcn_wave_barrier();
+                }
+                // first tile of this wave for the next layer pass (the next step's first layer sees one more row)
+                if (!(lastLayer && step == P.steps - 1)) issueKV(Ln, lastLayer ? pos + 1 : pos);
+            }
+            // gate/up rows of this wave's first two FFN units, and the second gain vector
+            {
+                int rows[XS1];
+#pragma unroll
+                for (int k = 0; k < XS1 / 2; k++) {
+                    const int q = lw + XLW * k;
+                    rows[2 * k] = q < fs ? 2 * (X * fs + q) : -1;
+                    rows[2 * k + 1] = q < fs ? 2 * (X * fs + q) + 1 : -1;
+                }
+                issue_rows<WT, XS1>(s1.r, uni_ptr((const WT*)L.W13), d, rows, nch);
+                issue_gain<WT>(gn, uni_ptr(L.g2), nch);
+            }
+            X_BARRIER(); // 3
+            // ------------------------------------------------------------------ phase C
+            if (nh > 0) {
+                const int rs = lane / CPS, c = lane % CPS;
+                const int ad = uni(L.ad);
+                for (int p = 0; (p * XLW + lw) * N < d; p++) {
+                    const int row = (p * XLW + lw) * N + rs;
+                    float acc = 0.f;
+#pragma unroll
+                    for (int j = 0; j < XNH; j++)
+                        if (j < nh) {
+                            const typename PVec<WT>::Raw w = p == 0 ? s2.r[j] : p == 1 ? s2.r[XNH + j]
+                                : PVec<WT>::load(uni_ptr((const WT*)L.Wo) + (size_t)row * ad + (X + XCDS * j) * XHD + c * N);
+                            acc = chunk_dot_lds<WT>(w, S.as + j * XHD + c * N, acc);
+                        }
+#pragma unroll
+                    for (int o = CPS / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, MLH_WAVE);
+                    if (c == 0) xst(P.h1P + (size_t)X * d + row, acc, lt);
+                }
+            }
+            issue_w2<WT>(s2, uni_ptr((const WT*)L.W2), X, fs, F, lw, d);
+            X_BARRIER(); // 4
+            // ------------------------------------------------------------------ phase D
+            {
+                float xn[XCH][N];
+                normed_columns<WT>(S.h1s, gn, d, nch, xn);
+#pragma unroll
+                for (int k = 0; k < XS1 / 2; k++) {
+                    const int q = lw + XLW * k;
+                    if (q < fs) {
+                        const float g = pwave_sum(row_dot_reg<WT>(s1.r, 2 * k, nch, xn)), up = pwave_sum(row_dot_reg<WT>(s1.r, 2 * k + 1, nch, xn));
+                        if (lane == 0) lst(P.uL + (size_t)X * fs + q, psilu(g) * up, lt); // inference.cu:262-281
+                    }
+                }
+                if (lw + (XS1 / 2) * XLW < fs) {
+                    const WT* W13 = uni_ptr((const WT*)L.W13);
+                    for (int q = lw + (XS1 / 2) * XLW; q < fs; q += XLW) {
+                        const int pr = X * fs + q;
+                        const float g = pwave_sum(row_dot_stream<WT>(W13, d, 2 * pr, nch, xn));
+                        const float up = pwave_sum(row_dot_stream<WT>(W13, d, 2 * pr + 1, nch, xn));
+                        if (lane == 0) lst(P.uL + (size_t)X * fs + q, psilu(g) * up, lt);
+                    }
+                }
+            }
+            if (!lastLayer) {
+                issueA(Ln);
+            } else { // LM-head rows gwl, gwl + TWL, ... and the final gain
+                int rows[XS1];
+#pragma unroll
+                for (int k = 0; k < XS1; k++) rows[k] = gwl + TWL * k < V ? gwl + TWL * k : -1;
+                issue_rows<WT, XS1>(s1.r, E, d, rows, nch);
+                issue_gain<WT>(gn, a.gF, nch);
+            }
+            X_BARRIER(); // 5
+            // ------------------------------------------------------------------ phase E
+            {
+                const int CR = fs / N;
+                const WT* W2x = uni_ptr((const WT*)L.W2) + (size_t)X * fs;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const int row = lw + XLW * k;
+                    if (row < d) {
+                        float acc = 0.f;
+#pragma unroll
+                        for (int c0 = 0; c0 < 2; c0++) {
+                            const int cc = lane + 64 * c0;
+                            if (cc < CR) acc = chunk_dot_lds<WT>(s2.r[k * 2 + c0], S.us + cc * N, acc);
+                        }
+                        for (int cc = lane + 128; cc < CR; cc += 64)
+                            acc = chunk_dot_lds<WT>(PVec<WT>::load(W2x + (size_t)row * F + cc * N), S.us + cc * N, acc);
+                        acc = pwave_sum(acc);
+                        if (lane == 0) xst(P.xP + (size_t)X * d + row, acc, lt); // inference.cu:283-291 (the readers add the residual)
+                    }
+                }
+                for (int row = lw + 4 * XLW; row < d; row += XLW) {
+                    float acc = 0.f;
+                    for (int cc = lane; cc < CR; cc += 64)
+                        acc = chunk_dot_lds<WT>(PVec<WT>::load(W2x + (size_t)row * F + cc * N), S.us + cc * N, acc);
+                    acc = pwave_sum(acc);
+                    if (lane == 0) xst(P.xP + (size_t)X * d + row, acc, lt);
+                }
+            }
+            if (!lastLayer) {
+                issue_wo<WT>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, lw, d);
+            } else {
+                const int rows[2] = {gwl + XS1 * TWL < V ? gwl + XS1 * TWL : -1, gwl + (XS1 + 1) * TWL < V ? gwl + (XS1 + 1) * TWL : -1};
+                issue_rows<WT, 2>(s2.r, E, d, rows, nch);
+            }
+        }
+
+        // ---------------------------------------------------------------------- LM head + argmax
+        X_BARRIER(); // final x in LDS
+        {
+            float xn[XCH][N];
+            normed_columns<WT>(S.xs, gn, d, nch, xn); // inference.cu:705-715
+            float best = -3.0e38f;
+            int bidx = 0x7fffffff;
+            auto take = [&](int row, float acc) { // rows ascend per wave: ties keep the lower index
+                acc = pwave_sum(acc);
+                if (lane == 0) a.logits[(size_t)P.seq * V + row] = acc;
+                if (acc > best) { best = acc; bidx = row; }
+            };
+#pragma unroll
+            for (int k = 0; k < XS1; k++)
+                if (gwl + TWL * k < V) take(gwl + TWL * k, row_dot_reg<WT>(s1.r, k, nch, xn));
+#pragma unroll
+            for (int k = 0; k < 2; k++)
+                if (gwl + TWL * (XS1 + k) < V) take(gwl + TWL * (XS1 + k), row_dot_reg<WT>(s2.r, k, nch, xn));
+            for (int row = gwl + (XS1 + 2) * TWL; row < V; row += TWL) take(row, row_dot_stream<WT>(E, d, row, nch, xn));
+            if (lane == 0) { S.bestv[wave] = best; S.besti[wave] = bidx; }
+        }
+        if (step + 1 < P.steps) { // first layer of the next step
+            const LayerDev& L0 = S.Ls[P.NL - 1];
+            issueA(L0);
+            issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, lw, d);
+        }
+        X_BARRIER(); // best logits in LDS
+        X_BARRIER(); // next token in LDS
+        tok = S.ctl[1];
+        pos += 1;
+    }
+    (void)tok;
+}
+
+template <typename WT>
+__global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
+    extern __shared__ float lds[];
+    const StepArgs& a = P.a;
+    const int d = a.dim, wave = uni(threadIdx.x >> 6);
+    XShared S;
+    S.xs = lds;
+    S.h1s = S.xs + d;
+    S.qkvs = S.h1s + d;                 // [4][nh * 64] q | k | v | gate of the XCD's heads
+    S.as = S.qkvs + 4 * XNH * XHD;      // [nh * 64] mixing output
+    S.us = S.as + XNH * XHD;            // [fs]
+    S.scratch = S.us + ((P.fs + 3) & ~3); // [max(d / 4, 2 * grid)]
+    S.bestv = S.scratch + 512;
+    S.besti = reinterpret_cast<int*>(S.bestv + 16);
+    S.ctl = S.besti + 16;               // [0] a wait expired, [1] next token
+    S.tiles = reinterpret_cast<float*>(S.ctl + 16); // [XAW][K tile | V tile]
+    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 8192);
+    for (int i = threadIdx.x; i < P.NL * (int)(sizeof(LayerDev) / 4); i += XWG)
+        reinterpret_cast<uint32_t*>(S.Ls)[i] = reinterpret_cast<const uint32_t*>(P.layers)[i];
+    if (threadIdx.x == 0) {
+        // The exchange inside an XCD needs to know which workgroups share an L2: the XCD is read from the hardware
+        // register, the rank inside it is the order of arrival.  256 workgroups of this size on 256 compute units
+        // put exactly XPER on every XCD; anything else is reported instead of trusted.
+        unsigned xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        xcc &= 15u;
+        unsigned rank = XPER;
+        if (xcc < XCDS && gridDim.x == XCDS * XPER) rank = __hip_atomic_fetch_add(P.xcdCount + xcc, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool bad = rank >= XPER;
+        S.ctl[0] = bad ? 1 : 0;
+        S.ctl[1] = 0;
+        S.ctl[2] = (int)xcc;
+        S.ctl[3] = (int)rank;
+        if (bad) astu(P.abortFlag, 2u);
+    }
+    lds_barrier();
+    if (uni(S.ctl[0])) return;
+    const int X = uni(S.ctl[2]), r = uni(S.ctl[3]);
+    const int tok = uni(a.tok[0]), pos = uni(a.pos[P.seq]);
+    const unsigned tagBase = *P.tagCounter; // tags never repeat from launch to launch: nothing has to be cleared
+    if (wave == XWORK) xcd_communicator<WT>(P, S, tok, pos, tagBase, X, r);
+    else xcd_worker<WT>(P, S, tok, pos, tagBase, X, r);
+}
+
+// before every launch: abort flag and per-XCD arrival counters
+__global__ void k_xcd_prep(unsigned* abortFlag, unsigned* xcdCount) {
+    if (threadIdx.x == 0) *abortFlag = 0u;
+    if (threadIdx.x < XCDS) xcdCount[threadIdx.x] = 0u;
+}
+
+__global__ void k_xcd_zero(unsigned* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// ----------------------------------------------------------------------------
+// host side
+// ----------------------------------------------------------------------------
+static size_t xcd_lds_bytes(const mlh_ctx* c) {
+    const mlh_hparams& hp = c->hp;
+    const int fs = hp.ffnDim / XCDS;
+    return ((size_t)2 * hp.dim + 5 * XNH * XHD + ((fs + 3) & ~3) + 512 + 48 + XAW * 8192) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
+}
+
+// Exchange words (64-bit) the kernel needs for this model.
+size_t mlh_xcd_words(const mlh_ctx* c) {
+    const mlh_hparams& hp = c->hp;
+    return (size_t)XCDS * (4 * XNH * XHD) + (size_t)XCDS * XNH * c->pagesPerSeq * (XHD + 2) + (size_t)4 * XCDS * hp.dim + hp.ffnDim +
+           2 * (size_t)XCDS * XPER + 64;
+}
+
+// True when the XCD-rank kernel supports this context's shape: attention layers only, head size 64, no PLE,
+// a 256-unit chip, rows that fit the register sets.
+bool mlh_xcd_supported(const mlh_ctx* c) {
+    const mlh_hparams& hp = c->hp;
+    if (c->numCUs != XCDS * XPER || !c->xcdWords) return false;
+    for (int t = 0; t < hp.transformers; t++)
+        if (hp.layerKinds[t] != MLH_KIND_ATTENTION) return false;
+    const int N = hp.weightDtype == MLH_DTYPE_BF16 ? 8 : 4;
+    if (hp.headDim != XHD || hp.pleDim != 0) return false;
+    if (hp.dim != hp.attnHeads * XHD || hp.dim > XCH * 64 * N || hp.dim % (64 * N) || hp.dim % XPER) return false;
+    if (hp.attnHeads > XCDS * XNH) return false;
+    if (hp.ffnDim % (XCDS * N)) return false;
+    if (hp.dim / 4 > 512 || hp.dim % N) return false;
+    return xcd_lds_bytes(c) <= 160 * 1024;
+}
+
+template <typename WT>
+static int launch_xcd(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+    int perCu = 0;
+    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT>, XWG, ldsBytes));
+    if (perCu < 1) { c->err = "XCD-rank decode kernel does not fit on a compute unit"; return -1; }
+    // one workgroup per compute unit, all resident at once (the occupancy query says each unit can hold one); waits are bounded
+    hipLaunchKernelGGL((k_decode_xcd<WT>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
+    MLH_CHECK(c, hipGetLastError());
+    return 0;
+}
+
+// Puts the exchange words and the tag counter back to zero (after a launch that gave up a wait).
+int mlh_xcd_reset(mlh_ctx* c) {
+    if (!c->xcdBuf) return 0;
+    const size_t words32 = c->xcdWords * 2;
+    hipLaunchKernelGGL(k_xcd_zero, dim3((unsigned)((words32 + 255) / 256)), dim3(256), 0, c->stream, (unsigned*)c->xcdBuf, words32);
+    hipLaunchKernelGGL(k_xcd_zero, dim3(1), dim3(64), 0, c->stream, c->d_sync + 64 * 21, (size_t)1);
+    MLH_CHECK(c, hipGetLastError());
+    return 0;
+}
+
+// Enqueues `steps` decode steps of sequence 0 (slot 0) in one launch of the XCD-rank kernel.
+int mlh_launch_xcd(mlh_ctx* c, int steps) {
+    const mlh_hparams& hp = c->hp;
+    XcdArgs P;
+    mlh_fill_args(c, P.a, 1, c->d_tok);
+    P.layers = c->d_layers;
+    P.NL = hp.transformers;
+    P.steps = steps;
+    P.seq = 0;
+    P.abortFlag = c->d_sync + 64 * 20;
+    P.tagCounter = c->d_sync + 64 * 21;
+    P.xcdCount = c->d_sync + 64 * 22;
+    P.maxTiles = c->pagesPerSeq;
+    P.fs = hp.ffnDim / XCDS;
+    P.timing = c->d_timing;
+    u64* t = c->xcdBuf;
+    P.qkvStride = 4 * XNH * XHD;
+    P.qkvL = t; t += (size_t)XCDS * P.qkvStride;
+    P.partStride = XNH * c->pagesPerSeq * (XHD + 2);
+    P.partL = t; t += (size_t)XCDS * P.partStride;
+    P.h1P = t; t += (size_t)XCDS * hp.dim;
+    P.h1L = t; t += (size_t)XCDS * hp.dim;
+    P.xP = t; t += (size_t)XCDS * hp.dim;
+    P.xL = t; t += (size_t)XCDS * hp.dim;
+    P.uL = t; t += hp.ffnDim;
+    P.amax = t;
+    const size_t ldsBytes = xcd_lds_bytes(c);
+    hipLaunchKernelGGL(k_xcd_prep, dim3(1), dim3(64), 0, c->stream, P.abortFlag, P.xcdCount);
+    return hp.weightDtype == MLH_DTYPE_BF16 ? launch_xcd<bf16_t>(c, P, ldsBytes) : launch_xcd<float>(c, P, ldsBytes);
+}

@@ -201,6 +201,12 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
     c->taggedWords = (size_t)2 * d + c->maxRowsA + (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2) + c->maxAd + F + 2 * (size_t)c->numCUs + 64;
     if ((rc = dev_alloc(c, &c->tagged, c->taggedWords)))
         return bail(rc);
+    c->xcdWords = mlh_xcd_words(c);
+    if ((rc = dev_alloc(c, &c->xcdBuf, c->xcdWords))) return bail(rc);
+    if (hipMemset(c->xcdBuf, 0, c->xcdWords * 8) != hipSuccess || hipMemset(c->d_sync, 0, 64 * 24 * 4) != hipSuccess) {
+        c->err = "clearing the exchange words failed";
+        return bail(-2);
+    }
     if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1)))) return bail(rc);
     c->copyBytes = (size_t)256 << 20;
     char *cs, *cd;
@@ -582,11 +588,14 @@ static void dump_persistent_timing(mlh_ctx* c) {
     const char* names[15] = {"A.norm", "A.rows", "A->B sync", "B.mix", "B->C sync", "C.prologue", "C.rows", "C->D sync",
                                     "D.norm", "D.rows", "D->E sync", "E.load", "E.rows", "E->A sync", "x.load"};
     double tot[15] = {0};
+    const bool xcd = c->usePersistent == 3 && mlh_xcd_supported(c);
     for (int l = 0; l < c->hp.transformers; l++)
-        for (int k = 0; k < 15; k++) tot[k] += (double)(t[l * 16 + k + 1] - t[l * 16 + k]) / 100.0; // 100 MHz clock
+        for (int k = 0; k < (xcd ? 5 : 15); k++) tot[k] += (double)(t[l * 16 + k + 1] - t[l * 16 + k]) / 100.0; // 100 MHz clock
     static const char* tnames[15] = {"x.wait", "A.norm", "A.rows", "B.mix", "C.wait", "C.rows", "h1.wait", "D.norm", "D.rows",
                                      "u.wait", "E.rows", "-", "-", "-", "-"};
+    static const char* xnames[15] = {"x.exchange", "A+hop", "B+hop", "C+2hops", "D+hop", "-", "-", "-", "-", "-", "-", "-", "-", "-", "-"};
     if (c->usePersistent == 2) for (int k = 0; k < 15; k++) names[k] = tnames[k];
+    if (xcd) for (int k = 0; k < 15; k++) names[k] = xnames[k];
     fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
     double sum = 0;
     for (int k = 0; k < 15; k++) { fprintf(stderr, " %s=%.2f", names[k], tot[k] / c->hp.transformers); sum += tot[k] / c->hp.transformers; }
@@ -598,7 +607,9 @@ static int check_persistent_abort(mlh_ctx* c) {
     unsigned flag = 0;
     MLH_CHECK(c, hipMemcpy(&flag, c->d_sync + 64 * 20, 4, hipMemcpyDeviceToHost));
     if (flag) {
-        c->err = "persistent decode kernel abandoned a grid-barrier wait (were all workgroups resident?)";
+        c->err = flag == 2 ? "XCD-rank decode kernel: the workgroups did not spread evenly over the XCDs"
+                           : "persistent decode kernel abandoned a wait (were all workgroups resident?)";
+        if (c->usePersistent == 3 && mlh_xcd_reset(c) == 0) (void)hipStreamSynchronize(c->stream); // tags of the abandoned launch must not be met again
         return -3;
     }
     return 0;
@@ -606,7 +617,7 @@ static int check_persistent_abort(mlh_ctx* c) {
 
 static int run_steps(mlh_ctx* c, int nseq, int steps) {
     int rc;
-    if (use_persistent(c, nseq)) return mlh_launch_persistent(c, steps);
+    if (use_persistent(c, nseq)) return (c->usePersistent == 3 && mlh_xcd_supported(c)) ? mlh_launch_xcd(c, steps) : mlh_launch_persistent(c, steps);
     if (c->graphSteps >= 1) {
         const int k = c->graphSteps;
         int done = 0;
@@ -760,10 +771,12 @@ extern "C" int mlh_set_graph(mlh_ctx* c, int stepsPerGraph) {
 
 extern "C" int mlh_set_persistent(mlh_ctx* c, int enabled) {
     if (!c) return -1;
-    if (enabled < 0 || enabled > 2) { c->err = "persistent mode must be 0, 1 or 2"; return -1; }
+    if (enabled < 0 || enabled > 3) { c->err = "persistent mode must be 0..3"; return -1; }
     c->usePersistent = enabled;
     return 0;
 }
+
+extern "C" int mlh_xcd_decode_supported(mlh_ctx* c) { return c && mlh_xcd_supported(c) ? 1 : 0; }
 
 extern "C" int mlh_synchronize(mlh_ctx* c) {
     if (!c) return -1;

@@ -122,7 +122,9 @@ struct mlh_ctx {
     // persistent batch-1 decode kernel
     int numCUs = 0;
     bool coopLaunch = false;
-    int usePersistent = 1;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange
+    int usePersistent = 1;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange; 3: XCD ranks
+    unsigned long long* xcdBuf = nullptr; // (value, tag) exchange words of mode 3
+    size_t xcdWords = 0;
     unsigned long long* tagged = nullptr; // (value, tag) exchange words of mode 2
     size_t taggedWords = 0;
     LayerDev* d_layers = nullptr;  // device copy of `layers`
@@ -197,6 +199,12 @@ int mlh_launch_softmax_rows(mlh_ctx* c, const float* logits, float* probs, const
 // kernels_persistent.hip
 bool mlh_persistent_supported(const mlh_ctx* c);
 int mlh_launch_persistent(mlh_ctx* c, int steps);
+
+// kernels_xcd.hip
+size_t mlh_xcd_words(const mlh_ctx* c);
+bool mlh_xcd_supported(const mlh_ctx* c);
+int mlh_xcd_reset(mlh_ctx* c);
+int mlh_launch_xcd(mlh_ctx* c, int steps);
 
 #define MLH_CHECK(ctx, expr)                                                               \
     do {                                                                                   \
