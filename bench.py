@@ -11,9 +11,11 @@ HBM), the roofline of the dominant kernel measured live with HIP events on the c
 whole-step bytes-per-token roofline, and the CPU baseline (PyTorch restatement of the reference's
 pytorch_verification model on this host's cores) timed on a bounded sample of the same workload.
 
-Three decode paths exist and all are timed; `value` is the one named in config.decode_path:
+Four decode paths exist and all are timed; `value` is the one named in config.decode_path:
+  xcd         one launch covers all K steps; every XCD is a tensor-parallel rank (its heads, its FFN units),
+              exchanges inside an XCD go through its L2, two per layer cross XCDs (default)
   persistent  one launch of the persistent kernel covers all K steps, phases separated by a grid barrier
-              built from agent-scope atomics (default)
+              built from agent-scope atomics
   tagged      the same kernel without barriers: consumers spin on (value, tag) words
   kernels     a sequence of per-phase kernels per step (plain launches or hipGraph replays)
 """
@@ -208,7 +210,7 @@ def main():
     ap.add_argument("--steps", type=int, default=512)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
-    ap.add_argument("--path", choices=["persistent", "kernels", "tagged"], default="persistent",
+    ap.add_argument("--path", choices=["xcd", "persistent", "kernels", "tagged"], default="xcd",
                     help="decode path reported as `value`")
     ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
     ap.add_argument("--leg", choices=["all", "batched", "prefill"], default="all",
@@ -237,10 +239,13 @@ def main():
     dev.set_graph(args.graph_steps)
 
     paths = {}
-    order = [args.path] if args.only_path else ["kernels", "persistent", "tagged"]
+    if args.path == "xcd" and not dev.xcd_decode_supported():
+        print("bench.py: the XCD-rank kernel does not cover this device; use --path persistent", file=sys.stderr)
+        return 4
+    order = [args.path] if args.only_path else ["kernels", "persistent", "tagged", "xcd"]
     ids_by_path = {}
     for name in order:
-        wall, ev_ms, ids = timed_decode(dev, prompt, K, W, {"kernels": 0, "persistent": 1, "tagged": 2}[name], hp.maxL)
+        wall, ev_ms, ids = timed_decode(dev, prompt, K, W, {"kernels": 0, "persistent": 1, "tagged": 2, "xcd": 3}[name], hp.maxL)
         paths[name] = {"tok_s": K / wall, "ms_per_step": wall / K * 1e3, "event_ms_per_step": ev_ms / K}
         ids_by_path[name] = ids[:, 0]
     if any(not np.array_equal(v, ids_by_path[args.path]) for v in ids_by_path.values()):
@@ -277,11 +282,11 @@ def main():
                          "GBps": round(algo.get(name, 0.0) / us / 1e3, 1) if us > 0 else None}
     copy_us, copy_bytes = dev.time_kernel(m.K_COPY, iters=20)
 
-    if args.path in ("persistent", "tagged"):
+    if args.path in ("persistent", "tagged", "xcd"):
         # the dominant (only) kernel: one launch = K tokens; duration from HIP events around the launch
         launch_us = chosen["event_ms_per_step"] * K * 1e3
         launch_bytes = mean_bytes * K
-        roofline = {"kernel": "k_decode_persistent" if args.path == "persistent" else "k_decode_tagged", "bound": "hbm", "achieved": launch_bytes / launch_us / 1e3,
+        roofline = {"kernel": {"persistent": "k_decode_persistent", "tagged": "k_decode_tagged", "xcd": "k_decode_xcd"}[args.path], "bound": "hbm", "achieved": launch_bytes / launch_us / 1e3,
                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": launch_bytes / launch_us / 1e3 / HBM_PEAK_GBPS,
                     "traffic": None, "avg_launch_us": launch_us, "algo_bytes_per_launch": launch_bytes,
                     "tokens_per_launch": K}

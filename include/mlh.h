@@ -174,7 +174,7 @@ int mlh_read_probs(mlh_ctx* ctx, int seq, float* out);
  * of a captured hipGraph that covers k consecutive decode steps (at most 64). */
 int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
 
-/* Batch-1 decode (nseq = 1): mode 1 (default) runs, when the shape allows it, as ONE launch of a
+/* Batch-1 decode (nseq = 1): mode 1 runs, when the shape allows it, as ONE launch of a
  * persistent kernel (one workgroup per compute unit) that decodes all requested steps: the ~60
  * dependent phases of a token are separated by grid barriers instead of kernel launches.  Mode 2 is
  * the same kernel without barriers (consumers spin on tagged data words).  Both need every compute
@@ -183,7 +183,7 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
  * Mode 3 treats each of the eight XCDs as a tensor-parallel rank (heads and FFN units are split over the
  * XCDs, exchanges inside an XCD go through its L2, only two per layer cross XCDs); it covers models of
  * attention layers with head size 64 and no per-layer embeddings on a 256-unit device
- * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise. */
+ * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default. */
 int mlh_set_persistent(mlh_ctx* ctx, int mode);
 
 /* 1 when mode 3 of mlh_set_persistent applies to this context's model and device, else 0

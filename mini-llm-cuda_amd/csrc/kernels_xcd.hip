@@ -43,7 +43,7 @@
 #define XLW (XWORK * XPER)      // worker waves per XCD
 #define XNH 4                   // heads per XCD at most
 #define XAW 2                   // worker waves of a workgroup that take attention units
-#define XCH 4                   // 16-byte chunks per lane of a full-width row kept in registers
+#define XCB 24                  // softmax partials the communicator fetches per round
 #define XSPIN (1u << 20)
 #define XHD 64
 
@@ -79,71 +79,6 @@ __device__ __forceinline__ u64 xld(const u64* p) { return __hip_atomic_load(p, _
 __device__ __forceinline__ void lst(u64* p, float v, unsigned tag) { __hip_atomic_store(p, xpack(v, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
 __device__ __forceinline__ u64 lld(const u64* p) { return __builtin_nontemporal_load(p); }
 
-// One wave fetches n tagged words into LDS, NB loads per lane in flight, reading again until every tag is there.
-template <bool CROSS, int NB>
-__device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, float* dst, const unsigned* abortFlag, bool& ok) {
-    const int lane = threadIdx.x & 63;
-    for (int base = 0; base < n; base += 64 * NB) {
-        u64 w[NB];
-        for (unsigned spins = 0;; spins++) {
-            asm volatile("" ::: "memory"); // the loads below are repeated every round
-            bool all = true;
-#pragma unroll
-            for (int k = 0; k < NB; k++) {
-                const int i = base + k * 64 + lane;
-                const u64* p = src + (i < n ? i : n - 1);
-                w[k] = CROSS ? xld(p) : lld(p);
-                all = all && (unsigned)(w[k] >> 32) == tag;
-            }
-            if (all) break;
-            if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(abortFlag))) { ok = false; break; }
-        }
-#pragma unroll
-        for (int k = 0; k < NB; k++) {
-            const int i = base + k * 64 + lane;
-            if (i < n) dst[i] = __uint_as_float((unsigned)w[k]);
-        }
-    }
-}
-
-// Sum of the eight XCDs' partials over this workgroup's slice [s0, s0 + sl) plus the residual, published inside
-// the XCD; then the whole vector is fetched from the XCD's 32 slices.  have[X'] false: that XCD contributes nothing.
-__device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int s0, int sl, unsigned tag, unsigned haveMask,
-                                                     const float* resid, float* scratch, u64* pub, float* dst,
-                                                     const unsigned* abortFlag, bool& ok) {
-    const int lane = threadIdx.x & 63;
-    const int n = XCDS * sl;
-    constexpr int NB = 8;
-    u64 w[NB];
-    for (unsigned spins = 0;; spins++) {
-        asm volatile("" ::: "memory");
-        bool all = true;
-#pragma unroll
-        for (int k = 0; k < NB; k++) {
-            const int i = k * 64 + lane;
-            const int xc = i / sl, e = i - xc * sl;
-            const bool need = i < n && ((haveMask >> xc) & 1u);
-            w[k] = need ? xld(part + (size_t)xc * d + s0 + e) : ((u64)tag << 32);
-            all = all && (unsigned)(w[k] >> 32) == tag;
-        }
-        if (all) break;
-        if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(abortFlag))) { ok = false; break; }
-    }
-#pragma unroll
-    for (int k = 0; k < NB; k++) {
-        const int i = k * 64 + lane;
-        if (i < n) scratch[i] = __uint_as_float((unsigned)w[k]);
-    }
-    __builtin_amdgcn_wave_barrier();
-    for (int e = lane; e < sl; e += 64) {
-        float s = 0.f;
-#pragma unroll
-        for (int xc = 0; xc < XCDS; xc++) s += scratch[xc * sl + e]; // fixed order: the result does not depend on timing
-        lst(pub + s0 + e, s + resid[s0 + e], tag);
-    }
-    poll_vec<false, 8>(pub, d, tag, dst, abortFlag, ok);
-}
-
 // Values that are the same in every lane of a wave, said so to the compiler: address arithmetic on them is then
 // done once per wave on the scalar unit, and loads take the form scalar base + 32-bit lane offset.
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -154,9 +89,120 @@ __device__ __forceinline__ T* uni_ptr(T* p) { // p points into global memory (th
     return (T*)(__attribute__((address_space(1))) T*)u;
 }
 
-template <typename WT, int NR> struct XRows { typename PVec<WT>::Raw r[NR * XCH]; }; // NR full-width rows
+// Pins a wave-uniform pointer in scalar registers as an opaque value: without this the optimiser re-associates
+// (base + row offset) + lane offset into (base + lane offset) + row offset, hoists the per-lane part out of the loops
+// and ends up with one 64-bit vector address per load site, held in registers across the whole kernel.
+template <typename T>
+__device__ __forceinline__ const T* pin_uniform(const T* p) { // p: wave-uniform, into global memory
+    u64 v = (u64)p;
+    asm("" : "+s"(v));
+    return (const T*)(__attribute__((address_space(1))) const T*)v;
+}
+
+// One tagged word at (wave-uniform base) + lane offset + constant, both in bytes (scalar base, one offset register).
+template <bool CROSS>
+__device__ __forceinline__ u64 ldw(const u64* base, unsigned laneBytes, unsigned constBytes) {
+    asm volatile("" : "+v"(laneBytes));
+    const u64* p = reinterpret_cast<const u64*>(reinterpret_cast<const char*>(base) + (size_t)laneBytes + constBytes);
+    return CROSS ? xld(p) : lld(p);
+}
+
+// One wave fetches n tagged words into LDS, NB loads per lane and round, reading again until every tag is there.
+// With PIPE two rounds are in flight, a fraction of a round trip apart: the answer to a round that just missed the
+// data is followed closely by the next one instead of by a whole new round trip.  All 64 lanes take part.
+template <bool CROSS, int NB, bool PIPE>
+__device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, float* dst, const unsigned* abortFlag, bool& ok) {
+    const int lane = threadIdx.x & 63;
+    for (int base = 0; base < n; base += 64 * NB) {
+        u64 wA[NB], wB[NB];
+        auto issue = [&](u64 (&w)[NB]) {
+            asm volatile("" ::: "memory"); // the loads are repeated every round
+#pragma unroll
+            for (int k = 0; k < NB; k++) {
+                const int i0 = base + k * 64; // wave-uniform
+                if (i0 < n) w[k] = ldw<CROSS>(pin_uniform(src + i0), (unsigned)min(lane, n - 1 - i0) * 8u, 0u);
+                else w[k] = (u64)tag << 32;
+            }
+        };
+        auto good = [&](const u64 (&w)[NB]) {
+            bool all = true;
+#pragma unroll
+            for (int k = 0; k < NB; k++) all = all && (unsigned)(w[k] >> 32) == tag;
+            return __all(all) != 0;
+        };
+        auto keep = [&](const u64 (&w)[NB]) {
+#pragma unroll
+            for (int k = 0; k < NB; k++) {
+                const int i = base + k * 64 + lane;
+                if (i < n) dst[i] = __uint_as_float((unsigned)w[k]);
+            }
+        };
+        issue(wA);
+        for (unsigned spins = 0;; spins++) {
+            if (PIPE) {
+                __builtin_amdgcn_s_sleep(CROSS ? 8 : 3);
+                issue(wB);
+            }
+            if (good(wA)) { keep(wA); break; }
+            if (PIPE) __builtin_amdgcn_s_sleep(CROSS ? 8 : 3);
+            issue(wA);
+            if (PIPE && good(wB)) { keep(wB); break; }
+            if (!ok || spins > XSPIN || ((spins & 127) == 127 && aldu(abortFlag))) { ok = false; break; }
+        }
+    }
+}
+
+// Sum of the eight XCDs' partials over this workgroup's slice [s0, s0 + sl) (sl <= 64) plus the residual, published
+// inside the XCD; then the whole vector is fetched from the XCD's 32 slices.  haveMask bit X' clear: that XCD
+// contributes nothing.
+__device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int s0, int sl, unsigned tag, unsigned haveMask,
+                                                     const float* resid, float* scratch, u64* pub, float* dst,
+                                                     const unsigned* abortFlag, bool& ok, u64* stamp = nullptr) {
+    const int lane = threadIdx.x & 63;
+    const unsigned lb = (unsigned)min(lane, sl - 1) * 8u;
+    u64 wA[XCDS], wB[XCDS];
+    auto issue = [&](u64 (&w)[XCDS]) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int xc = 0; xc < XCDS; xc++) {
+            if ((haveMask >> xc) & 1u) w[xc] = ldw<true>(pin_uniform(part + (size_t)xc * d + s0), lb, 0u);
+            else w[xc] = (u64)tag << 32;
+        }
+    };
+    auto good = [&](const u64 (&w)[XCDS]) {
+        bool all = true;
+#pragma unroll
+        for (int xc = 0; xc < XCDS; xc++) all = all && (unsigned)(w[xc] >> 32) == tag;
+        return __all(all) != 0;
+    };
+    auto total = [&](const u64 (&w)[XCDS]) { // fixed order: the result does not depend on timing
+        float t = 0.f;
+#pragma unroll
+        for (int xc = 0; xc < XCDS; xc++) t += __uint_as_float((unsigned)w[xc]);
+        return t;
+    };
+    float sum = 0.f;
+    issue(wA);
+    for (unsigned spins = 0;; spins++) {
+        __builtin_amdgcn_s_sleep(8);
+        issue(wB);
+        if (good(wA)) { sum = total(wA); break; }
+        __builtin_amdgcn_s_sleep(8);
+        issue(wA);
+        if (good(wB)) { sum = total(wB); break; }
+        if (!ok || spins > XSPIN || ((spins & 127) == 127 && aldu(abortFlag))) { ok = false; break; }
+    }
+    if (stamp && lane == 0) stamp[0] = wall_clock64();
+    if (lane < sl) lst(pub + s0 + lane, sum + resid[s0 + lane], tag);
+    if (stamp && lane == 0) stamp[1] = wall_clock64();
+    poll_vec<false, 16, false>(pub, d, tag, dst, abortFlag, ok);
+    (void)scratch;
+}
+
+// NCH (template parameter of the kernel): 16-byte chunks per lane of a full-width row, dim / (64 N)
+template <typename WT, int NR, int NCH> struct XRows { typename PVec<WT>::Raw r[NR * NCH]; }; // NR full-width rows
 template <typename WT> struct XPf { typename PVec<WT>::Raw r[8]; };
-template <typename WT> struct XGain { f32x4 g[XCH][PVec<WT>::N / 4]; };
+template <typename WT, int NCH> struct XGain { f32x4 g[NCH][PVec<WT>::N / 4]; };
 
 // weights (16 bytes) times N activations in registers
 template <typename WT>
@@ -183,16 +229,6 @@ __device__ __forceinline__ float chunk_dot_lds(const typename PVec<WT>::Raw& w, 
     return acc;
 }
 
-// Pins a wave-uniform pointer in scalar registers as an opaque value: without this the optimiser re-associates
-// (base + row offset) + lane offset into (base + lane offset) + row offset, hoists the per-lane part out of the loops
-// and ends up with one 64-bit vector address per load site, held in registers across the whole kernel.
-template <typename T>
-__device__ __forceinline__ const T* pin_uniform(const T* p) { // p: wave-uniform, into global memory
-    u64 v = (u64)p;
-    asm("" : "+s"(v));
-    return (const T*)(__attribute__((address_space(1))) const T*)v;
-}
-
 // 16 bytes at (wave-uniform base) + (32-bit lane offset in bytes) + constant: the addressing mode that needs no
 // 64-bit arithmetic per lane (scalar base register + one offset register + immediate).
 // (The empty statement keeps the widening of the lane offset next to the load: instruction selection works block by
@@ -207,79 +243,71 @@ __device__ __forceinline__ f32x4 load16f(const void* base, unsigned laneBytes, u
     return *reinterpret_cast<const f32x4*>(reinterpret_cast<const char*>(base) + (size_t)laneBytes + constBytes);
 }
 
-// NR full-width rows (wave-uniform indices; < 0: none) of the wave-uniform matrix W go into registers: lane l holds
-// columns (ch 64 + l) N .. + N of every row, ch < nch.  Registers of absent rows and chunks keep what they held.
-template <typename WT, int NR>
-__device__ __forceinline__ void issue_rows(typename PVec<WT>::Raw (&dst)[NR * XCH], const WT* W, size_t ld, const int (&rows)[NR], int nch) {
+// NR full-width rows (wave-uniform, valid indices) of the wave-uniform matrix W go into registers: lane l holds
+// columns (ch 64 + l) N .. + N of every row.  Every register is assigned on every call (callers clamp indices
+// instead of skipping loads), so nothing of an earlier phase stays live in them.
+template <typename WT, int NR, int NCH>
+__device__ __forceinline__ void issue_rows(typename PVec<WT>::Raw (&dst)[NR * NCH], const WT* W, size_t ld, const int (&rows)[NR]) {
     const unsigned lb = (threadIdx.x & 63u) * 16u;
 #pragma unroll
-    for (int k = 0; k < NR; k++)
-        if (rows[k] >= 0) {
-            const WT* rp = pin_uniform(W + (size_t)rows[k] * ld);
+    for (int k = 0; k < NR; k++) {
+        const WT* rp = pin_uniform(W + (size_t)rows[k] * ld);
 #pragma unroll
-            for (int ch = 0; ch < XCH; ch++)
-                if (ch < nch) dst[k * XCH + ch] = load16<WT>(rp, lb, ch * 1024u);
-        }
+        for (int ch = 0; ch < NCH; ch++) dst[k * NCH + ch] = load16<WT>(rp, lb, ch * 1024u);
+    }
 }
-template <typename WT>
-__device__ __forceinline__ void issue_gain(XGain<WT>& gn, const float* gain, int nch) {
+template <typename WT, int NCH>
+__device__ __forceinline__ void issue_gain(XGain<WT, NCH>& gn, const float* gain) {
     constexpr int N = PVec<WT>::N;
     const unsigned lb = (threadIdx.x & 63u) * (N * 4u);
     gain = pin_uniform(gain);
 #pragma unroll
-    for (int ch = 0; ch < XCH; ch++)
-        if (ch < nch)
+    for (int ch = 0; ch < NCH; ch++)
 #pragma unroll
-            for (int q = 0; q < N / 4; q++) gn.g[ch][q] = load16f(gain, lb, ch * 64u * N * 4u + q * 16u);
+        for (int q = 0; q < N / 4; q++) gn.g[ch][q] = load16f(gain, lb, ch * 64u * N * 4u + q * 16u);
 }
 
 // xn = gain * (src / sqrt(mean(src^2) + 1e-8)) for this lane's columns (inference.cu:24-50, 83-95); every wave
 // computes the mean itself from the vector in LDS, so no workgroup reduction is needed.
-template <typename WT>
-__device__ __forceinline__ void normed_columns(const float* src, const XGain<WT>& gn, int d, int nch, float (&xn)[XCH][PVec<WT>::N]) {
+template <typename WT, int NCH>
+__device__ __forceinline__ void normed_columns(const float* src, const XGain<WT, NCH>& gn, int d, float (&xn)[NCH][PVec<WT>::N]) {
     constexpr int N = PVec<WT>::N;
     const int c0 = (threadIdx.x & 63) * N;
     float ss = 0.f;
 #pragma unroll
-    for (int ch = 0; ch < XCH; ch++)
-        if (ch < nch) {
+    for (int ch = 0; ch < NCH; ch++)
 #pragma unroll
-            for (int q = 0; q < N / 4; q++) {
-                const f32x4 v = *reinterpret_cast<const f32x4*>(src + ch * 64 * N + c0 + 4 * q);
-                xn[ch][4 * q] = v.x; xn[ch][4 * q + 1] = v.y; xn[ch][4 * q + 2] = v.z; xn[ch][4 * q + 3] = v.w;
-                ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
-            }
+        for (int q = 0; q < N / 4; q++) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(src + ch * 64 * N + c0 + 4 * q);
+            xn[ch][4 * q] = v.x; xn[ch][4 * q + 1] = v.y; xn[ch][4 * q + 2] = v.z; xn[ch][4 * q + 3] = v.w;
+            ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
         }
     ss = pwave_sum(ss);
-    const float r = sqrtf(ss / (float)d + 1e-8f);
+    const float ri = 1.0f / sqrtf(ss / (float)d + 1e-8f); // one division per wave; the elements are multiplied
 #pragma unroll
-    for (int ch = 0; ch < XCH; ch++)
-        if (ch < nch) {
+    for (int ch = 0; ch < NCH; ch++)
 #pragma unroll
-            for (int q = 0; q < N / 4; q++) {
-                const f32x4 g = gn.g[ch][q];
-                xn[ch][4 * q] = g.x * (xn[ch][4 * q] / r); xn[ch][4 * q + 1] = g.y * (xn[ch][4 * q + 1] / r);
-                xn[ch][4 * q + 2] = g.z * (xn[ch][4 * q + 2] / r); xn[ch][4 * q + 3] = g.w * (xn[ch][4 * q + 3] / r);
-            }
+        for (int q = 0; q < N / 4; q++) {
+            const f32x4 g = gn.g[ch][q];
+            xn[ch][4 * q] = g.x * (xn[ch][4 * q] * ri); xn[ch][4 * q + 1] = g.y * (xn[ch][4 * q + 1] * ri);
+            xn[ch][4 * q + 2] = g.z * (xn[ch][4 * q + 2] * ri); xn[ch][4 * q + 3] = g.w * (xn[ch][4 * q + 3] * ri);
         }
 }
 
-template <typename WT, int NRAW>
-__device__ __forceinline__ float row_dot_reg(const typename PVec<WT>::Raw (&r)[NRAW], int which, int nch, const float (&xn)[XCH][PVec<WT>::N]) {
+template <typename WT, int NCH, int NRAW>
+__device__ __forceinline__ float row_dot_reg(const typename PVec<WT>::Raw (&r)[NRAW], int which, const float (&xn)[NCH][PVec<WT>::N]) {
     float acc = 0.f;
 #pragma unroll
-    for (int ch = 0; ch < XCH; ch++)
-        if (ch < nch) acc = chunk_dot_reg<WT>(r[which * XCH + ch], xn[ch], acc);
+    for (int ch = 0; ch < NCH; ch++) acc = chunk_dot_reg<WT>(r[which * NCH + ch], xn[ch], acc);
     return acc;
 }
-template <typename WT>
-__device__ __forceinline__ float row_dot_stream(const WT* W, size_t ld, int row, int nch, const float (&xn)[XCH][PVec<WT>::N]) {
+template <typename WT, int NCH>
+__device__ __forceinline__ float row_dot_stream(const WT* W, size_t ld, int row, const float (&xn)[NCH][PVec<WT>::N]) {
     const WT* rp = pin_uniform(W + (size_t)row * ld);
     const unsigned lb = (threadIdx.x & 63u) * 16u;
     float acc = 0.f;
 #pragma unroll
-    for (int ch = 0; ch < XCH; ch++)
-        if (ch < nch) acc = chunk_dot_reg<WT>(load16<WT>(rp, lb, ch * 1024u), xn[ch], acc);
+    for (int ch = 0; ch < NCH; ch++) acc = chunk_dot_reg<WT>(load16<WT>(rp, lb, ch * 1024u), xn[ch], acc);
     return acc;
 }
 
@@ -290,35 +318,35 @@ __device__ __forceinline__ int rowA_of(int offK, int offV, int offG, int X, int 
     return off + (X + XCDS * j) * XHD + i;
 }
 
-// Wo columns of the XCD's heads: a pass covers N rows per wave (64/N lanes per 64-column head segment).
+// Wo columns of the XCD's heads: a pass covers N rows per wave (64/N lanes per 64-column head segment).  Rows
+// and heads beyond the end are clamped to the last valid one (loaded, never used).
 template <typename WT>
-__device__ __forceinline__ void issue_wo(XPf<WT>& pf, const WT* Wo, int ad, int X, int nh, int lw, int d) {
+__device__ __forceinline__ void issue_wo(XPf<WT>& pf, const WT* Wo, int ad, int X, int nh, int heads, int lw, int d) {
     constexpr int N = PVec<WT>::N, CPS = XHD / N;
     const unsigned lane = threadIdx.x & 63u;
     const unsigned lb = ((lane / CPS) * (unsigned)ad + (lane % CPS) * N) * (unsigned)sizeof(WT); // row within the pass, chunk within the head segment
 #pragma unroll
-    for (int p = 0; p < 2; p++)
-        if ((p * XLW + lw) * N < d) {
-            const WT* rp = pin_uniform(Wo + (size_t)((p * XLW + lw) * N) * ad + X * XHD);
+    for (int p = 0; p < 2; p++) {
+        const int rb = min((p * XLW + lw) * N, d - N);
 #pragma unroll
-            for (int j = 0; j < XNH; j++)
-                if (j < nh) pf.r[p * XNH + j] = load16<WT>(rp, lb, j * XCDS * XHD * (unsigned)sizeof(WT));
+        for (int j = 0; j < XNH; j++) {
+            const int h = min(X + XCDS * min(j, max(nh, 1) - 1), heads - 1);
+            pf.r[p * XNH + j] = load16<WT>(pin_uniform(Wo + (size_t)rb * ad + h * XHD), lb, 0u);
         }
+    }
 }
-// W2 columns [X fs, (X+1) fs): rows lw, lw + XLW, ...; four rows x two chunks per lane are prefetched.
+// W2 columns [X fs, (X+1) fs): rows lw, lw + XLW, ...; four rows x two chunks per lane are prefetched (clamped likewise).
 template <typename WT>
 __device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int fs, int F, int lw, int d) {
     constexpr int N = PVec<WT>::N;
     const int lane = threadIdx.x & 63, CR = fs / N;
-    const unsigned lb = (threadIdx.x & 63u) * 16u;
+    const unsigned lb0 = (unsigned)min(lane, CR - 1) * 16u, lb1 = (unsigned)min(lane + 64, CR - 1) * 16u;
 #pragma unroll
-    for (int k = 0; k < 4; k++)
-        if (lw + XLW * k < d) {
-            const WT* rp = pin_uniform(W2 + (size_t)(lw + XLW * k) * F + (size_t)X * fs);
-#pragma unroll
-            for (int c0 = 0; c0 < 2; c0++)
-                if (lane + 64 * c0 < CR) pf.r[k * 2 + c0] = load16<WT>(rp, lb, c0 * 1024u);
-        }
+    for (int k = 0; k < 4; k++) {
+        const WT* rp = pin_uniform(W2 + (size_t)min(lw + XLW * k, d - 1) * F + (size_t)X * fs);
+        pf.r[k * 2] = load16<WT>(rp, lb0, 0u);
+        pf.r[k * 2 + 1] = load16<WT>(rp, lb1, 0u);
+    }
 }
 
 // K and V tile (64 rows x 64 floats each) of one head, rows below `lim`, global -> LDS without registers.  An
@@ -393,14 +421,15 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
                 for (int j = 0; j < XNH; j++)
                     if (j < nh) { gq[j] = uni_ptr(L.gq)[(X + XCDS * j) * XHD + lane]; gk[j] = uni_ptr(L.gk)[(X + XCDS * j) * XHD + lane]; }
             if (t != P.NL - 1) // partial x of the layer below, all XCDs, + its residual h1
-                reduce_publish_fetch(P.xP, d, s0, sl, lt - 1, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok);
+                reduce_publish_fetch(P.xP, d, s0, sl, lt - 1, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok,
+                                     (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 6 : nullptr);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 1);
             X_BARRIER(); // 1: x in LDS
 
             // q | k | v | gate of the XCD's heads; per-head RMSNorm (inference.cu:52-81, 97-111), RoPE on adjacent
             // pairs (inference.cu:113-134); workgroup 0 of the XCD appends the new K/V rows to the cache
-            poll_vec<false, 8>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok);
+            poll_vec<false, 8, false>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok);
             {
                 float* qs = S.qkvs;
                 float* ks = qs + nh * XHD;
@@ -432,68 +461,82 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             X_STAMP(ts + 2);
             X_BARRIER(); // 2: q, k, v, gate in LDS
 
+            // diagnostic: every workgroup's clock at points of the last layer pass (skew between workgroups)
+            u64* skew = (P.timing && t == 0 && step == P.steps - 1) ? P.timing + 16 * (P.NL + 1) + 4 * wg : nullptr;
             // softmax partials of the XCD's heads -> mixing output (lane = dimension), gate (inference.cu:241-250)
             {
                 const int U = nh * ntiles;
                 const float* gs = S.qkvs + 3 * nh * XHD;
                 float M = -1.0e30f, num = 0.f, den = 0.f;
                 int cur = 0;
-                for (int u0 = 0; u0 < U; u0 += 16) {
-                    u64 wa[16], wml;
+                int tlc = 0; // tiles of the current head already taken in
+                // One wave does this for the whole workgroup, so instructions count: the weights exp(m - M) of all
+                // units of a batch are formed at once (lane = unit); per unit only a broadcast and a multiply-add remain.
+                for (int u0 = 0; u0 < U; u0 += XCB) {
+                    u64 wa[XCB], wm, wl;
+                    const u64* ub = pin_uniform(partL + (size_t)u0 * (XHD + 2));
+                    const unsigned uOff = (unsigned)(min(u0 + (lane & 31), U - 1) - u0) * ((XHD + 2) * 8u);
                     for (unsigned spins = 0;; spins++) {
                         asm volatile("" ::: "memory");
                         bool all = true;
 #pragma unroll
-                        for (int k = 0; k < 16; k++) {
-                            const int u = u0 + k < U ? u0 + k : U - 1, j = u / ntiles, tl = u - j * ntiles;
-                            wa[k] = lld(partL + ((size_t)j * P.maxTiles + tl) * (XHD + 2) + lane);
+                        for (int k = 0; k < XCB; k++) {
+                            if (u0 + k < U) wa[k] = ldw<false>(ub, (unsigned)lane * 8u, k * ((XHD + 2) * 8u));
+                            else wa[k] = (u64)lt << 32;
                             all = all && (unsigned)(wa[k] >> 32) == lt;
                         }
-                        {   // lanes 0..15: running maxima of the 16 units, lanes 16..31: their sums
-                            const int k = lane & 15, u = u0 + k < U ? u0 + k : U - 1, j = u / ntiles, tl = u - j * ntiles;
-                            wml = lld(partL + ((size_t)j * P.maxTiles + tl) * (XHD + 2) + XHD + ((lane >> 4) & 1));
-                            all = all && (unsigned)(wml >> 32) == lt;
-                        }
+                        wm = ldw<false>(ub, uOff, XHD * 8u);       // lane k < 32: running maximum of unit u0 + k
+                        wl = ldw<false>(ub, uOff, (XHD + 1) * 8u); //              and its sum of exponentials
+                        all = all && (unsigned)(wm >> 32) == lt && (unsigned)(wl >> 32) == lt;
                         if (__all(all)) break;
                         if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(P.abortFlag))) { ok = false; break; }
                     }
-                    const float ml = __uint_as_float((unsigned)wml);
+                    if (skew && lane == 0 && u0 == 0) skew[2] = wall_clock64();
+                    const float mk = __uint_as_float((unsigned)wm), lk = __uint_as_float((unsigned)wl);
+                    const int nb = U - u0 < XCB ? U - u0 : XCB;
+                    for (int k0 = 0; k0 < nb;) { // the heads that have units in this batch, one after the other
+                        const int take = nb - k0 < ntiles - tlc ? nb - k0 : ntiles - tlc;
+                        const bool mine = lane >= k0 && lane < k0 + take;
+                        // (a single wave issues one instruction every four cycles, whatever its kind: the hardware
+                        // exponential and reciprocal, and no branches around the units of other heads -- their
+                        // weight is zero)
+                        const float Mn = fmaxf(M, pwave_max(mine ? mk : -1.0e30f));
+                        const float corr = __expf(M - Mn);
+                        const float w = mine ? __expf(mk - Mn) : 0.f;
+                        den = fmaf(den, corr, pwave_sum(w * lk));
+                        num *= corr;
 #pragma unroll
-                    for (int k = 0; k < 16; k++) {
-                        if (u0 + k < U) {
-                            const int j = (u0 + k) / ntiles;
-                            if (j != cur) {
-                                float v = num / den;
-                                if (a.gating) v = v * psigmoid(gs[cur * XHD + lane]);
-                                S.as[cur * XHD + lane] = v;
-                                cur = j; M = -1.0e30f; num = 0.f; den = 0.f;
+                        for (int k8 = 0; k8 < XCB; k8 += 8)
+                            if (k8 < nb) {
+#pragma unroll
+                                for (int k = k8; k < k8 + 8; k++)
+                                    num = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k)), __uint_as_float((unsigned)wa[k]), num);
                             }
-                            const float mk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ml), k));
-                            const float lk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ml), 16 + k));
-                            const float Mn = fmaxf(M, mk), corr = expf(M - Mn), w = expf(mk - Mn);
-                            num = fmaf(w, __uint_as_float((unsigned)wa[k]), num * corr);
-                            den = fmaf(w, lk, den * corr);
-                            M = Mn;
+                        M = Mn;
+                        tlc += take;
+                        k0 += take;
+                        if (tlc == ntiles) { // the head is complete
+                            float v = num * __builtin_amdgcn_rcpf(den);
+                            if (a.gating) v = v * __builtin_amdgcn_rcpf(1.0f + __expf(-gs[cur * XHD + lane])); // inference.cu:248
+                            S.as[cur * XHD + lane] = v;
+                            cur++; tlc = 0; M = -1.0e30f; num = 0.f; den = 0.f;
                         }
                     }
-                }
-                if (U > 0) {
-                    float v = num / den;
-                    if (a.gating) v = v * psigmoid(gs[cur * XHD + lane]);
-                    S.as[cur * XHD + lane] = v;
                 }
             }
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 3);
+            if (skew && lane == 0) skew[3] = wall_clock64();
             X_BARRIER(); // 3: mixing output of the XCD's heads in LDS
 
             // h1 = x + sum of the XCDs' Wo partials (inference.cu:252-260)
-            reduce_publish_fetch(P.h1P, d, s0, sl, lt, headMask, S.xs, S.scratch, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok);
+            reduce_publish_fetch(P.h1P, d, s0, sl, lt, headMask, S.xs, S.scratch, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok,
+                                 (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 8 : nullptr);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 4);
             X_BARRIER(); // 4: h1 in LDS
 
-            poll_vec<false, 8>(P.uL + (size_t)X * P.fs, P.fs, lt, S.us, P.abortFlag, ok);
+            poll_vec<false, 8, false>(P.uL + (size_t)X * P.fs, P.fs, lt, S.us, P.abortFlag, ok);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 5);
             X_BARRIER(); // 5: the XCD's FFN activations in LDS
@@ -518,7 +561,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
                 xst(P.amax + 2 * wg, v, tagBase + (unsigned)step + 1);
                 xst(P.amax + 2 * wg + 1, __uint_as_float((unsigned)i), tagBase + (unsigned)step + 1);
             }
-            poll_vec<true, 8>(P.amax, 2 * (int)gridDim.x, tagBase + (unsigned)step + 1, S.scratch, P.abortFlag, ok);
+            poll_vec<true, 8, true>(P.amax, 2 * (int)gridDim.x, tagBase + (unsigned)step + 1, S.scratch, P.abortFlag, ok);
             v = -3.0e38f; i = 0x7fffffff;
             for (int k = lane; k < (int)gridDim.x; k += 64) {
                 const float v2 = S.scratch[2 * k];
@@ -555,12 +598,11 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
 }
 
 // ------------------------------------------------------------------------------------------------ workers
-template <typename WT>
+template <typename WT, int NCH>
 __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
     constexpr int N = PVec<WT>::N, CPS = XHD / N;
     const StepArgs& a = P.a;
     const int d = a.dim, F = a.ffn, V = a.vocab, fs = P.fs;
-    const int nch = d / (64 * N); // 16-byte chunks per lane of a full-width row
     const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6), wg = blockIdx.x;
     const int lw = wave * XPER + r;             // worker wave within the XCD: consecutive rows land on different workgroups
     const int gwl = wave * (int)gridDim.x + wg; // worker wave within the grid (LM head)
@@ -575,17 +617,17 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     const int aslot = wave * XPER + r; // attention unit slot of this wave (waves below XAW only)
     const WT* E = (const WT*)a.E;
 
-    XRows<WT, XS1> s1; // rows of phases A / D / LM head
+    XRows<WT, XS1, NCH> s1; // rows of phases A / D / LM head
     XPf<WT> s2;      // rows of phases C / E / LM head
-    XGain<WT> gn;
+    XGain<WT, NCH> gn;
     // first-phase rows lw, lw + XLW, ... of layer Lx and its first gain vector
     auto issueA = [&](const LayerDev& Lx) {
         const int offK = uni(Lx.offK), offV = uni(Lx.offV), offG = uni(Lx.offG);
         int rows[XS1];
 #pragma unroll
-        for (int k = 0; k < XS1; k++) rows[k] = lw + XLW * k < RA ? rowA_of(offK, offV, offG, X, nh, lw + XLW * k) : -1;
-        issue_rows<WT, XS1>(s1.r, uni_ptr((const WT*)Lx.Wa), d, rows, nch);
-        issue_gain<WT>(gn, uni_ptr(Lx.g1), nch);
+        for (int k = 0; k < XS1; k++) rows[k] = nh > 0 ? rowA_of(offK, offV, offG, X, nh, min(lw + XLW * k, RA - 1)) : 0;
+        issue_rows<WT, XS1, NCH>(s1.r, uni_ptr((const WT*)Lx.Wa), d, rows);
+        issue_gain<WT, NCH>(gn, uni_ptr(Lx.g1));
     };
     // first K/V tile of this wave in layer Lx when the sequence holds npos rows
     auto issueKV = [&](const LayerDev& Lx, int npos) {
@@ -597,10 +639,14 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             issue_kv_tile(uni_ptr((const float*)Lx.K) + base, uni_ptr((const float*)Lx.V) + base, d, npos - tl * 64, tK, tV);
         }
     };
+    if (wave < XAW) { // the tiles must never hold anything but finite numbers (rows beyond the sequence get weight zero)
+        for (int i = lane * 4; i < 8192; i += 256) *reinterpret_cast<f32x4*>(tK + i) = (f32x4)(0.f);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
     {
         const LayerDev& L0 = S.Ls[P.NL - 1];
         issueA(L0);
-        issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, lw, d);
+        issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
         if (wave < XAW) issueKV(L0, pos);
     }
 
@@ -612,15 +658,19 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             const bool lastLayer = t == 0;
             const LayerDev& Ln = S.Ls[lastLayer ? P.NL - 1 : t - 1];
             X_BARRIER(); // 1
+            const int ts = (P.NL - 1 - t) * 16;
+            const bool stampW = P.timing && wg == 0 && wave == 0 && lane == 0 && step == P.steps - 1;
+#define W_STAMP(slot) do { if (stampW) P.timing[ts + (slot)] = wall_clock64(); } while (0)
+            W_STAMP(10);
             // ------------------------------------------------------------------ phase A
             {
-                float xn[XCH][N];
-                normed_columns<WT>(S.xs, gn, d, nch, xn);
+                float xn[NCH][N];
+                normed_columns<WT, NCH>(S.xs, gn, d, xn);
 #pragma unroll
                 for (int k = 0; k < XS1; k++) {
                     const int rho = lw + XLW * k;
                     if (rho < RA) {
-                        const float acc = pwave_sum(row_dot_reg<WT>(s1.r, k, nch, xn));
+                        const float acc = pwave_sum(row_dot_reg<WT, NCH>(s1.r, k, xn));
                         if (lane == 0) lst(qkvL + rho, acc, lt);
                     }
                 }
@@ -628,11 +678,12 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     const int offK = uni(L.offK), offV = uni(L.offV), offG = uni(L.offG);
                     const WT* Wa = uni_ptr((const WT*)L.Wa);
                     for (int rho = lw + XS1 * XLW; rho < RA; rho += XLW) {
-                        const float acc = pwave_sum(row_dot_stream<WT>(Wa, d, rowA_of(offK, offV, offG, X, nh, rho), nch, xn));
+                        const float acc = pwave_sum(row_dot_stream<WT, NCH>(Wa, d, rowA_of(offK, offV, offG, X, nh, rho), xn));
                         if (lane == 0) lst(qkvL + rho, acc, lt);
                     }
                 }
             }
+            W_STAMP(11);
             X_BARRIER(); // 2
             // ------------------------------------------------------------------ phase B
             if (wave < XAW) {
@@ -674,23 +725,20 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     float acc = 0.f;
                     const float* vcol = tV + (lane & 3);
                     const int pc = lane >> 2;
-                    if (nv == 64) {
+                    // all 64 rows: rows from nv on hold older K/V rows or the zeros of the start of the kernel, and
+                    // their weights are zero
 #pragma unroll 8
-                        for (int jj = 0; jj < 64; jj++) {
-                            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj));
-                            acc = fmaf(pj, vcol[jj * 64 + ((pc ^ (jj & 15)) << 2)], acc);
-                        }
-                    } else {
-                        for (int jj = 0; jj < nv; jj++) { // rows from nv on hold whatever the tile held before
-                            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj));
-                            acc = fmaf(pj, vcol[jj * 64 + ((pc ^ (jj & 15)) << 2)], acc);
-                        }
+                    for (int jj = 0; jj < 64; jj++) {
+                        const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj));
+                        acc = fmaf(pj, vcol[jj * 64 + ((pc ^ (jj & 15)) << 2)], acc);
                     }
-                    u64* out = partL + ((size_t)j * P.maxTiles + tl) * (XHD + 2);
+                    u64* out = partL + ((size_t)j * ntiles + tl) * (XHD + 2); // heads one after the other, as the combine reads them
                     lst(out + lane, acc, lt);
                     if (lane == 0) { lst(out + XHD, m, lt); lst(out + XHD + 1, l, lt); }
                     __builtin_amdgcn_wave_barrier();
                 }
+                if (P.timing && t == 0 && step == P.steps - 1 && lane == 0)
+                    P.timing[16 * (P.NL + 1) + 4 * wg + wave] = aslot < U ? wall_clock64() : 0;
                 // first tile of this wave for the next layer pass (the next step's first layer sees one more row)
                 if (!(lastLayer && step == P.steps - 1)) issueKV(Ln, lastLayer ? pos + 1 : pos);
             }
@@ -699,14 +747,16 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 int rows[XS1];
 #pragma unroll
                 for (int k = 0; k < XS1 / 2; k++) {
-                    const int q = lw + XLW * k;
-                    rows[2 * k] = q < fs ? 2 * (X * fs + q) : -1;
-                    rows[2 * k + 1] = q < fs ? 2 * (X * fs + q) + 1 : -1;
+                    const int q = min(lw + XLW * k, fs - 1);
+                    rows[2 * k] = 2 * (X * fs + q);
+                    rows[2 * k + 1] = 2 * (X * fs + q) + 1;
                 }
-                issue_rows<WT, XS1>(s1.r, uni_ptr((const WT*)L.W13), d, rows, nch);
-                issue_gain<WT>(gn, uni_ptr(L.g2), nch);
+                issue_rows<WT, XS1, NCH>(s1.r, uni_ptr((const WT*)L.W13), d, rows);
+                issue_gain<WT, NCH>(gn, uni_ptr(L.g2));
             }
+            W_STAMP(12);
             X_BARRIER(); // 3
+            W_STAMP(13);
             // ------------------------------------------------------------------ phase C
             if (nh > 0) {
                 const int rs = lane / CPS, c = lane % CPS;
@@ -721,22 +771,22 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                                 : PVec<WT>::load(uni_ptr((const WT*)L.Wo) + (size_t)row * ad + (X + XCDS * j) * XHD + c * N);
                             acc = chunk_dot_lds<WT>(w, S.as + j * XHD + c * N, acc);
                         }
-#pragma unroll
-                    for (int o = CPS / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, MLH_WAVE);
+                    acc = pgroup_sum<CPS>(acc);
                     if (c == 0) xst(P.h1P + (size_t)X * d + row, acc, lt);
                 }
             }
+            W_STAMP(14);
             issue_w2<WT>(s2, uni_ptr((const WT*)L.W2), X, fs, F, lw, d);
             X_BARRIER(); // 4
             // ------------------------------------------------------------------ phase D
             {
-                float xn[XCH][N];
-                normed_columns<WT>(S.h1s, gn, d, nch, xn);
+                float xn[NCH][N];
+                normed_columns<WT, NCH>(S.h1s, gn, d, xn);
 #pragma unroll
                 for (int k = 0; k < XS1 / 2; k++) {
                     const int q = lw + XLW * k;
                     if (q < fs) {
-                        const float g = pwave_sum(row_dot_reg<WT>(s1.r, 2 * k, nch, xn)), up = pwave_sum(row_dot_reg<WT>(s1.r, 2 * k + 1, nch, xn));
+                        const float g = pwave_sum(row_dot_reg<WT, NCH>(s1.r, 2 * k, xn)), up = pwave_sum(row_dot_reg<WT, NCH>(s1.r, 2 * k + 1, xn));
                         if (lane == 0) lst(P.uL + (size_t)X * fs + q, psilu(g) * up, lt); // inference.cu:262-281
                     }
                 }
@@ -744,8 +794,8 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     const WT* W13 = uni_ptr((const WT*)L.W13);
                     for (int q = lw + (XS1 / 2) * XLW; q < fs; q += XLW) {
                         const int pr = X * fs + q;
-                        const float g = pwave_sum(row_dot_stream<WT>(W13, d, 2 * pr, nch, xn));
-                        const float up = pwave_sum(row_dot_stream<WT>(W13, d, 2 * pr + 1, nch, xn));
+                        const float g = pwave_sum(row_dot_stream<WT, NCH>(W13, d, 2 * pr, xn));
+                        const float up = pwave_sum(row_dot_stream<WT, NCH>(W13, d, 2 * pr + 1, xn));
                         if (lane == 0) lst(P.uL + (size_t)X * fs + q, psilu(g) * up, lt);
                     }
                 }
@@ -755,9 +805,9 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             } else { // LM-head rows gwl, gwl + TWL, ... and the final gain
                 int rows[XS1];
 #pragma unroll
-                for (int k = 0; k < XS1; k++) rows[k] = gwl + TWL * k < V ? gwl + TWL * k : -1;
-                issue_rows<WT, XS1>(s1.r, E, d, rows, nch);
-                issue_gain<WT>(gn, a.gF, nch);
+                for (int k = 0; k < XS1; k++) rows[k] = min(gwl + TWL * k, V - 1);
+                issue_rows<WT, XS1, NCH>(s1.r, E, d, rows);
+                issue_gain<WT, NCH>(gn, a.gF);
             }
             X_BARRIER(); // 5
             // ------------------------------------------------------------------ phase E
@@ -789,18 +839,20 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 }
             }
             if (!lastLayer) {
-                issue_wo<WT>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, lw, d);
+                issue_wo<WT>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, a.heads, lw, d);
             } else {
-                const int rows[2] = {gwl + XS1 * TWL < V ? gwl + XS1 * TWL : -1, gwl + (XS1 + 1) * TWL < V ? gwl + (XS1 + 1) * TWL : -1};
-                issue_rows<WT, 2>(s2.r, E, d, rows, nch);
+                // two more LM-head rows; the second register set has room for them when a row has at most 4 chunks
+                const int rows[2] = {min(gwl + XS1 * TWL, V - 1), min(gwl + (XS1 + 1) * TWL, V - 1)};
+                typename PVec<WT>::Raw (&lm)[2 * NCH] = reinterpret_cast<typename PVec<WT>::Raw (&)[2 * NCH]>(s2.r);
+                issue_rows<WT, 2, NCH>(lm, E, d, rows);
             }
         }
 
         // ---------------------------------------------------------------------- LM head + argmax
         X_BARRIER(); // final x in LDS
         {
-            float xn[XCH][N];
-            normed_columns<WT>(S.xs, gn, d, nch, xn); // inference.cu:705-715
+            float xn[NCH][N];
+            normed_columns<WT, NCH>(S.xs, gn, d, xn); // inference.cu:705-715
             float best = -3.0e38f;
             int bidx = 0x7fffffff;
             auto take = [&](int row, float acc) { // rows ascend per wave: ties keep the lower index
@@ -810,17 +862,17 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             };
 #pragma unroll
             for (int k = 0; k < XS1; k++)
-                if (gwl + TWL * k < V) take(gwl + TWL * k, row_dot_reg<WT>(s1.r, k, nch, xn));
+                if (gwl + TWL * k < V) take(gwl + TWL * k, row_dot_reg<WT, NCH>(s1.r, k, xn));
 #pragma unroll
             for (int k = 0; k < 2; k++)
-                if (gwl + TWL * (XS1 + k) < V) take(gwl + TWL * (XS1 + k), row_dot_reg<WT>(s2.r, k, nch, xn));
-            for (int row = gwl + (XS1 + 2) * TWL; row < V; row += TWL) take(row, row_dot_stream<WT>(E, d, row, nch, xn));
+                if (gwl + TWL * (XS1 + k) < V) take(gwl + TWL * (XS1 + k), row_dot_reg<WT, NCH>(reinterpret_cast<const typename PVec<WT>::Raw (&)[2 * NCH]>(s2.r), k, xn));
+            for (int row = gwl + (XS1 + 2) * TWL; row < V; row += TWL) take(row, row_dot_stream<WT, NCH>(E, d, row, xn));
             if (lane == 0) { S.bestv[wave] = best; S.besti[wave] = bidx; }
         }
         if (step + 1 < P.steps) { // first layer of the next step
             const LayerDev& L0 = S.Ls[P.NL - 1];
             issueA(L0);
-            issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, lw, d);
+            issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
         }
         X_BARRIER(); // best logits in LDS
         X_BARRIER(); // next token in LDS
@@ -830,7 +882,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     (void)tok;
 }
 
-template <typename WT>
+template <typename WT, int NCH>
 __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     extern __shared__ float lds[];
     const StepArgs& a = P.a;
@@ -871,7 +923,7 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     const int tok = uni(a.tok[0]), pos = uni(a.pos[P.seq]);
     const unsigned tagBase = *P.tagCounter; // tags never repeat from launch to launch: nothing has to be cleared
     if (wave == XWORK) xcd_communicator<WT>(P, S, tok, pos, tagBase, X, r);
-    else xcd_worker<WT>(P, S, tok, pos, tagBase, X, r);
+    else xcd_worker<WT, NCH>(P, S, tok, pos, tagBase, X, r);
 }
 
 // before every launch: abort flag and per-XCD arrival counters
@@ -910,21 +962,21 @@ bool mlh_xcd_supported(const mlh_ctx* c) {
         if (hp.layerKinds[t] != MLH_KIND_ATTENTION) return false;
     const int N = hp.weightDtype == MLH_DTYPE_BF16 ? 8 : 4;
     if (hp.headDim != XHD || hp.pleDim != 0) return false;
-    if (hp.dim != hp.attnHeads * XHD || hp.dim > XCH * 64 * N || hp.dim % (64 * N) || hp.dim % XPER) return false;
+    if (hp.dim != hp.attnHeads * XHD || hp.dim > 4 * 64 * N || hp.dim % (64 * N) || hp.dim % XPER) return false;
     if (hp.attnHeads > XCDS * XNH) return false;
     if (hp.ffnDim % (XCDS * N)) return false;
     if (hp.dim / 4 > 512 || hp.dim % N) return false;
     return xcd_lds_bytes(c) <= 160 * 1024;
 }
 
-template <typename WT>
+template <typename WT, int NCH>
 static int launch_xcd(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
-    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
     int perCu = 0;
-    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT>, XWG, ldsBytes));
+    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH>, XWG, ldsBytes));
     if (perCu < 1) { c->err = "XCD-rank decode kernel does not fit on a compute unit"; return -1; }
     // one workgroup per compute unit, all resident at once (the occupancy query says each unit can hold one); waits are bounded
-    hipLaunchKernelGGL((k_decode_xcd<WT>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
+    hipLaunchKernelGGL((k_decode_xcd<WT, NCH>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
     MLH_CHECK(c, hipGetLastError());
     return 0;
 }
@@ -967,5 +1019,18 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.amax = t;
     const size_t ldsBytes = xcd_lds_bytes(c);
     hipLaunchKernelGGL(k_xcd_prep, dim3(1), dim3(64), 0, c->stream, P.abortFlag, P.xcdCount);
-    return hp.weightDtype == MLH_DTYPE_BF16 ? launch_xcd<bf16_t>(c, P, ldsBytes) : launch_xcd<float>(c, P, ldsBytes);
+    if (hp.weightDtype == MLH_DTYPE_BF16) {
+        switch (hp.dim / 512) { // chunks of 8 values per lane and row
+            case 1: return launch_xcd<bf16_t, 1>(c, P, ldsBytes);
+            case 2: return launch_xcd<bf16_t, 2>(c, P, ldsBytes);
+            case 3: return launch_xcd<bf16_t, 3>(c, P, ldsBytes);
+            default: return launch_xcd<bf16_t, 4>(c, P, ldsBytes);
+        }
+    }
+    switch (hp.dim / 256) { // chunks of 4 values per lane and row
+        case 1: return launch_xcd<float, 1>(c, P, ldsBytes);
+        case 2: return launch_xcd<float, 2>(c, P, ldsBytes);
+        case 3: return launch_xcd<float, 3>(c, P, ldsBytes);
+        default: return launch_xcd<float, 4>(c, P, ldsBytes);
+    }
 }

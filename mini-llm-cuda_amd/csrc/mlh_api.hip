@@ -207,7 +207,7 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         c->err = "clearing the exchange words failed";
         return bail(-2);
     }
-    if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1)))) return bail(rc);
+    if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1) + 4 * 256))) return bail(rc);
     c->copyBytes = (size_t)256 << 20;
     char *cs, *cd;
     if ((rc = dev_alloc(c, &cs, c->copyBytes)) || (rc = dev_alloc(c, &cd, c->copyBytes))) return bail(rc);
@@ -596,6 +596,35 @@ static void dump_persistent_timing(mlh_ctx* c) {
     static const char* xnames[15] = {"x.exchange", "A+hop", "B+hop", "C+2hops", "D+hop", "-", "-", "-", "-", "-", "-", "-", "-", "-", "-"};
     if (c->usePersistent == 2) for (int k = 0; k < 15; k++) names[k] = tnames[k];
     if (xcd) for (int k = 0; k < 15; k++) names[k] = xnames[k];
+    if (xcd) { // skew between workgroups at four points of the last layer pass
+        std::vector<unsigned long long> sk(4 * 256);
+        if (hipMemcpy(sk.data(), c->d_timing + 16 * (c->hp.transformers + 1), sk.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
+            const char* what[4] = {"attention wave 0 end", "attention wave 1 end", "partials all seen", "combine done"};
+            unsigned long long t0 = ~0ull;
+            for (int w = 0; w < 256; w++) if (sk[4 * w]) t0 = std::min(t0, sk[4 * w]);
+            for (int k = 0; k < 4; k++) {
+                std::vector<double> v;
+                for (int w = 0; w < 256; w++) v.push_back(sk[4 * w + k] ? ((double)sk[4 * w + k] - (double)t0) / 100.0 : -1.0);
+                double perX[8] = {0};
+                std::vector<double> sorted = v;
+                std::sort(sorted.begin(), sorted.end());
+                const size_t first = std::lower_bound(sorted.begin(), sorted.end(), 0.0) - sorted.begin(), cnt = 256 - first;
+                if (!cnt) continue;
+                fprintf(stderr, "[xcd skew] %-20s n %zu min %.2f median %.2f max %.2f us (first 8 workgroups:", what[k], cnt, sorted[first], sorted[first + cnt / 2], sorted[255]);
+                for (int w = 0; w < 8; w++) fprintf(stderr, " %.2f", v[w]);
+                fprintf(stderr, ")\n");
+                (void)perX;
+            }
+        }
+    }
+    if (xcd) { // raw stamps relative to the start of the layer pass: communicator 0-9, worker wave 0 10-14
+        double rel[16] = {0};
+        for (int l = 0; l < c->hp.transformers; l++)
+            for (int k = 0; k < 15; k++) rel[k] += ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 / c->hp.transformers;
+        fprintf(stderr, "[xcd stamps, us from layer start] x: cross %.2f publish %.2f ready %.2f | workerA start %.2f end %.2f | qkv ready %.2f | attention end(w0) %.2f | "
+                        "combine %.2f workerC start %.2f end %.2f | h1: cross %.2f publish %.2f ready %.2f | u ready %.2f\n",
+                rel[6], rel[7], rel[1], rel[10], rel[11], rel[2], rel[12], rel[3], rel[13], rel[14], rel[8], rel[9], rel[4], rel[5]);
+    }
     fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
     double sum = 0;
     for (int k = 0; k < 15; k++) { fprintf(stderr, " %s=%.2f", names[k], tot[k] / c->hp.transformers); sum += tot[k] / c->hp.transformers; }

@@ -122,7 +122,8 @@ struct mlh_ctx {
     // persistent batch-1 decode kernel
     int numCUs = 0;
     bool coopLaunch = false;
-    int usePersistent = 1;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange; 3: XCD ranks
+    int usePersistent = 3;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange;
+                                   // 3: XCD ranks where the model and device allow it, else as 1
     unsigned long long* xcdBuf = nullptr; // (value, tag) exchange words of mode 3
     size_t xcdWords = 0;
     unsigned long long* tagged = nullptr; // (value, tag) exchange words of mode 2

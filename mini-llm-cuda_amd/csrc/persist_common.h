@@ -20,15 +20,40 @@ __device__ __forceinline__ void astu(unsigned* p, unsigned v) { __hip_atomic_sto
 // prefetch with each barrier; inside this kernel threads of a workgroup exchange data through LDS only.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// Wave-wide reductions on the data-parallel-primitive path of the vector ALU (a handful of cycles per step) instead of
+// LDS-crossbar shuffles (a hundred-odd cycles each): within rows of 16 lanes by quad permutes and mirrors, across the
+// four rows by row broadcasts; lane 63 then holds the result and every lane receives it through a scalar register.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v, float fill) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(fill), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
 __device__ __forceinline__ float pwave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, MLH_WAVE);
+    v += dpp_move<0xB1, 0xf>(v, 0.f);  // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xf>(v, 0.f);  // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xf>(v, 0.f); // row_half_mirror
+    v += dpp_move<0x140, 0xf>(v, 0.f); // row_mirror: every lane holds the sum of its row
+    v += dpp_move<0x142, 0xa>(v, 0.f); // row_bcast15 into rows 1 and 3
+    v += dpp_move<0x143, 0xc>(v, 0.f); // row_bcast31 into rows 2 and 3
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+// Sum within aligned groups of W = 8 or 16 lanes; every lane of a group receives it.
+template <int W>
+__device__ __forceinline__ float pgroup_sum(float v) {
+    static_assert(W == 8 || W == 16, "group of 8 or 16 lanes");
+    v += dpp_move<0xB1, 0xf>(v, 0.f);
+    v += dpp_move<0x4E, 0xf>(v, 0.f);
+    v += dpp_move<0x141, 0xf>(v, 0.f);
+    if (W == 16) v += dpp_move<0x140, 0xf>(v, 0.f);
     return v;
 }
 __device__ __forceinline__ float pwave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MLH_WAVE));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x4E, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x141, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x140, 0xf>(v, v));
+    v = fmaxf(v, dpp_move<0x142, 0xa>(v, v));
+    v = fmaxf(v, dpp_move<0x143, 0xc>(v, v));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ __forceinline__ float psigmoid(float v) { return 1.0f / (1.0f + expf(-v)); } // inference.cu:248
 __device__ __forceinline__ float psilu(float v) { return v / (1.0f + expf(-v)); }       // inference.cu:270

@@ -49,7 +49,7 @@ def make(pkg, orc, hp, seed, bf16=False):
     return model, dev, w
 
 
-@pytest.mark.parametrize("persistent", [2, 1, 0], ids=["tagged", "persistent", "kernels"])
+@pytest.mark.parametrize("persistent", [3, 2, 1, 0], ids=["xcd", "tagged", "persistent", "kernels"])
 @pytest.mark.parametrize("kind,plen,steps", [("attn", 16, 40), ("attn_flags", 16, 40), ("hybrid", 16, 40),
                                              ("hybrid_flags", 16, 40), ("hd128", 16, 40), ("attn_long", 300, 12)])
 def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
@@ -58,6 +58,8 @@ def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
     hp = small_cfg(pkg, kind)
     model, dev, w = make(pkg, orc, hp, seed=11)
     dev.set_persistent(persistent)
+    if persistent == 3 and kind in ("attn", "attn_flags", "attn_long"):
+        assert dev.xcd_decode_supported()  # on the 256-unit MI355X; else the run below would silently be the barrier kernel
     prompt = pkg.random_tokens(11, 0, hp.vocabSize, plen)
     dev.prefill(0, prompt)
     ids, logits = [], []
@@ -72,7 +74,7 @@ def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
     dev.close()
 
 
-@pytest.mark.parametrize("persistent", [2, 1, 0], ids=["tagged", "persistent", "kernels"])
+@pytest.mark.parametrize("persistent", [3, 2, 1, 0], ids=["xcd", "tagged", "persistent", "kernels"])
 def test_config1_golden_horizon(pkg, orc, persistent):
     """Configuration 1 at full size: 16-token prompt, 128 greedy steps on the device loop, checked
     against the oracle and against the committed golden ids."""
@@ -92,6 +94,47 @@ def test_config1_golden_horizon(pkg, orc, persistent):
         assert np.array_equal(ids, g["ids"])
     # logits after the last fed token (generated token 127 of 128) against the golden full logits of step 127
     assert_logits_close(dev.logits(0), g["full_logits"][3], FP32_RTOL, "cfg1 golden step 127")
+    dev.close()
+
+
+@pytest.mark.parametrize("case", ["heads12", "bf16_dim512", "two_combine_batches", "shuffled_pages"])
+def test_xcd_rank_kernel_shapes(pkg, orc, case):
+    """The XCD-rank kernel on the shapes its work split distinguishes: XCDs with two heads and with one
+    (12 heads over 8 XCDs), bf16 weights (8 values per 16-byte chunk), more softmax partials per XCD than
+    one combine round fetches, and a shuffled page table; several launches in a row (the tags run on)."""
+    bf16 = case == "bf16_dim512"
+    kw = dict(transformers=2, vocabSize=1024, headDim=64)
+    if bf16:
+        hp = pkg.config(1, dim=512, attnHeads=8, ffnDim=1024, maxL=200, weightDtype=pkg.DTYPE_BF16, **kw)
+    elif case == "two_combine_batches":
+        hp = pkg.config(1, dim=768, attnHeads=12, ffnDim=512, maxL=900, qkRmsNorm=1, queryGating=1, **kw)
+    else:
+        hp = pkg.config(1, dim=768, attnHeads=12, ffnDim=512, maxL=200, **kw)
+    model, dev, w = make(pkg, orc, hp, seed=23, bf16=bf16)
+    dev.set_persistent(3)
+    assert dev.xcd_decode_supported()
+    if case == "shuffled_pages":
+        dev.set_page_table(np.random.default_rng(3).permutation((hp.maxL + 63) // 64 * hp.maxSeqs).astype(np.int32))
+    plen = 840 if case == "two_combine_batches" else 60  # 14 tiles x 2 heads = 28 partials on the two-head XCDs
+    prompt = pkg.random_tokens(23, 0, hp.vocabSize, plen)
+    if bf16:
+        dev.set_prefill_mode(1)  # the MFMA prefill rounds activations to half; here only the decode kernel is under test
+    dev.prefill(0, prompt)
+    dec = orc.Decoder(w, "f64")
+    for t in prompt:
+        nxt, lg = dec.step(int(t))
+    tok = dev.greedy_token(0)
+    rtol = BF16_RTOL if bf16 else FP32_RTOL
+    for launch, n in enumerate((1, 5, 3, 1)):  # the prompt ends inside a tile: the last launches cross into the next one
+        out = dev.decode_loop([tok], n)[:, 0]
+        feed = [tok] + [int(v) for v in out[:-1]]
+        for t in feed:
+            nxt, lg = dec.step(t)
+        worst = assert_logits_close(dev.logits(0), lg, rtol, f"{case} launch {launch}")
+        if not bf16:
+            assert worst < 1e-4
+        tok = int(out[-1])
+        assert tok == nxt or abs(float(lg[tok]) - float(lg[nxt])) < (2e-2 if bf16 else GAP_TOL)
     dev.close()
 
 
