@@ -351,8 +351,9 @@ __device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int f
 
 // K and V tile (64 rows x 64 floats each) of one head, rows below `lim`, global -> LDS without registers.  An
 // instruction moves 1 KB: lane i's 16 bytes land at base + 16 i, i.e. row 4q + i/16, slot i%16; the lane fetches the
-// piece that belongs there under the swizzle slot = piece ^ (row & 15), which makes the per-lane row reads of the
-// score loop conflict-free.  Kh, Vh: wave-uniform pointers to row 0 of the head's slice of the page.
+// piece that belongs there: for K under the swizzle slot = piece ^ (row & 15), which makes the per-lane row reads of
+// the score loop conflict-free; V stays row-major (the P.V loop reads a row across the lanes).  Kh, Vh: wave-uniform
+// pointers to row 0 of the head's slice of the page.
 __device__ __forceinline__ void issue_kv_tile(const float* Kh, const float* Vh, int d, int lim, float* tK, float* tV) {
     const unsigned lane = threadIdx.x & 63u;
 #pragma unroll
@@ -361,11 +362,11 @@ __device__ __forceinline__ void issue_kv_tile(const float* Kh, const float* Vh, 
         // row 4q of the tile is the wave-uniform part of the address, the lane adds (lane / 16) rows and its piece
         const char* Kq = pin_uniform(reinterpret_cast<const char*>(Kh + (size_t)(4 * q) * d));
         const char* Vq = pin_uniform(reinterpret_cast<const char*>(Vh + (size_t)(4 * q) * d));
-        unsigned lb = ((lane >> 4) * (unsigned)d + piece * 4u) * 4u;
+        unsigned lbK = ((lane >> 4) * (unsigned)d + piece * 4u) * 4u, lbV = ((lane >> 4) * (unsigned)d + (lane & 15) * 4u) * 4u;
         if ((int)row < lim) {
-            asm volatile("" : "+v"(lb));
-            __builtin_amdgcn_global_load_lds(Kq + (size_t)lb, tK + q * 256, 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(Vq + (size_t)lb, tV + q * 256, 16, 0, 0);
+            asm volatile("" : "+v"(lbK), "+v"(lbV));
+            __builtin_amdgcn_global_load_lds(Kq + (size_t)lbK, tK + q * 256, 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(Vq + (size_t)lbV, tV + q * 256, 16, 0, 0);
         }
     }
 }
@@ -403,9 +404,6 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
     bool ok = true;
 
     for (int step = 0; step < P.steps; step++) {
-        const float rc = a.rope[(size_t)pos * XHD + (lane & ~1)], rsn = a.rope[(size_t)pos * XHD + (lane | 1)];
-        const int pageNew = a.pageTable[P.seq * a.pagesPerSeq + (pos >> 6)];
-        const int T = pos + 1, ntiles = (T + 63) >> 6;
         // embedding gather (inference.cu:9-22): every workgroup keeps its own copy of the residual stream
         for (int i = lane; i < d; i += 64) S.xs[i] = PVec<WT>::one((const WT*)a.E + (size_t)tok * d + i);
 
@@ -414,12 +412,6 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             const unsigned lt = tagBase + (unsigned)(step * P.NL + (P.NL - 1 - t) + 1);
             const int ts = (P.NL - 1 - t) * 16;
             X_STAMP(ts + 0);
-            // q/k gains of this layer: issued ahead of the wait for x, whose answer comes later anyway
-            float gq[XNH], gk[XNH];
-            if (a.qkNorm)
-#pragma unroll
-                for (int j = 0; j < XNH; j++)
-                    if (j < nh) { gq[j] = uni_ptr(L.gq)[(X + XCDS * j) * XHD + lane]; gk[j] = uni_ptr(L.gk)[(X + XCDS * j) * XHD + lane]; }
             if (t != P.NL - 1) // partial x of the layer below, all XCDs, + its residual h1
                 reduce_publish_fetch(P.xP, d, s0, sl, lt - 1, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok,
                                      (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 6 : nullptr);
@@ -427,106 +419,14 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             X_STAMP(ts + 1);
             X_BARRIER(); // 1: x in LDS
 
-            // q | k | v | gate of the XCD's heads; per-head RMSNorm (inference.cu:52-81, 97-111), RoPE on adjacent
-            // pairs (inference.cu:113-134); workgroup 0 of the XCD appends the new K/V rows to the cache
+            // q | k | v | gate rows of the XCD's heads, as the workers produced them; the attention waves take it from there
             poll_vec<false, 8, false>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok);
-            {
-                float* qs = S.qkvs;
-                float* ks = qs + nh * XHD;
-                float* vs = ks + nh * XHD;
-#pragma unroll
-                for (int j = 0; j < XNH; j++)
-                    if (j < nh) {
-                        const int h = X + XCDS * j;
-                        float q = qs[j * XHD + lane], k = ks[j * XHD + lane];
-                        if (a.qkNorm) {
-                            const float sq = pwave_sum(q * q), sk = pwave_sum(k * k);
-                            const float rq = sqrtf(sq / (float)XHD + 1e-8f), rk = sqrtf(sk / (float)XHD + 1e-8f);
-                            q = gq[j] * (q / rq);
-                            k = gk[j] * (k / rk);
-                        }
-                        const float qo = __shfl_xor(q, 1, MLH_WAVE), ko = __shfl_xor(k, 1, MLH_WAVE);
-                        if (lane & 1) { q = rsn * qo + rc * q; k = rsn * ko + rc * k; }
-                        else { q = rc * q - rsn * qo; k = rc * k - rsn * ko; }
-                        qs[j * XHD + lane] = q;
-                        ks[j * XHD + lane] = k;
-                        if (r == 0) { // write-through: read from the next step on, by whichever workgroup takes the tile
-                            const size_t o = ((size_t)pageNew * MLH_KV_PAGE + (pos & 63)) * d + h * XHD + lane;
-                            ast(uni_ptr(L.K) + o, k);
-                            ast(uni_ptr(L.V) + o, vs[j * XHD + lane]);
-                        }
-                    }
-            }
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 2);
             X_BARRIER(); // 2: q, k, v, gate in LDS
 
-            // diagnostic: every workgroup's clock at points of the last layer pass (skew between workgroups)
-            u64* skew = (P.timing && t == 0 && step == P.steps - 1) ? P.timing + 16 * (P.NL + 1) + 4 * wg : nullptr;
-            // softmax partials of the XCD's heads -> mixing output (lane = dimension), gate (inference.cu:241-250)
-            {
-                const int U = nh * ntiles;
-                const float* gs = S.qkvs + 3 * nh * XHD;
-                float M = -1.0e30f, num = 0.f, den = 0.f;
-                int cur = 0;
-                int tlc = 0; // tiles of the current head already taken in
-                // One wave does this for the whole workgroup, so instructions count: the weights exp(m - M) of all
-                // units of a batch are formed at once (lane = unit); per unit only a broadcast and a multiply-add remain.
-                for (int u0 = 0; u0 < U; u0 += XCB) {
-                    u64 wa[XCB], wm, wl;
-                    const u64* ub = pin_uniform(partL + (size_t)u0 * (XHD + 2));
-                    const unsigned uOff = (unsigned)(min(u0 + (lane & 31), U - 1) - u0) * ((XHD + 2) * 8u);
-                    for (unsigned spins = 0;; spins++) {
-                        asm volatile("" ::: "memory");
-                        bool all = true;
-#pragma unroll
-                        for (int k = 0; k < XCB; k++) {
-                            if (u0 + k < U) wa[k] = ldw<false>(ub, (unsigned)lane * 8u, k * ((XHD + 2) * 8u));
-                            else wa[k] = (u64)lt << 32;
-                            all = all && (unsigned)(wa[k] >> 32) == lt;
-                        }
-                        wm = ldw<false>(ub, uOff, XHD * 8u);       // lane k < 32: running maximum of unit u0 + k
-                        wl = ldw<false>(ub, uOff, (XHD + 1) * 8u); //              and its sum of exponentials
-                        all = all && (unsigned)(wm >> 32) == lt && (unsigned)(wl >> 32) == lt;
-                        if (__all(all)) break;
-                        if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(P.abortFlag))) { ok = false; break; }
-                    }
-                    if (skew && lane == 0 && u0 == 0) skew[2] = wall_clock64();
-                    const float mk = __uint_as_float((unsigned)wm), lk = __uint_as_float((unsigned)wl);
-                    const int nb = U - u0 < XCB ? U - u0 : XCB;
-                    for (int k0 = 0; k0 < nb;) { // the heads that have units in this batch, one after the other
-                        const int take = nb - k0 < ntiles - tlc ? nb - k0 : ntiles - tlc;
-                        const bool mine = lane >= k0 && lane < k0 + take;
-                        // (a single wave issues one instruction every four cycles, whatever its kind: the hardware
-                        // exponential and reciprocal, and no branches around the units of other heads -- their
-                        // weight is zero)
-                        const float Mn = fmaxf(M, pwave_max(mine ? mk : -1.0e30f));
-                        const float corr = __expf(M - Mn);
-                        const float w = mine ? __expf(mk - Mn) : 0.f;
-                        den = fmaf(den, corr, pwave_sum(w * lk));
-                        num *= corr;
-#pragma unroll
-                        for (int k8 = 0; k8 < XCB; k8 += 8)
-                            if (k8 < nb) {
-#pragma unroll
-                                for (int k = k8; k < k8 + 8; k++)
-                                    num = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k)), __uint_as_float((unsigned)wa[k]), num);
-                            }
-                        M = Mn;
-                        tlc += take;
-                        k0 += take;
-                        if (tlc == ntiles) { // the head is complete
-                            float v = num * __builtin_amdgcn_rcpf(den);
-                            if (a.gating) v = v * __builtin_amdgcn_rcpf(1.0f + __expf(-gs[cur * XHD + lane])); // inference.cu:248
-                            S.as[cur * XHD + lane] = v;
-                            cur++; tlc = 0; M = -1.0e30f; num = 0.f; den = 0.f;
-                        }
-                    }
-                }
-            }
-            if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+            // (softmax partials are combined by the attention waves, one head per wave)
             X_STAMP(ts + 3);
-            if (skew && lane == 0) skew[3] = wall_clock64();
             X_BARRIER(); // 3: mixing output of the XCD's heads in LDS
 
             // h1 = x + sum of the XCDs' Wo partials (inference.cu:252-260)
@@ -629,13 +529,19 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
         issue_rows<WT, XS1, NCH>(s1.r, uni_ptr((const WT*)Lx.Wa), d, rows);
         issue_gain<WT, NCH>(gn, uni_ptr(Lx.g1));
     };
-    // first K/V tile of this wave in layer Lx when the sequence holds npos rows
+    // first K/V tile of this wave in layer Lx when the sequence holds npos rows, and the q/k gains of its head
+    float gqv = 1.f, gkv = 1.f;
+    // (the tile index of a wave's first unit never changes, so its page is looked up once)
+    const int pageFirst = (wave < XAW && nh > 0 && aslot / nh < a.pagesPerSeq) ? uni(a.pageTable[P.seq * a.pagesPerSeq + aslot / nh]) : 0;
     auto issueKV = [&](const LayerDev& Lx, int npos) {
         const int nt = (npos + 64) >> 6;
         if (aslot < nh * nt) {
             const int j = aslot % nh, tl = aslot / nh;
-            const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + tl]);
-            const size_t base = ((size_t)page * MLH_KV_PAGE) * d + (X + XCDS * j) * XHD;
+            if (a.qkNorm) {
+                gqv = uni_ptr(Lx.gq)[(X + XCDS * j) * XHD + lane];
+                gkv = uni_ptr(Lx.gk)[(X + XCDS * j) * XHD + lane];
+            }
+            const size_t base = ((size_t)pageFirst * MLH_KV_PAGE) * d + (X + XCDS * j) * XHD;
             issue_kv_tile(uni_ptr((const float*)Lx.K) + base, uni_ptr((const float*)Lx.V) + base, d, npos - tl * 64, tK, tV);
         }
     };
@@ -650,8 +556,18 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
         if (wave < XAW) issueKV(L0, pos);
     }
 
+    float* qh = S.tiles + XAW * 8192 + (wave < XAW ? wave : 0) * 64; // this wave's query after norm and RoPE
+    bool ok = true; // attention waves poll the softmax partials (bounded)
+
     for (int step = 0; step < P.steps; step++) {
         const int T = pos + 1, ntiles = (T + 63) >> 6, newTile = pos >> 6;
+        float rc = 1.f, rsn = 0.f; // RoPE of this step's position: lanes (2i, 2i+1) hold the pair i (inference.cu:113-134)
+        int pageNew = 0; // page that receives this step's K/V row
+        if (wave < XAW) {
+            rc = a.rope[(size_t)pos * XHD + (lane & ~1)];
+            rsn = a.rope[(size_t)pos * XHD + (lane | 1)];
+            pageNew = uni(a.pageTable[P.seq * a.pagesPerSeq + newTile]);
+        }
         for (int t = P.NL - 1; t >= 0; t--) {
             const LayerDev& L = S.Ls[t];
             const unsigned lt = tagBase + (unsigned)(step * P.NL + (P.NL - 1 - t) + 1);
@@ -688,32 +604,52 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             // ------------------------------------------------------------------ phase B
             if (wave < XAW) {
                 const int U = nh * ntiles;
-                const float* qsAll = S.qkvs;
+                const float* qsAll = S.qkvs; // rows as the first phase produced them
                 const float* ksAll = qsAll + nh * XHD;
                 const float* vsAll = ksAll + nh * XHD;
+                const float* gsAll = vsAll + nh * XHD;
+                // per-head RMSNorm (inference.cu:52-81, 97-111) and RoPE of a 64-vector held one element per lane
+                auto norm_rope = [&](float v, float gain) {
+                    if (a.qkNorm) v = gain * (v / sqrtf(pwave_sum(v * v) / (float)XHD + 1e-8f));
+                    const float o = dpp_move<0xB1, 0xf>(v, 0.f); // the other element of the pair
+                    return (lane & 1) ? rsn * o + rc * v : rc * v - rsn * o;
+                };
+                const bool dbg = P.timing && t == 0 && step == P.steps - 1 && lane == 0 && wave == 0;
+                if (dbg) P.timing[16 * (P.NL + 1) + 4 * wg + 1] = aslot < U ? wall_clock64() : 0;
                 for (int u = aslot; u < U; u += XAW * XPER) {
-                    const int j = u % nh, tl = u / nh, j0 = tl << 6;
+                    const int j = u % nh, tl = u / nh, j0 = tl << 6, h = X + XCDS * j;
                     if (u != aslot) { // tiles beyond the first one were not fetched ahead
                         const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + tl]);
-                        const size_t base = ((size_t)page * MLH_KV_PAGE) * d + (X + XCDS * j) * XHD;
+                        const size_t base = ((size_t)page * MLH_KV_PAGE) * d + h * XHD;
                         issue_kv_tile(uni_ptr((const float*)L.K) + base, uni_ptr((const float*)L.V) + base, d, pos - j0, tK, tV);
+                        if (a.qkNorm) { gqv = uni_ptr(L.gq)[h * XHD + lane]; gkv = uni_ptr(L.gk)[h * XHD + lane]; }
                     }
-                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the tile has landed in LDS
+                    qh[lane] = norm_rope(qsAll[j * XHD + lane], gqv);
+                    // The tile has landed in LDS.  A tile fetched a layer ahead is older than the dozens of weight loads
+                    // issued since (loads and stores retire in issue order): the few stores of the first phase may stay
+                    // in flight.
+                    if (u == aslot) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    if (dbg) P.timing[16 * (P.NL + 1) + 4 * wg + 3] = wall_clock64();
                     const int nv = T - j0 < 64 ? T - j0 : 64;       // keys of this tile, the new one included
-                    if (tl == newTile && lane < 16) {                // this step's row comes from LDS, not from the cache
+                    if (tl == newTile) { // this step's row comes from the first phase, not from the cache; it is appended here
                         const int rn = pos - j0;
-                        *reinterpret_cast<f32x4*>(tK + rn * 64 + ((lane ^ (rn & 15)) << 2)) = *reinterpret_cast<const f32x4*>(ksAll + j * XHD + lane * 4);
-                        *reinterpret_cast<f32x4*>(tV + rn * 64 + ((lane ^ (rn & 15)) << 2)) = *reinterpret_cast<const f32x4*>(vsAll + j * XHD + lane * 4);
+                        const float kn = norm_rope(ksAll[j * XHD + lane], gkv), vn = vsAll[j * XHD + lane];
+                        tK[rn * 64 + ((((lane >> 2) ^ (rn & 15)) << 2) | (lane & 3))] = kn;
+                        tV[rn * 64 + lane] = vn;
+                        // write-through: read from the next step on, by whichever workgroup of this XCD takes the tile
+                        const size_t o = ((size_t)pageNew * MLH_KV_PAGE + rn) * d + h * XHD + lane;
+                        ast(uni_ptr(L.K) + o, kn);
+                        ast(uni_ptr(L.V) + o, vn);
                     }
                     __builtin_amdgcn_wave_barrier();
                     float s = 0.f;
                     {
                         const float* kr = tK + lane * 64;
-                        const float* qs = qsAll + j * XHD;
-#pragma unroll 4
+#pragma unroll 8
                         for (int p = 0; p < 16; p++) {
                             const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + ((p ^ (lane & 15)) << 2));
-                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qs + p * 4);
+                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qh + p * 4);
                             s = fmaf(kk.x, qq.x, s); s = fmaf(kk.y, qq.y, s); s = fmaf(kk.z, qq.z, s); s = fmaf(kk.w, qq.w, s);
                         }
                     }
@@ -722,23 +658,77 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     const float m = pwave_max(s);
                     const float e = valid ? expf(s - m) : 0.f;
                     const float l = pwave_sum(e);
-                    float acc = 0.f;
-                    const float* vcol = tV + (lane & 3);
-                    const int pc = lane >> 2;
                     // all 64 rows: rows from nv on hold older K/V rows or the zeros of the start of the kernel, and
-                    // their weights are zero
-#pragma unroll 8
-                    for (int jj = 0; jj < 64; jj++) {
-                        const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj));
-                        acc = fmaf(pj, vcol[jj * 64 + ((pc ^ (jj & 15)) << 2)], acc);
+                    // their weights are zero.  Sixteen rows are fetched before they are used, so that the LDS latency
+                    // is paid four times, not sixty-four.
+                    float acc = 0.f;
+                    const float* vcol = tV + lane;
+#pragma unroll
+                    for (int jj0 = 0; jj0 < 64; jj0 += 16) {
+                        float vr[16];
+#pragma unroll
+                        for (int i = 0; i < 16; i++) vr[i] = vcol[(jj0 + i) * 64];
+#pragma unroll
+                        for (int i = 0; i < 16; i++)
+                            acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj0 + i)), vr[i], acc);
                     }
-                    u64* out = partL + ((size_t)j * ntiles + tl) * (XHD + 2); // heads one after the other, as the combine reads them
+                    u64* out = partL + ((size_t)j * ntiles + tl) * (XHD + 2); // a head's tiles one after the other, as the combine reads them
                     lst(out + lane, acc, lt);
                     if (lane == 0) { lst(out + XHD, m, lt); lst(out + XHD + 1, l, lt); }
                     __builtin_amdgcn_wave_barrier();
                 }
                 if (P.timing && t == 0 && step == P.steps - 1 && lane == 0)
                     P.timing[16 * (P.NL + 1) + 4 * wg + wave] = aslot < U ? wall_clock64() : 0;
+                W_STAMP(12);
+                // Softmax partials of the XCD's heads -> mixing output (lane = dimension), gate (inference.cu:241-250):
+                // every workgroup needs it, so its attention waves take one head each.  A single wave issues one
+                // instruction every four cycles whatever its kind: the weights exp(m - M) of a batch of tiles are
+                // formed at once (lane = tile), per tile only a broadcast and a multiply-add remain.
+                for (int j = wave; j < nh; j += XAW) {
+                    float M = -1.0e30f, num = 0.f, den = 0.f;
+                    for (int t0 = 0; t0 < ntiles; t0 += XCB) {
+                        const int nb = ntiles - t0 < XCB ? ntiles - t0 : XCB;
+                        u64 wa[XCB], wm, wl;
+                        const u64* ub = pin_uniform(partL + ((size_t)j * ntiles + t0) * (XHD + 2));
+                        const unsigned uOff = (unsigned)min(lane & 31, nb - 1) * ((XHD + 2) * 8u);
+                        for (unsigned spins = 0;; spins++) {
+                            asm volatile("" ::: "memory");
+                            bool all = true;
+#pragma unroll
+                            for (int k = 0; k < XCB; k++) {
+                                if (k < nb) wa[k] = ldw<false>(ub, (unsigned)lane * 8u, k * ((XHD + 2) * 8u));
+                                else wa[k] = (u64)lt << 32;
+                                all = all && (unsigned)(wa[k] >> 32) == lt;
+                            }
+                            wm = ldw<false>(ub, uOff, XHD * 8u);       // lane k < 32: running maximum of tile t0 + k
+                            wl = ldw<false>(ub, uOff, (XHD + 1) * 8u); //              and its sum of exponentials
+                            all = all && (unsigned)(wm >> 32) == lt && (unsigned)(wl >> 32) == lt;
+                            if (__all(all)) break;
+                            if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(P.abortFlag))) { ok = false; break; }
+                        }
+                        const float mk = __uint_as_float((unsigned)wm), lk = __uint_as_float((unsigned)wl);
+                        const bool mine = lane < nb;
+                        const float Mn = fmaxf(M, pwave_max(mine ? mk : -1.0e30f));
+                        const float corr = __expf(M - Mn);
+                        const float w = mine ? __expf(mk - Mn) : 0.f;
+                        den = fmaf(den, corr, pwave_sum(w * lk));
+                        num *= corr;
+#pragma unroll
+                        for (int k8 = 0; k8 < XCB; k8 += 8)
+                            if (k8 < nb) {
+#pragma unroll
+                                for (int k = k8; k < k8 + 8; k++)
+                                    num = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), k)), __uint_as_float((unsigned)wa[k]), num);
+                            }
+                        M = Mn;
+                    }
+                    float v = num * __builtin_amdgcn_rcpf(den);
+                    if (a.gating) v = v * __builtin_amdgcn_rcpf(1.0f + __expf(-gsAll[j * XHD + lane])); // inference.cu:248
+                    S.as[j * XHD + lane] = v;
+                }
+                if (dbg) P.timing[16 * (P.NL + 1) + 4 * wg + 2] = wave < nh ? wall_clock64() : 0;
+                W_STAMP(15);
+                if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
                 // first tile of this wave for the next layer pass (the next step's first layer sees one more row)
                 if (!(lastLayer && step == P.steps - 1)) issueKV(Ln, lastLayer ? pos + 1 : pos);
             }
@@ -754,7 +744,6 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 issue_rows<WT, XS1, NCH>(s1.r, uni_ptr((const WT*)L.W13), d, rows);
                 issue_gain<WT, NCH>(gn, uni_ptr(L.g2));
             }
-            W_STAMP(12);
             X_BARRIER(); // 3
             W_STAMP(13);
             // ------------------------------------------------------------------ phase C
@@ -898,7 +887,7 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     S.besti = reinterpret_cast<int*>(S.bestv + 16);
     S.ctl = S.besti + 16;               // [0] a wait expired, [1] next token
     S.tiles = reinterpret_cast<float*>(S.ctl + 16); // [XAW][K tile | V tile]
-    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 8192);
+    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 8192 + XAW * 64); // (after the tiles: one query vector per attention wave)
     for (int i = threadIdx.x; i < P.NL * (int)(sizeof(LayerDev) / 4); i += XWG)
         reinterpret_cast<uint32_t*>(S.Ls)[i] = reinterpret_cast<const uint32_t*>(P.layers)[i];
     if (threadIdx.x == 0) {
@@ -943,7 +932,7 @@ __global__ void k_xcd_zero(unsigned* p, size_t n) {
 static size_t xcd_lds_bytes(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
     const int fs = hp.ffnDim / XCDS;
-    return ((size_t)2 * hp.dim + 5 * XNH * XHD + ((fs + 3) & ~3) + 512 + 48 + XAW * 8192) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
+    return ((size_t)2 * hp.dim + 5 * XNH * XHD + ((fs + 3) & ~3) + 512 + 48 + XAW * 8192 + XAW * 64) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
 }
 
 // Exchange words (64-bit) the kernel needs for this model.

@@ -599,7 +599,18 @@ static void dump_persistent_timing(mlh_ctx* c) {
     if (xcd) { // skew between workgroups at four points of the last layer pass
         std::vector<unsigned long long> sk(4 * 256);
         if (hipMemcpy(sk.data(), c->d_timing + 16 * (c->hp.transformers + 1), sk.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-            const char* what[4] = {"attention wave 0 end", "attention wave 1 end", "partials all seen", "combine done"};
+            {   // per workgroup with a unit on wave 0: wait for the tile, unit, combine
+                std::vector<double> a1, a2, a3;
+                for (int w = 0; w < 256; w++)
+                    if (sk[4 * w] && sk[4 * w + 1]) {
+                        a1.push_back(((double)sk[4 * w + 3] - (double)sk[4 * w + 1]) / 100.0);
+                        a2.push_back(((double)sk[4 * w] - (double)sk[4 * w + 3]) / 100.0);
+                        a3.push_back(((double)sk[4 * w + 2] - (double)sk[4 * w]) / 100.0);
+                    }
+                auto pr = [&](const char* nm, std::vector<double>& v) { std::sort(v.begin(), v.end()); if (!v.empty()) fprintf(stderr, "[xcd unit] %-28s n %zu min %.2f median %.2f max %.2f us\n", nm, v.size(), v[0], v[v.size() / 2], v.back()); };
+                pr("barrier 2 -> tile waited for", a1); pr("tile ready -> unit end", a2); pr("unit end -> combine done", a3);
+            }
+            const char* what[4] = {"attention wave 0 end", "wave 0 unit start", "wave 0 combine done", "wave 0 tile ready"};
             unsigned long long t0 = ~0ull;
             for (int w = 0; w < 256; w++) if (sk[4 * w]) t0 = std::min(t0, sk[4 * w]);
             for (int k = 0; k < 4; k++) {
@@ -620,10 +631,15 @@ static void dump_persistent_timing(mlh_ctx* c) {
     if (xcd) { // raw stamps relative to the start of the layer pass: communicator 0-9, worker wave 0 10-14
         double rel[16] = {0};
         for (int l = 0; l < c->hp.transformers; l++)
-            for (int k = 0; k < 15; k++) rel[k] += ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 / c->hp.transformers;
+            for (int k = 0; k < 16; k++) rel[k] += ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 / c->hp.transformers;
+        for (int l = 0; l < c->hp.transformers; l++) {
+            fprintf(stderr, "[xcd layer %2d]", l);
+            for (int k = 0; k < 16; k++) fprintf(stderr, " %d:%.2f", k, t[l * 16 + k] ? ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 : -1.0);
+            fprintf(stderr, "\n");
+        }
         fprintf(stderr, "[xcd stamps, us from layer start] x: cross %.2f publish %.2f ready %.2f | workerA start %.2f end %.2f | qkv ready %.2f | attention end(w0) %.2f | "
-                        "combine %.2f workerC start %.2f end %.2f | h1: cross %.2f publish %.2f ready %.2f | u ready %.2f\n",
-                rel[6], rel[7], rel[1], rel[10], rel[11], rel[2], rel[12], rel[3], rel[13], rel[14], rel[8], rel[9], rel[4], rel[5]);
+                        "combine(w0) %.2f workerC start %.2f end %.2f | h1: cross %.2f publish %.2f ready %.2f | u ready %.2f\n",
+                rel[6], rel[7], rel[1], rel[10], rel[11], rel[2], rel[12], rel[15], rel[13], rel[14], rel[8], rel[9], rel[4], rel[5]);
     }
     fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
     double sum = 0;
