@@ -32,6 +32,8 @@
 // fetched global -> LDS directly (no registers) a whole layer ahead.
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include "mlh_internal.h"
 #include "persist_common.h"
 
@@ -68,6 +70,9 @@ struct XcdArgs {
     u64* xL;                    // [XCDS][d]
     u64* amax;                  // [grid][2]
     u64* timing;                // optional: communicator of workgroup 0, last step, 8 stamps per layer
+    int napRound;               // 64-cycle units between two reads of the partial sums from other XCDs
+    int nap[5];                 // 64-cycle units a consumer stays away before its first read of: partial sums from other
+                                // XCDs, the gathered slices, q|k|v rows, FFN activations, softmax partials
 };
 
 __device__ __forceinline__ u64 xpack(float v, unsigned tag) { return ((u64)tag << 32) | __float_as_uint(v); }
@@ -107,12 +112,21 @@ __device__ __forceinline__ u64 ldw(const u64* base, unsigned laneBytes, unsigned
     return CROSS ? xld(p) : lld(p);
 }
 
+// Keeps this wave off the memory system for about n x 64 cycles.  Reading before anything can have arrived only
+// competes with the producers' stores: a first read delayed by the known minimum latency arrives just as early.
+__device__ __forceinline__ void nap64(int n) {
+    for (; n >= 16; n -= 16) __builtin_amdgcn_s_sleep(16);
+    for (; n >= 4; n -= 4) __builtin_amdgcn_s_sleep(4);
+    for (; n > 0; n--) __builtin_amdgcn_s_sleep(1);
+}
+
 // One wave fetches n tagged words into LDS, NB loads per lane and round, reading again until every tag is there.
 // With PIPE two rounds are in flight, a fraction of a round trip apart: the answer to a round that just missed the
 // data is followed closely by the next one instead of by a whole new round trip.  All 64 lanes take part.
 template <bool CROSS, int NB, bool PIPE>
-__device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, float* dst, const unsigned* abortFlag, bool& ok) {
+__device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, float* dst, const unsigned* abortFlag, bool& ok, int nap = 0) {
     const int lane = threadIdx.x & 63;
+    nap64(nap);
     for (int base = 0; base < n; base += 64 * NB) {
         u64 wA[NB], wB[NB];
         auto issue = [&](u64 (&w)[NB]) {
@@ -152,13 +166,15 @@ __device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, fl
     }
 }
 
-// Sum of the eight XCDs' partials over this workgroup's slice [s0, s0 + sl) (sl <= 64) plus the residual, published
-// inside the XCD; then the whole vector is fetched from the XCD's 32 slices.  haveMask bit X' clear: that XCD
-// contributes nothing.
-__device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int s0, int sl, unsigned tag, unsigned haveMask,
-                                                     const float* resid, float* scratch, u64* pub, float* dst,
-                                                     const unsigned* abortFlag, bool& ok, u64* stamp = nullptr) {
+// A vector that every workgroup needs, out of the eight XCDs' partial sums: workgroup `rank` of every XCD adds the
+// eight partials of slice [rank sl, (rank + 1) sl) (sl = d / 32 <= 64) and the residual and publishes the slice inside
+// the XCD; then every workgroup fetches the whole vector from its XCD's 32 slices.  haveMask bit X' clear: that XCD
+// contributes nothing.  Reads across XCDs disturb the stores they wait for, so the first one comes late (napCross).
+__device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int rank, unsigned tag, unsigned haveMask,
+                                                     const float* resid, u64* pub, float* dst, const unsigned* abortFlag, bool& ok,
+                                                     int napCross, int napGather, int napRound, u64* stamp = nullptr) {
     const int lane = threadIdx.x & 63;
+    const int sl = d / XPER, s0 = rank * sl;
     const unsigned lb = (unsigned)min(lane, sl - 1) * 8u;
     u64 wA[XCDS], wB[XCDS];
     auto issue = [&](u64 (&w)[XCDS]) {
@@ -182,12 +198,13 @@ __device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int
         return t;
     };
     float sum = 0.f;
+    nap64(napCross);
     issue(wA);
     for (unsigned spins = 0;; spins++) {
-        __builtin_amdgcn_s_sleep(8);
+        nap64(napRound);
         issue(wB);
         if (good(wA)) { sum = total(wA); break; }
-        __builtin_amdgcn_s_sleep(8);
+        nap64(napRound);
         issue(wA);
         if (good(wB)) { sum = total(wB); break; }
         if (!ok || spins > XSPIN || ((spins & 127) == 127 && aldu(abortFlag))) { ok = false; break; }
@@ -195,8 +212,7 @@ __device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int
     if (stamp && lane == 0) stamp[0] = wall_clock64();
     if (lane < sl) lst(pub + s0 + lane, sum + resid[s0 + lane], tag);
     if (stamp && lane == 0) stamp[1] = wall_clock64();
-    poll_vec<false, 16, false>(pub, d, tag, dst, abortFlag, ok);
-    (void)scratch;
+    poll_vec<false, 16, false>(pub, d, tag, dst, abortFlag, ok, napGather);
 }
 
 // NCH (template parameter of the kernel): 16-byte chunks per lane of a full-width row, dim / (64 N)
@@ -396,7 +412,6 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
     const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
     const int np = 3 + (a.gating ? 1 : 0);
     const int RA = np * nh * XHD;
-    const int sl = d / XPER, s0 = r * sl;
     unsigned headMask = 0; // XCDs that own at least one head
     for (int xc = 0; xc < XCDS; xc++) headMask |= (a.heads > xc ? 1u : 0u) << xc;
     u64* qkvL = P.qkvL + (size_t)X * P.qkvStride;
@@ -413,14 +428,14 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             const int ts = (P.NL - 1 - t) * 16;
             X_STAMP(ts + 0);
             if (t != P.NL - 1) // partial x of the layer below, all XCDs, + its residual h1
-                reduce_publish_fetch(P.xP, d, s0, sl, lt - 1, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok,
+                reduce_publish_fetch(P.xP, d, r, lt - 1, 0xffu, S.h1s, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound,
                                      (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 6 : nullptr);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 1);
             X_BARRIER(); // 1: x in LDS
 
             // q | k | v | gate rows of the XCD's heads, as the workers produced them; the attention waves take it from there
-            poll_vec<false, 8, false>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok);
+            poll_vec<false, 8, false>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok, P.nap[2]);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 2);
             X_BARRIER(); // 2: q, k, v, gate in LDS
@@ -430,13 +445,13 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             X_BARRIER(); // 3: mixing output of the XCD's heads in LDS
 
             // h1 = x + sum of the XCDs' Wo partials (inference.cu:252-260)
-            reduce_publish_fetch(P.h1P, d, s0, sl, lt, headMask, S.xs, S.scratch, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok,
+            reduce_publish_fetch(P.h1P, d, r, lt, headMask, S.xs, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound,
                                  (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 8 : nullptr);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 4);
             X_BARRIER(); // 4: h1 in LDS
 
-            poll_vec<false, 8, false>(P.uL + (size_t)X * P.fs, P.fs, lt, S.us, P.abortFlag, ok);
+            poll_vec<false, 8, false>(P.uL + (size_t)X * P.fs, P.fs, lt, S.us, P.abortFlag, ok, P.nap[3]);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 5);
             X_BARRIER(); // 5: the XCD's FFN activations in LDS
@@ -444,7 +459,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
 
         // ---------------------------------------------------------------------- LM head + argmax
         const unsigned ltLast = tagBase + (unsigned)(step * P.NL + P.NL);
-        reduce_publish_fetch(P.xP, d, s0, sl, ltLast, 0xffu, S.h1s, S.scratch, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok);
+        reduce_publish_fetch(P.xP, d, r, ltLast, 0xffu, S.h1s, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound);
         if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
         X_BARRIER(); // final x in LDS
         X_BARRIER(); // the workers' best logits in LDS
@@ -505,6 +520,8 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     const int d = a.dim, F = a.ffn, V = a.vocab, fs = P.fs;
     const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6), wg = blockIdx.x;
     const int lw = wave * XPER + r;             // worker wave within the XCD: consecutive rows land on different workgroups
+    const int lwF = (XWORK - 1 - wave) * XPER + r; // the same in reverse wave order, for the FFN units: a second unit, where
+                                                   // there is one, goes to the last waves, not to the attention waves
     const int gwl = wave * (int)gridDim.x + wg; // worker wave within the grid (LM head)
     const int TWL = XWORK * (int)gridDim.x;
     const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
@@ -684,6 +701,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 // every workgroup needs it, so its attention waves take one head each.  A single wave issues one
                 // instruction every four cycles whatever its kind: the weights exp(m - M) of a batch of tiles are
                 // formed at once (lane = tile), per tile only a broadcast and a multiply-add remain.
+                if (wave < nh) nap64(P.nap[4]);
                 for (int j = wave; j < nh; j += XAW) {
                     float M = -1.0e30f, num = 0.f, den = 0.f;
                     for (int t0 = 0; t0 < ntiles; t0 += XCB) {
@@ -737,7 +755,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 int rows[XS1];
 #pragma unroll
                 for (int k = 0; k < XS1 / 2; k++) {
-                    const int q = min(lw + XLW * k, fs - 1);
+                    const int q = min(lwF + XLW * k, fs - 1);
                     rows[2 * k] = 2 * (X * fs + q);
                     rows[2 * k + 1] = 2 * (X * fs + q) + 1;
                 }
@@ -773,15 +791,15 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 normed_columns<WT, NCH>(S.h1s, gn, d, xn);
 #pragma unroll
                 for (int k = 0; k < XS1 / 2; k++) {
-                    const int q = lw + XLW * k;
+                    const int q = lwF + XLW * k;
                     if (q < fs) {
                         const float g = pwave_sum(row_dot_reg<WT, NCH>(s1.r, 2 * k, xn)), up = pwave_sum(row_dot_reg<WT, NCH>(s1.r, 2 * k + 1, xn));
                         if (lane == 0) lst(P.uL + (size_t)X * fs + q, psilu(g) * up, lt); // inference.cu:262-281
                     }
                 }
-                if (lw + (XS1 / 2) * XLW < fs) {
+                if (lwF + (XS1 / 2) * XLW < fs) {
                     const WT* W13 = uni_ptr((const WT*)L.W13);
-                    for (int q = lw + (XS1 / 2) * XLW; q < fs; q += XLW) {
+                    for (int q = lwF + (XS1 / 2) * XLW; q < fs; q += XLW) {
                         const int pr = X * fs + q;
                         const float g = pwave_sum(row_dot_stream<WT, NCH>(W13, d, 2 * pr, xn));
                         const float up = pwave_sum(row_dot_stream<WT, NCH>(W13, d, 2 * pr + 1, xn));
@@ -995,6 +1013,16 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.maxTiles = c->pagesPerSeq;
     P.fs = hp.ffnDim / XCDS;
     P.timing = c->d_timing;
+    {
+        static const int dflt[5] = {50, 0, 0, 0, 0};
+        const char* er = getenv("MLH_XCD_NAP_ROUND");
+        P.napRound = er ? std::max(0, std::min(400, atoi(er))) : 3;
+        static const char* names[5] = {"MLH_XCD_NAP_CROSS", "MLH_XCD_NAP_GATHER", "MLH_XCD_NAP_QKV", "MLH_XCD_NAP_U", "MLH_XCD_NAP_PART"};
+        for (int k = 0; k < 5; k++) {
+            const char* e = getenv(names[k]);
+            P.nap[k] = e ? std::max(0, std::min(400, atoi(e))) : dflt[k];
+        }
+    }
     u64* t = c->xcdBuf;
     P.qkvStride = 4 * XNH * XHD;
     P.qkvL = t; t += (size_t)XCDS * P.qkvStride;
