@@ -211,7 +211,6 @@ __device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int
     }
     if (stamp && lane == 0) stamp[0] = wall_clock64();
     if (lane < sl) lst(pub + s0 + lane, sum + resid[s0 + lane], tag);
-    if (stamp && lane == 0) stamp[1] = wall_clock64();
     poll_vec<false, 16, false>(pub, d, tag, dst, abortFlag, ok, napGather);
 }
 
@@ -807,6 +806,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     }
                 }
             }
+            W_STAMP(7);
             if (!lastLayer) {
                 issueA(Ln);
             } else { // LM-head rows gwl, gwl + TWL, ... and the final gain
@@ -845,6 +845,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     if (lane == 0) xst(P.xP + (size_t)X * d + row, acc, lt);
                 }
             }
+            W_STAMP(9);
             if (!lastLayer) {
                 issue_wo<WT>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, a.heads, lw, d);
             } else {

@@ -637,9 +637,11 @@ static void dump_persistent_timing(mlh_ctx* c) {
             for (int k = 0; k < 16; k++) fprintf(stderr, " %d:%.2f", k, t[l * 16 + k] ? ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 : -1.0);
             fprintf(stderr, "\n");
         }
-        fprintf(stderr, "[xcd stamps, us from layer start] x: cross %.2f publish %.2f ready %.2f | workerA start %.2f end %.2f | qkv ready %.2f | attention end(w0) %.2f | "
-                        "combine(w0) %.2f workerC start %.2f end %.2f | h1: cross %.2f publish %.2f ready %.2f | u ready %.2f\n",
-                rel[6], rel[7], rel[1], rel[10], rel[11], rel[2], rel[12], rel[15], rel[13], rel[14], rel[8], rel[9], rel[4], rel[5]);
+        fprintf(stderr, "[xcd stamps, us from layer start] x: partials seen %.2f gathered %.2f | worker A %.2f..%.2f | q,k,v in LDS %.2f | "
+                        "wave 0: units done %.2f combine done %.2f | worker C %.2f..%.2f | h1: partials seen %.2f gathered %.2f | worker D end %.2f | "
+                        "u in LDS %.2f | worker E end %.2f\n",
+                rel[6], rel[1], rel[10], rel[11], rel[2], rel[12], rel[15], rel[13], rel[14], rel[8], rel[4], rel[7], rel[5], rel[9]);
+
     }
     fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
     double sum = 0;
