@@ -70,6 +70,7 @@ struct XcdArgs {
     u64* xL;                    // [XCDS][d]
     u64* amax;                  // [grid][2]
     u64* timing;                // optional: communicator of workgroup 0, last step, 8 stamps per layer
+    int wide;                   // slices of 64 elements (d / 64 readers per XCD) instead of d / 32 elements (32 readers)
     int napRound;               // 64-cycle units between two reads of the partial sums from other XCDs
     int nap[5];                 // 64-cycle units a consumer stays away before its first read of: partial sums from other
                                 // XCDs, the gathered slices, q|k|v rows, FFN activations, softmax partials
@@ -172,9 +173,14 @@ __device__ __forceinline__ void poll_vec(const u64* src, int n, unsigned tag, fl
 // contributes nothing.  Reads across XCDs disturb the stores they wait for, so the first one comes late (napCross).
 __device__ __forceinline__ void reduce_publish_fetch(const u64* part, int d, int rank, unsigned tag, unsigned haveMask,
                                                      const float* resid, u64* pub, float* dst, const unsigned* abortFlag, bool& ok,
-                                                     int napCross, int napGather, int napRound, u64* stamp = nullptr) {
+                                                     int napCross, int napGather, int napRound, bool wide, u64* stamp = nullptr) {
     const int lane = threadIdx.x & 63;
-    const int sl = d / XPER, s0 = rank * sl;
+    const int sl = wide ? 64 : d / XPER, s0 = rank * sl;
+    if (s0 >= d) { // (wide slices: only d / 64 workgroups of the XCD read the other XCDs' partial sums)
+        nap64(napCross + 24);
+        poll_vec<false, 16, false>(pub, d, tag, dst, abortFlag, ok, napGather);
+        return;
+    }
     const unsigned lb = (unsigned)min(lane, sl - 1) * 8u;
     u64 wA[XCDS], wB[XCDS];
     auto issue = [&](u64 (&w)[XCDS]) {
@@ -427,7 +433,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             const int ts = (P.NL - 1 - t) * 16;
             X_STAMP(ts + 0);
             if (t != P.NL - 1) // partial x of the layer below, all XCDs, + its residual h1
-                reduce_publish_fetch(P.xP, d, r, lt - 1, 0xffu, S.h1s, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound,
+                reduce_publish_fetch(P.xP, d, r, lt - 1, 0xffu, S.h1s, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound, P.wide != 0,
                                      (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 6 : nullptr);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 1);
@@ -444,7 +450,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             X_BARRIER(); // 3: mixing output of the XCD's heads in LDS
 
             // h1 = x + sum of the XCDs' Wo partials (inference.cu:252-260)
-            reduce_publish_fetch(P.h1P, d, r, lt, headMask, S.xs, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound,
+            reduce_publish_fetch(P.h1P, d, r, lt, headMask, S.xs, P.h1L + (size_t)X * d, S.h1s, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound, P.wide != 0,
                                  (P.timing && wg == 0 && step == P.steps - 1) ? P.timing + ts + 8 : nullptr);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 4);
@@ -458,7 +464,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
 
         // ---------------------------------------------------------------------- LM head + argmax
         const unsigned ltLast = tagBase + (unsigned)(step * P.NL + P.NL);
-        reduce_publish_fetch(P.xP, d, r, ltLast, 0xffu, S.h1s, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound);
+        reduce_publish_fetch(P.xP, d, r, ltLast, 0xffu, S.h1s, P.xL + (size_t)X * d, S.xs, P.abortFlag, ok, P.nap[0], P.nap[1], P.napRound, P.wide != 0);
         if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
         X_BARRIER(); // final x in LDS
         X_BARRIER(); // the workers' best logits in LDS
@@ -1015,7 +1021,9 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.fs = hp.ffnDim / XCDS;
     P.timing = c->d_timing;
     {
-        static const int dflt[5] = {50, 0, 0, 0, 0};
+        static const int dflt[5] = {44, 0, 0, 0, 0};
+        const char* ew = getenv("MLH_XCD_WIDE");
+        P.wide = ew ? atoi(ew) : 1;
         const char* er = getenv("MLH_XCD_NAP_ROUND");
         P.napRound = er ? std::max(0, std::min(400, atoi(er))) : 3;
         static const char* names[5] = {"MLH_XCD_NAP_CROSS", "MLH_XCD_NAP_GATHER", "MLH_XCD_NAP_QKV", "MLH_XCD_NAP_U", "MLH_XCD_NAP_PART"};
