@@ -357,12 +357,23 @@ __device__ __forceinline__ void g_ast(float* p, float v) {
 }
 
 #define GSK_COUNTERS 1024 // tiles a split-K launch may have (N <= 32768)
+#define GSK_WAVES 8       // waves of a skinny-GEMM workgroup: they split K, and each keeps two chunks of loads in flight --
+                          // with few waves the kernel waits on memory latency chunk after chunk, not on bandwidth
+
+// Sum of the waves' partial accumulators, in a fixed order.
+template <int MB>
+__device__ __forceinline__ float red_sum(const float (&red)[GSK_WAVES][MB][16][64], int mb, int i, int lane) {
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < GSK_WAVES; w += 2) t += red[w][mb][i][lane] + red[w + 1][mb][i][lane];
+    return t;
+}
 
 template <typename T, int MB, int EPI>
-__global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
+__global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
                                                           void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
                                                           unsigned* counters, float* partials, float alpha) {
-    __shared__ float red[4][MB][16][64];
+    __shared__ float red[GSK_WAVES][MB][16][64];
     __shared__ int lastFlag;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = blockIdx.x * 32, n32 = lane & 31, half = lane >> 5;
@@ -393,13 +404,15 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) GemmTraits<T>::mma(fb[buf][p], fa[buf][mb][p], acc[mb]);
     };
+    // (The product itself bounds this kernel at M = 64 in fp32: 32 rows x 64 tokens x K on one compute unit's matrix
+    // cores is 5.8 us at K = 768, whatever the number of waves or of loads in flight.)
     int c = cbeg + wave;
     if (c < cend) load(c, 0);
-    for (; c < cend; c += 8) { // two chunks per trip so the buffers are addressed statically
-        if (c + 4 < cend) load(c + 4, 1);
+    for (; c < cend; c += 2 * GSK_WAVES) { // two chunks per trip so the buffers are addressed statically
+        if (c + GSK_WAVES < cend) load(c + GSK_WAVES, 1);
         mul(0);
-        if (c + 4 < cend) {
-            if (c + 8 < cend) load(c + 8, 0);
+        if (c + GSK_WAVES < cend) {
+            if (c + 2 * GSK_WAVES < cend) load(c + 2 * GSK_WAVES, 0);
             mul(1);
         }
     }
@@ -408,16 +421,16 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
 #pragma unroll
         for (int i = 0; i < 16; i++) red[wave][mb][i][lane] = acc[mb][i];
     __syncthreads();
-    // the workgroup's tile: MB x 4 groups of four accumulator elements per lane, wave w takes groups w, w + 4
+    // the workgroup's tile: MB x 4 groups of four accumulator elements per lane, wave w takes groups w, w + GSK_WAVES, ...
     const size_t tileFloats = (size_t)MB * 16 * 64;
     float* myPart = partials + ((size_t)blockIdx.x * ks + kslice) * tileFloats;
     if (ks > 1) {
-        for (int g = wave; g < MB * 4; g += 4) {
+        for (int g = wave; g < MB * 4; g += GSK_WAVES) {
             const int mb = g >> 2, i4 = g & 3;
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int i = 4 * i4 + j;
-                g_ast(myPart + ((size_t)mb * 16 + i) * 64 + lane, (red[0][mb][i][lane] + red[1][mb][i][lane]) + (red[2][mb][i][lane] + red[3][mb][i][lane]));
+                g_ast(myPart + ((size_t)mb * 16 + i) * 64 + lane, red_sum(red, mb, i, lane));
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // the stores above have been acknowledged ...
@@ -430,7 +443,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
         __syncthreads();
         if (!lastFlag) return;
     }
-    for (int g = wave; g < MB * 4; g += 4) {
+    for (int g = wave; g < MB * 4; g += GSK_WAVES) {
         const int mb = g >> 2, i4 = g & 3;
         float v[4];
 #pragma unroll
@@ -441,7 +454,7 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_skinny(const T* __restrict__ 
                 for (int q = 0; q < ks; q++) sum += g_ald(partials + ((size_t)blockIdx.x * ks + q) * tileFloats + ((size_t)mb * 16 + i) * 64 + lane);
                 v[j] = sum;
             } else {
-                v[j] = (red[0][mb][i][lane] + red[1][mb][i][lane]) + (red[2][mb][i][lane] + red[3][mb][i][lane]);
+                v[j] = red_sum(red, mb, i, lane);
             }
         }
 #pragma unroll
@@ -483,9 +496,9 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
     unsigned* counters = (unsigned*)ws;
     float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
     if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_SWIGLU>), grid, dim3(GSK_WAVES * 64), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
     else
-        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GTHREADS), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
+        hipLaunchKernelGGL((k_gemm_skinny<T, MB, GEMM_EPI_PLAIN>), grid, dim3(GSK_WAVES * 64), 0, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
     return hipGetLastError();
 }
 
