@@ -477,6 +477,133 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny(const T* __restr
     }
 }
 
+// The same for 32 < M <= 64 in fp32 with 16 weight rows per workgroup (v_mfma_f32_16x16x4f32, four token blocks of
+// 16).  At this size the product is bound by the matrix cores of the compute units it runs on -- 32 rows x 64 tokens
+// x K = 768 take one unit 5.8 us -- and a matrix of a few thousand rows in 32-row tiles occupies a third of the chip:
+// tiles of 16 rows double the units at work.  Lane l holds weight row l % 16 (token l % 16 of a block) and the
+// 16 bytes at K offset (l / 16) * 16 of each 64-byte half chunk; element e of those vectors meets element e.
+template <int EPI>
+__global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb,
+                                                                   void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
+                                                                   unsigned* counters, float* partials, float alpha) {
+    __shared__ float red[GSK_WAVES][4][4][64];
+    __shared__ int lastFlag;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n0 = blockIdx.x * 16, n16 = lane & 15, kq = lane >> 4;
+    const int ks = gridDim.y, kslice = blockIdx.y;
+    const int nchunks = (int)(((size_t)K * 4) / GKB);
+    const int cbeg = (int)((long)nchunks * kslice / ks), cend = (int)((long)nchunks * (kslice + 1) / ks);
+    const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n16, N - 1) * ldb * 4 + kq * 16;
+    const unsigned char* arow[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) arow[tb] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(tb * 16 + n16, M - 1) * lda * 4 + kq * 16;
+    f32x4 acc[4];
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++) acc[tb] = (f32x4)(0.f);
+    f32x4 fb[2][2], fa[2][4][2];
+    auto load = [&](int c, int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) fb[buf][p] = *reinterpret_cast<const f32x4*>(brow + (size_t)c * GKB + p * 64);
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+            for (int p = 0; p < 2; p++) fa[buf][tb][p] = *reinterpret_cast<const f32x4*>(arow[tb] + (size_t)c * GKB + p * 64);
+    };
+    auto mul = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int tb = 0; tb < 4; tb++) acc[tb] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[buf][p][e], fa[buf][tb][p][e], acc[tb], 0, 0, 0);
+    };
+    int c = cbeg + wave;
+    if (c < cend) load(c, 0);
+    for (; c < cend; c += 2 * GSK_WAVES) {
+        if (c + GSK_WAVES < cend) load(c + GSK_WAVES, 1);
+        mul(0);
+        if (c + GSK_WAVES < cend) {
+            if (c + 2 * GSK_WAVES < cend) load(c + 2 * GSK_WAVES, 0);
+            mul(1);
+        }
+    }
+#pragma unroll
+    for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) red[wave][tb][r][lane] = acc[tb][r];
+    __syncthreads();
+    auto wsum = [&](int tb, int r) { // fixed order
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < GSK_WAVES; w += 2) t += red[w][tb][r][lane] + red[w + 1][tb][r][lane];
+        return t;
+    };
+    const size_t tileFloats = 4 * 4 * 64;
+    float* myPart = partials + ((size_t)blockIdx.x * ks + kslice) * tileFloats;
+    if (ks > 1) {
+        if (wave < 4) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) g_ast(myPart + ((size_t)wave * 4 + r) * 64 + lane, wsum(wave, r));
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = __hip_atomic_fetch_add(counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            lastFlag = prev == (unsigned)(ks - 1);
+            if (lastFlag) __hip_atomic_store(counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        if (!lastFlag) return;
+    }
+    if (wave >= 4) return;
+    const int tb = wave; // one token block per wave
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        if (ks > 1) {
+            float sum = 0.f;
+            for (int q = 0; q < ks; q++) sum += g_ald(partials + ((size_t)blockIdx.x * ks + q) * tileFloats + ((size_t)tb * 4 + r) * 64 + lane);
+            v[r] = sum * alpha;
+        } else {
+            v[r] = wsum(tb, r) * alpha;
+        }
+    }
+    const int m = tb * 16 + n16, n = n0 + 4 * kq; // accumulator element r: weight row 4 (lane / 16) + r, token lane % 16
+    if (m >= M) return;
+    if (EPI == GEMM_EPI_SWIGLU) {
+#pragma unroll
+        for (int j = 0; j < 4; j += 2)
+            if (n + j + 1 < N) ((float*)Cv)[(size_t)m * ldc + ((n + j) >> 1)] = (v[j] / (1.0f + expf(-v[j]))) * v[j + 1];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (n + j < N) {
+                float o = v[j];
+                if (R) o += R[(size_t)m * ldr + n + j];
+                ((float*)Cv)[(size_t)m * ldc + n + j] = o;
+            }
+    }
+}
+
+static hipError_t launch_gemm_skinny16(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                                       const float* R, int ldr, int M, int N, int K, void* ws, float alpha) {
+    const int nblocks = (N + 15) / 16;
+    const int nchunks = (int)(((size_t)K * 4) / GKB);
+    int ks = 1;
+    if (ws && nblocks <= 64 && nchunks >= 32) { // few rows, long K: also split K over workgroups (see launch_gemm_skinny)
+        ks = std::min(std::min(8, 256 / nblocks), std::max(1, nchunks / GSK_WAVES));
+        if ((size_t)nblocks * ks > 256 * 8) ks = 1;
+    }
+    const dim3 grid(nblocks, ks);
+    unsigned* counters = (unsigned*)ws;
+    float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_skinny16<GEMM_EPI_SWIGLU>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const float*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
+    else
+        hipLaunchKernelGGL((k_gemm_skinny16<GEMM_EPI_PLAIN>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const float*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
+    return hipGetLastError();
+}
+
 // Workspace for split-K: GSK_COUNTERS zeroed counters, then the partial tiles.
 size_t mlh_gemm_workspace_bytes(void) { return (size_t)GSK_COUNTERS * 4 + (size_t)256 * 8 * 2 * 16 * 64 * 4; }
 
@@ -520,6 +647,8 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
         GEMM_BY_TYPE((launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<f16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)));
+    if (M <= 64 && dtype == MLH_DTYPE_F32 && N <= 16 * GSK_COUNTERS && (N + 31) / 32 < 200) // the 32-row tiles would leave compute units idle
+        return launch_gemm_skinny16(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha);
     if (M <= 64)
         GEMM_BY_TYPE((launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),

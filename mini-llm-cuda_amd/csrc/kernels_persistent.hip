@@ -955,6 +955,9 @@ __global__ void __launch_bounds__(PWG) k_decode_tagged(PersistArgs P) {
             }
             pf_first<WT>(pf, (const WT*)L.Wo, L.ad, d, L.ad, gw, TW);
             P_STAMP(ts + 4);
+            // the GDN phase keeps q and k in `stage`, which the next phase overwrites: every wave must be done with them
+            // (there is no grid barrier here to do that as a side effect)
+            lds_barrier();
 
             // ------------------------------------------------------------------ phase C
             {
