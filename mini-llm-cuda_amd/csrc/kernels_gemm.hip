@@ -482,11 +482,16 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny(const T* __restr
 // x K = 768 take one unit 5.8 us -- and a matrix of a few thousand rows in 32-row tiles occupies a third of the chip:
 // tiles of 16 rows double the units at work.  Lane l holds weight row l % 16 (token l % 16 of a block) and the
 // 16 bytes at K offset (l / 16) * 16 of each 64-byte half chunk; element e of those vectors meets element e.
-template <int EPI>
+// With NORM the rows of A are RMS-normalised on the way in (inference.cu:24-50): C = (gain * A / rms(A)) . B^T.  The gain
+// multiplies the elements as they are loaded, the sum of squares of a row is gathered from the same loads, and
+// 1 / rms scales the finished product, so the normalised activations are never written to memory (gridDim.y = 1).
+template <int EPI, bool NORM>
 __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb,
                                                                    void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
-                                                                   unsigned* counters, float* partials, float alpha) {
+                                                                   unsigned* counters, float* partials, float alpha,
+                                                                   const float* __restrict__ gain) {
     __shared__ float red[GSK_WAVES][4][4][64];
+    __shared__ float ssred[GSK_WAVES][4][16];
     __shared__ int lastFlag;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int n0 = blockIdx.x * 16, n16 = lane & 15, kq = lane >> 4;
@@ -500,16 +505,32 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
     f32x4 acc[4];
 #pragma unroll
     for (int tb = 0; tb < 4; tb++) acc[tb] = (f32x4)(0.f);
-    f32x4 fb[2][2], fa[2][4][2];
+    f32x4 fb[2][2], fa[2][4][2], fg[2][2];
+    float ss[4] = {0.f, 0.f, 0.f, 0.f}; // NORM: this lane's share of the sums of squares of its four tokens
+    const unsigned char* grow = reinterpret_cast<const unsigned char*>(gain) + kq * 16;
     auto load = [&](int c, int buf) {
 #pragma unroll
         for (int p = 0; p < 2; p++) fb[buf][p] = *reinterpret_cast<const f32x4*>(brow + (size_t)c * GKB + p * 64);
+        if (NORM) {
+#pragma unroll
+            for (int p = 0; p < 2; p++) fg[buf][p] = *reinterpret_cast<const f32x4*>(grow + (size_t)c * GKB + p * 64);
+        }
 #pragma unroll
         for (int tb = 0; tb < 4; tb++)
 #pragma unroll
             for (int p = 0; p < 2; p++) fa[buf][tb][p] = *reinterpret_cast<const f32x4*>(arow[tb] + (size_t)c * GKB + p * 64);
     };
     auto mul = [&](int buf) {
+        if (NORM) {
+#pragma unroll
+            for (int tb = 0; tb < 4; tb++)
+#pragma unroll
+                for (int p = 0; p < 2; p++) {
+                    const f32x4 x = fa[buf][tb][p];
+                    ss[tb] = fmaf(x.x, x.x, ss[tb]); ss[tb] = fmaf(x.y, x.y, ss[tb]); ss[tb] = fmaf(x.z, x.z, ss[tb]); ss[tb] = fmaf(x.w, x.w, ss[tb]);
+                    fa[buf][tb][p] = x * fg[buf][p];
+                }
+        }
 #pragma unroll
         for (int p = 0; p < 2; p++)
 #pragma unroll
@@ -531,6 +552,15 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
     for (int tb = 0; tb < 4; tb++)
 #pragma unroll
         for (int r = 0; r < 4; r++) red[wave][tb][r][lane] = acc[tb][r];
+    if (NORM) { // lanes n16, n16 + 16, + 32, + 48 hold the four K quarters of token n16
+#pragma unroll
+        for (int tb = 0; tb < 4; tb++) {
+            float t = ss[tb];
+            t += __shfl_xor(t, 16, 64);
+            t += __shfl_xor(t, 32, 64);
+            if (lane < 16) ssred[wave][tb][lane] = t;
+        }
+    }
     __syncthreads();
     auto wsum = [&](int tb, int r) { // fixed order
         float t = 0.f;
@@ -569,6 +599,14 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
         }
     }
     const int m = tb * 16 + n16, n = n0 + 4 * kq; // accumulator element r: weight row 4 (lane / 16) + r, token lane % 16
+    if (NORM) {
+        float t = 0.f;
+#pragma unroll
+        for (int w = 0; w < GSK_WAVES; w++) t += ssred[w][tb][n16];
+        const float ri = 1.0f / sqrtf(t / (float)K + 1e-8f);
+#pragma unroll
+        for (int r = 0; r < 4; r++) v[r] *= ri;
+    }
     if (m >= M) return;
     if (EPI == GEMM_EPI_SWIGLU) {
 #pragma unroll
@@ -586,21 +624,23 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
 }
 
 static hipError_t launch_gemm_skinny16(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                                       const float* R, int ldr, int M, int N, int K, void* ws, float alpha) {
+                                       const float* R, int ldr, int M, int N, int K, void* ws, float alpha, const float* normGain) {
     const int nblocks = (N + 15) / 16;
     const int nchunks = (int)(((size_t)K * 4) / GKB);
     int ks = 1;
-    if (ws && nblocks <= 64 && nchunks >= 32) { // few rows, long K: also split K over workgroups (see launch_gemm_skinny)
+    if (ws && !normGain && nblocks <= 64 && nchunks >= 32) { // few rows, long K: also split K over workgroups (see launch_gemm_skinny)
         ks = std::min(std::min(8, 256 / nblocks), std::max(1, nchunks / GSK_WAVES));
         if ((size_t)nblocks * ks > 256 * 8) ks = 1;
     }
     const dim3 grid(nblocks, ks);
     unsigned* counters = (unsigned*)ws;
     float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
-    if (epi == GEMM_EPI_SWIGLU)
-        hipLaunchKernelGGL((k_gemm_skinny16<GEMM_EPI_SWIGLU>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const float*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
-    else
-        hipLaunchKernelGGL((k_gemm_skinny16<GEMM_EPI_PLAIN>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const float*)B, ldb, C, ldc, R, ldr, M, N, K, counters, partials, alpha);
+#define SK16(EPI_, NORM_)                                                                                                     \
+    hipLaunchKernelGGL((k_gemm_skinny16<EPI_, NORM_>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const float*)B, ldb, \
+                       C, ldc, R, ldr, M, N, K, counters, partials, alpha, normGain)
+    if (epi == GEMM_EPI_SWIGLU) { if (normGain) SK16(GEMM_EPI_SWIGLU, true); else SK16(GEMM_EPI_SWIGLU, false); }
+    else { if (normGain) SK16(GEMM_EPI_PLAIN, true); else SK16(GEMM_EPI_PLAIN, false); }
+#undef SK16
     return hipGetLastError();
 }
 
@@ -633,12 +673,18 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
 // epi = GEMM_EPI_PLAIN: C fp32 [M, N] (+ R).  epi = GEMM_EPI_SWIGLU: C is [M, N/2] in the operand type.
 // ws: optional zero-initialised workspace of mlh_gemm_workspace_bytes() (enables split-K for M <= 64); launches that
 // share a workspace must be ordered on one stream.
+// True when mlh_gemm_tn_epi can take `normGain` for this shape (the RMSNorm of A's rows fused into the product).
+bool mlh_gemm_norm_fusable(int dtype, int M, int N) {
+    return dtype == MLH_DTYPE_F32 && M > 32 && M <= 64 && N <= 16 * GSK_COUNTERS && (N + 31) / 32 < 200;
+}
+
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
-                           const float* R, int ldr, int M, int N, int K, void* ws, float alpha) {
+                           const float* R, int ldr, int M, int N, int K, void* ws, float alpha, const float* normGain) {
     const size_t esz = dtype == MLH_DTYPE_F32 ? 4 : 2;
     if (M <= 0 || N <= 0 || K <= 0 || ((size_t)K * esz) % GKB != 0 || ((size_t)lda * esz) % 16 != 0 || ((size_t)ldb * esz) % 16 != 0)
         return hipErrorInvalidValue;
     if (epi == GEMM_EPI_SWIGLU && (N & 1)) return hipErrorInvalidValue;
+    if (normGain && !mlh_gemm_norm_fusable(dtype, M, N)) return hipErrorInvalidValue;
     // M <= 64 (one row per sequence of a decode batch): weight-streaming skinny kernel; long M: 256 x 256 tiles
     // fed by direct-to-LDS loads; in between: 128 x 128 tiles
 #define GEMM_BY_TYPE(call_f32, call_bf16, call_f16) \
@@ -647,8 +693,8 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
         GEMM_BY_TYPE((launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<f16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)));
-    if (M <= 64 && dtype == MLH_DTYPE_F32 && N <= 16 * GSK_COUNTERS && (N + 31) / 32 < 200) // the 32-row tiles would leave compute units idle
-        return launch_gemm_skinny16(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha);
+    if (M > 32 && M <= 64 && dtype == MLH_DTYPE_F32 && N <= 16 * GSK_COUNTERS && (N + 31) / 32 < 200) // the 32-row tiles would leave compute units idle
+        return launch_gemm_skinny16(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha, normGain);
     if (M <= 64)
         GEMM_BY_TYPE((launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),

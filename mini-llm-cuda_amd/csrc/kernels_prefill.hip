@@ -1355,32 +1355,43 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
     hipStream_t st = c->stream;
     const int d_ = hp.dim, F = hp.ffnDim, dt = c->gemmDtype, n = nseq;
     const bool bf = hp.weightDtype == MLH_DTYPE_BF16;
-#define GEMM(epi, A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K)                                                \
-    do {                                                                                                         \
-        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, c->gemmWs, alpha);  \
-        if (e_ != hipSuccess) { c->err = std::string("batched step GEMM: ") + hipGetErrorString(e_); return -2; } \
+#define GEMMN(epi, A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K, G)                                                 \
+    do {                                                                                                            \
+        hipError_t e_ = mlh_gemm_tn_epi(st, dt, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, c->gemmWs, alpha, G);  \
+        if (e_ != hipSuccess) { c->err = std::string("batched step GEMM: ") + hipGetErrorString(e_); return -2; }    \
     } while (0)
+#define GEMM(epi, A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K) GEMMN(epi, A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K, nullptr)
     if (bf) hipLaunchKernelGGL((k_bd_embed<bf16_t>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);
     else hipLaunchKernelGGL((k_bd_embed<float>), dim3(cdiv(d_, PWG), n), dim3(PWG), 0, st, a);
     for (int t = hp.transformers - 1; t >= 0; t--) {
         const LayerDev& L = c->layers[t];
-        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (f16_t*)c->pfXn, n, d_);
-        else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (float*)c->pfXn, n, d_);
-        GEMM(0, c->pfXn, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
+        // (fp32, 33..64 sequences: the RMSNorm rides in the product, see mlh_gemm_norm_fusable)
+        if (mlh_gemm_norm_fusable(dt, n, L.rowsA)) {
+            GEMMN(0, c->x, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_, L.g1);
+        } else {
+            if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (f16_t*)c->pfXn, n, d_);
+            else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (float*)c->pfXn, n, d_);
+            GEMM(0, c->pfXn, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
+        }
         int rc = mlh_launch_one(c, L.kind == MLH_KIND_ATTENTION ? MLH_K_ATTN : MLH_K_GDN, t, nseq);
         if (rc) return rc;
         if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd + hp.pleDim);
         else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
         GEMM(0, c->pfA, c->maxAd + hp.pleDim, L.WoG, L.sWo, L.ad + hp.pleDim, c->h1, d_, c->x, d_, n, d_, L.ad + hp.pleDim);
-        if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (f16_t*)c->pfXn, n, d_);
-        else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (float*)c->pfXn, n, d_);
-        GEMM(1, c->pfXn, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_);
+        if (mlh_gemm_norm_fusable(dt, n, 2 * F)) {
+            GEMMN(1, c->h1, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_, L.g2);
+        } else {
+            if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (f16_t*)c->pfXn, n, d_);
+            else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (float*)c->pfXn, n, d_);
+            GEMM(1, c->pfXn, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_);
+        }
         GEMM(0, c->pfU, F, L.W2G, L.sW2, F, c->x, d_, c->h1, d_, n, d_, F);
     }
     if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (f16_t*)c->pfXn, n, d_);
     else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, c->gF, (float*)c->pfXn, n, d_);
     GEMM(0, c->pfXn, d_, c->EG, c->sE, d_, c->pfLogits, hp.vocabSize, nullptr, 0, n, hp.vocabSize, d_);
 #undef GEMM
+#undef GEMMN
     hipLaunchKernelGGL(k_bd_finish, dim3(n), dim3(PWG), 0, st, a, c->pfLogits, c->d_tok);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { c->err = std::string("batched step launch: ") + hipGetErrorString(e); return -2; }
