@@ -356,15 +356,16 @@ __device__ __forceinline__ void issue_wo(XPf<WT>& pf, const WT* Wo, int ad, int 
         }
     }
 }
-// W2 columns [X fs, (X+1) fs): rows lw, lw + XLW, ...; four rows x two chunks per lane are prefetched (clamped likewise).
+// W2 columns [X fs, (X+1) fs): a wave takes blocks of four consecutive rows (block wb first); the first block, two
+// chunks per lane, is prefetched (clamped likewise).
 template <typename WT>
-__device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int fs, int F, int lw, int d) {
+__device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int fs, int F, int wb, int d) {
     constexpr int N = PVec<WT>::N;
     const int lane = threadIdx.x & 63, CR = fs / N;
     const unsigned lb0 = (unsigned)min(lane, CR - 1) * 16u, lb1 = (unsigned)min(lane + 64, CR - 1) * 16u;
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        const WT* rp = pin_uniform(W2 + (size_t)min(lw + XLW * k, d - 1) * F + (size_t)X * fs);
+        const WT* rp = pin_uniform(W2 + (size_t)min(wb * 4 + k, d - 1) * F + (size_t)X * fs);
         pf.r[k * 2] = load16<WT>(rp, lb0, 0u);
         pf.r[k * 2 + 1] = load16<WT>(rp, lb1, 0u);
     }
@@ -481,7 +482,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
                 xst(P.amax + 2 * wg, v, tagBase + (unsigned)step + 1);
                 xst(P.amax + 2 * wg + 1, __uint_as_float((unsigned)i), tagBase + (unsigned)step + 1);
             }
-            poll_vec<true, 8, true>(P.amax, 2 * (int)gridDim.x, tagBase + (unsigned)step + 1, S.scratch, P.abortFlag, ok);
+            poll_vec<true, 8, true>(P.amax, 2 * (int)gridDim.x, tagBase + (unsigned)step + 1, S.scratch, P.abortFlag, ok, P.nap[0] / 2);
             v = -3.0e38f; i = 0x7fffffff;
             for (int k = lane; k < (int)gridDim.x; k += 64) {
                 const float v2 = S.scratch[2 * k];
@@ -525,6 +526,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     const int d = a.dim, F = a.ffn, V = a.vocab, fs = P.fs;
     const int lane = threadIdx.x & 63, wave = uni(threadIdx.x >> 6), wg = blockIdx.x;
     const int lw = wave * XPER + r;             // worker wave within the XCD: consecutive rows land on different workgroups
+    const int wbE = r * XWORK + wave;           // first block of four W2 rows of this wave
     const int lwF = (XWORK - 1 - wave) * XPER + r; // the same in reverse wave order, for the FFN units: a second unit, where
                                                    // there is one, goes to the last waves, not to the attention waves
     const int gwl = wave * (int)gridDim.x + wg; // worker wave within the grid (LM head)
@@ -788,7 +790,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 }
             }
             W_STAMP(14);
-            issue_w2<WT>(s2, uni_ptr((const WT*)L.W2), X, fs, F, lw, d);
+            issue_w2<WT>(s2, uni_ptr((const WT*)L.W2), X, fs, F, wbE, d);
             X_BARRIER(); // 4
             // ------------------------------------------------------------------ phase D
             {
@@ -825,12 +827,15 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             X_BARRIER(); // 5
             // ------------------------------------------------------------------ phase E
             {
+                // four consecutive rows per wave, written with one store: 32 contiguous bytes towards the memory side
+                // instead of four separate words
                 const int CR = fs / N;
                 const WT* W2x = uni_ptr((const WT*)L.W2) + (size_t)X * fs;
+                if (wbE * 4 < d) {
+                    float val = 0.f;
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const int row = lw + XLW * k;
-                    if (row < d) {
+                    for (int k = 0; k < 4; k++) {
+                        const int row = min(wbE * 4 + k, d - 1);
                         float acc = 0.f;
 #pragma unroll
                         for (int c0 = 0; c0 < 2; c0++) {
@@ -840,15 +845,21 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                         for (int cc = lane + 128; cc < CR; cc += 64)
                             acc = chunk_dot_lds<WT>(PVec<WT>::load(W2x + (size_t)row * F + cc * N), S.us + cc * N, acc);
                         acc = pwave_sum(acc);
-                        if (lane == 0) xst(P.xP + (size_t)X * d + row, acc, lt); // inference.cu:283-291 (the readers add the residual)
+                        val = lane == k ? acc : val;
                     }
+                    if (lane < 4 && wbE * 4 + lane < d) xst(P.xP + (size_t)X * d + wbE * 4 + lane, val, lt); // inference.cu:283-291 (the readers add the residual)
                 }
-                for (int row = lw + 4 * XLW; row < d; row += XLW) {
-                    float acc = 0.f;
-                    for (int cc = lane; cc < CR; cc += 64)
-                        acc = chunk_dot_lds<WT>(PVec<WT>::load(W2x + (size_t)row * F + cc * N), S.us + cc * N, acc);
-                    acc = pwave_sum(acc);
-                    if (lane == 0) xst(P.xP + (size_t)X * d + row, acc, lt);
+                for (int b = wbE + XLW; b * 4 < d; b += XLW) {
+                    float val = 0.f;
+                    for (int k = 0; k < 4; k++) {
+                        const int row = min(b * 4 + k, d - 1);
+                        float acc = 0.f;
+                        for (int cc = lane; cc < CR; cc += 64)
+                            acc = chunk_dot_lds<WT>(PVec<WT>::load(W2x + (size_t)row * F + cc * N), S.us + cc * N, acc);
+                        acc = pwave_sum(acc);
+                        val = lane == k ? acc : val;
+                    }
+                    if (lane < 4 && b * 4 + lane < d) xst(P.xP + (size_t)X * d + b * 4 + lane, val, lt);
                 }
             }
             W_STAMP(9);
