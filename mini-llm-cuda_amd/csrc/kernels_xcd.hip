@@ -8,7 +8,7 @@
 //
 //   XCD X owns the attention heads h = X, X+8, ... and the FFN units [X F/8, (X+1) F/8).
 //   A  RMSNorm(x) and the q|k|v|gate rows of the XCD's heads           -> inside the XCD  (inference.cu:388-465)
-//   B  attention of those heads, split over 64-key tiles               -> inside the XCD  (inference.cu:467-573)
+//   B  attention of those heads, split over 32-key tiles               -> inside the XCD  (inference.cu:467-573)
 //   C  combine + gate, then the Wo product over the XCD's COLUMNS      -> partial h1, across XCDs
 //      (inference.cu:241-250, 582-610)
 //      every workgroup adds the eight partials of its 1/32 slice, publishes the slice inside the XCD
@@ -48,6 +48,8 @@
 #define XCB 24                  // softmax partials the communicator fetches per round
 #define XSPIN (1u << 20)
 #define XHD 64
+#define XTK 32                  // keys per attention unit (half a KV page)
+#define XTILE (XTK * XHD)       // floats of a K or V tile
 
 typedef unsigned long long u64;
 
@@ -371,7 +373,7 @@ __device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int f
     }
 }
 
-// K and V tile (64 rows x 64 floats each) of one head, rows below `lim`, global -> LDS without registers.  An
+// K and V tile (XTK rows x 64 floats each) of one head, rows below `lim`, global -> LDS without registers.  An
 // instruction moves 1 KB: lane i's 16 bytes land at base + 16 i, i.e. row 4q + i/16, slot i%16; the lane fetches the
 // piece that belongs there: for K under the swizzle slot = piece ^ (row & 15), which makes the per-lane row reads of
 // the score loop conflict-free; V stays row-major (the P.V loop reads a row across the lanes).  Kh, Vh: wave-uniform
@@ -379,7 +381,7 @@ __device__ __forceinline__ void issue_w2(XPf<WT>& pf, const WT* W2, int X, int f
 __device__ __forceinline__ void issue_kv_tile(const float* Kh, const float* Vh, int d, int lim, float* tK, float* tV) {
     const unsigned lane = threadIdx.x & 63u;
 #pragma unroll
-    for (int q = 0; q < 16; q++) {
+    for (int q = 0; q < XTK / 4; q++) {
         const unsigned row = 4 * q + (lane >> 4), piece = (lane & 15) ^ (row & 15);
         // row 4q of the tile is the wave-uniform part of the address, the lane adds (lane / 16) rows and its piece
         const char* Kq = pin_uniform(reinterpret_cast<const char*>(Kh + (size_t)(4 * q) * d));
@@ -536,8 +538,8 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     const int RA = np * nh * XHD;
     u64* qkvL = P.qkvL + (size_t)X * P.qkvStride;
     u64* partL = P.partL + (size_t)X * P.partStride;
-    float* tK = S.tiles + (wave < XAW ? wave : 0) * 8192;
-    float* tV = tK + 4096;
+    float* tK = S.tiles + (wave < XAW ? wave : 0) * (2 * XTILE);
+    float* tV = tK + XTILE;
     const int aslot = wave * XPER + r; // attention unit slot of this wave (waves below XAW only)
     const WT* E = (const WT*)a.E;
 
@@ -556,21 +558,21 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     // first K/V tile of this wave in layer Lx when the sequence holds npos rows, and the q/k gains of its head
     float gqv = 1.f, gkv = 1.f;
     // (the tile index of a wave's first unit never changes, so its page is looked up once)
-    const int pageFirst = (wave < XAW && nh > 0 && aslot / nh < a.pagesPerSeq) ? uni(a.pageTable[P.seq * a.pagesPerSeq + aslot / nh]) : 0;
+    const int pageFirst = (wave < XAW && nh > 0 && aslot / nh < 2 * a.pagesPerSeq) ? uni(a.pageTable[P.seq * a.pagesPerSeq + ((aslot / nh) >> 1)]) : 0;
     auto issueKV = [&](const LayerDev& Lx, int npos) {
-        const int nt = (npos + 64) >> 6;
+        const int nt = (npos + XTK) / XTK;
         if (aslot < nh * nt) {
             const int j = aslot % nh, tl = aslot / nh;
             if (a.qkNorm) {
                 gqv = uni_ptr(Lx.gq)[(X + XCDS * j) * XHD + lane];
                 gkv = uni_ptr(Lx.gk)[(X + XCDS * j) * XHD + lane];
             }
-            const size_t base = ((size_t)pageFirst * MLH_KV_PAGE) * d + (X + XCDS * j) * XHD;
-            issue_kv_tile(uni_ptr((const float*)Lx.K) + base, uni_ptr((const float*)Lx.V) + base, d, npos - tl * 64, tK, tV);
+            const size_t base = ((size_t)pageFirst * MLH_KV_PAGE + (tl & 1) * XTK) * d + (X + XCDS * j) * XHD;
+            issue_kv_tile(uni_ptr((const float*)Lx.K) + base, uni_ptr((const float*)Lx.V) + base, d, npos - tl * XTK, tK, tV);
         }
     };
     if (wave < XAW) { // the tiles must never hold anything but finite numbers (rows beyond the sequence get weight zero)
-        for (int i = lane * 4; i < 8192; i += 256) *reinterpret_cast<f32x4*>(tK + i) = (f32x4)(0.f);
+        for (int i = lane * 4; i < 2 * XTILE; i += 256) *reinterpret_cast<f32x4*>(tK + i) = (f32x4)(0.f);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
     {
@@ -580,17 +582,17 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
         if (wave < XAW) issueKV(L0, pos);
     }
 
-    float* qh = S.tiles + XAW * 8192 + (wave < XAW ? wave : 0) * 64; // this wave's query after norm and RoPE
+    float* qh = S.tiles + XAW * 2 * XTILE + (wave < XAW ? wave : 0) * 64; // this wave's query after norm and RoPE
     bool ok = true; // attention waves poll the softmax partials (bounded)
 
     for (int step = 0; step < P.steps; step++) {
-        const int T = pos + 1, ntiles = (T + 63) >> 6, newTile = pos >> 6;
+        const int T = pos + 1, ntiles = (T + XTK - 1) / XTK, newTile = pos / XTK;
         float rc = 1.f, rsn = 0.f; // RoPE of this step's position: lanes (2i, 2i+1) hold the pair i (inference.cu:113-134)
         int pageNew = 0; // page that receives this step's K/V row
         if (wave < XAW) {
             rc = a.rope[(size_t)pos * XHD + (lane & ~1)];
             rsn = a.rope[(size_t)pos * XHD + (lane | 1)];
-            pageNew = uni(a.pageTable[P.seq * a.pagesPerSeq + newTile]);
+            pageNew = uni(a.pageTable[P.seq * a.pagesPerSeq + (pos >> 6)]);
         }
         for (int t = P.NL - 1; t >= 0; t--) {
             const LayerDev& L = S.Ls[t];
@@ -641,10 +643,10 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 const bool dbg = P.timing && t == 0 && step == P.steps - 1 && lane == 0 && wave == 0;
                 if (dbg) P.timing[16 * (P.NL + 1) + 4 * wg + 1] = aslot < U ? wall_clock64() : 0;
                 for (int u = aslot; u < U; u += XAW * XPER) {
-                    const int j = u % nh, tl = u / nh, j0 = tl << 6, h = X + XCDS * j;
+                    const int j = u % nh, tl = u / nh, j0 = tl * XTK, h = X + XCDS * j;
                     if (u != aslot) { // tiles beyond the first one were not fetched ahead
-                        const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + tl]);
-                        const size_t base = ((size_t)page * MLH_KV_PAGE) * d + h * XHD;
+                        const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + (tl >> 1)]);
+                        const size_t base = ((size_t)page * MLH_KV_PAGE + (tl & 1) * XTK) * d + h * XHD;
                         issue_kv_tile(uni_ptr((const float*)L.K) + base, uni_ptr((const float*)L.V) + base, d, pos - j0, tK, tV);
                         if (a.qkNorm) { gqv = uni_ptr(L.gq)[h * XHD + lane]; gkv = uni_ptr(L.gk)[h * XHD + lane]; }
                     }
@@ -655,40 +657,44 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     if (u == aslot) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
                     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                     if (dbg) P.timing[16 * (P.NL + 1) + 4 * wg + 3] = wall_clock64();
-                    const int nv = T - j0 < 64 ? T - j0 : 64;       // keys of this tile, the new one included
+                    const int nv = T - j0 < XTK ? T - j0 : XTK;     // keys of this tile, the new one included
                     if (tl == newTile) { // this step's row comes from the first phase, not from the cache; it is appended here
                         const int rn = pos - j0;
                         const float kn = norm_rope(ksAll[j * XHD + lane], gkv), vn = vsAll[j * XHD + lane];
                         tK[rn * 64 + ((((lane >> 2) ^ (rn & 15)) << 2) | (lane & 3))] = kn;
                         tV[rn * 64 + lane] = vn;
                         // write-through: read from the next step on, by whichever workgroup of this XCD takes the tile
-                        const size_t o = ((size_t)pageNew * MLH_KV_PAGE + rn) * d + h * XHD + lane;
+                        const size_t o = ((size_t)pageNew * MLH_KV_PAGE + (pos & 63)) * d + h * XHD + lane;
                         ast(uni_ptr(L.K) + o, kn);
                         ast(uni_ptr(L.V) + o, vn);
                     }
                     __builtin_amdgcn_wave_barrier();
+                    // scores: lanes l and l + 32 share key l % 32, each takes half of the 64 dimensions
+                    const int key = lane & 31, dh = lane >> 5;
                     float s = 0.f;
                     {
-                        const float* kr = tK + lane * 64;
-#pragma unroll 8
-                        for (int p = 0; p < 16; p++) {
-                            const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + ((p ^ (lane & 15)) << 2));
-                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qh + p * 4);
+                        const float* kr = tK + key * 64;
+#pragma unroll
+                        for (int p = 0; p < 8; p++) {
+                            const int pp = p + 8 * dh;
+                            const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + ((pp ^ (key & 15)) << 2));
+                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qh + pp * 4);
                             s = fmaf(kk.x, qq.x, s); s = fmaf(kk.y, qq.y, s); s = fmaf(kk.z, qq.z, s); s = fmaf(kk.w, qq.w, s);
                         }
                     }
-                    const bool valid = lane < nv;
+                    s += __shfl_xor(s, 32, MLH_WAVE);
+                    const bool valid = key < nv;
                     s = valid ? s / sqrtf((float)XHD) : -1.0e30f; // inference.cu:154
                     const float m = pwave_max(s);
-                    const float e = valid ? expf(s - m) : 0.f;
+                    const float e = (valid && dh == 0) ? expf(s - m) : 0.f; // lanes 0..31 carry the weights
                     const float l = pwave_sum(e);
-                    // all 64 rows: rows from nv on hold older K/V rows or the zeros of the start of the kernel, and
+                    // all XTK rows: rows from nv on hold older K/V rows or the zeros of the start of the kernel, and
                     // their weights are zero.  Sixteen rows are fetched before they are used, so that the LDS latency
-                    // is paid four times, not sixty-four.
+                    // is paid twice, not once per row.
                     float acc = 0.f;
                     const float* vcol = tV + lane;
 #pragma unroll
-                    for (int jj0 = 0; jj0 < 64; jj0 += 16) {
+                    for (int jj0 = 0; jj0 < XTK; jj0 += 16) {
                         float vr[16];
 #pragma unroll
                         for (int i = 0; i < 16; i++) vr[i] = vcol[(jj0 + i) * 64];
@@ -923,7 +929,7 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     S.besti = reinterpret_cast<int*>(S.bestv + 16);
     S.ctl = S.besti + 16;               // [0] a wait expired, [1] next token
     S.tiles = reinterpret_cast<float*>(S.ctl + 16); // [XAW][K tile | V tile]
-    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 8192 + XAW * 64); // (after the tiles: one query vector per attention wave)
+    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 2 * XTILE + XAW * 64); // (after the tiles: one query vector per attention wave)
     for (int i = threadIdx.x; i < P.NL * (int)(sizeof(LayerDev) / 4); i += XWG)
         reinterpret_cast<uint32_t*>(S.Ls)[i] = reinterpret_cast<const uint32_t*>(P.layers)[i];
     if (threadIdx.x == 0) {
@@ -968,13 +974,13 @@ __global__ void k_xcd_zero(unsigned* p, size_t n) {
 static size_t xcd_lds_bytes(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
     const int fs = hp.ffnDim / XCDS;
-    return ((size_t)2 * hp.dim + 5 * XNH * XHD + ((fs + 3) & ~3) + 512 + 48 + XAW * 8192 + XAW * 64) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
+    return ((size_t)2 * hp.dim + 5 * XNH * XHD + ((fs + 3) & ~3) + 512 + 48 + XAW * 2 * XTILE + XAW * 64) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
 }
 
 // Exchange words (64-bit) the kernel needs for this model.
 size_t mlh_xcd_words(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
-    return (size_t)XCDS * (4 * XNH * XHD) + (size_t)XCDS * XNH * c->pagesPerSeq * (XHD + 2) + (size_t)4 * XCDS * hp.dim + hp.ffnDim +
+    return (size_t)XCDS * (4 * XNH * XHD) + (size_t)XCDS * XNH * (MLH_KV_PAGE / XTK) * c->pagesPerSeq * (XHD + 2) + (size_t)4 * XCDS * hp.dim + hp.ffnDim +
            2 * (size_t)XCDS * XPER + 64;
 }
 
@@ -1046,7 +1052,7 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     u64* t = c->xcdBuf;
     P.qkvStride = 4 * XNH * XHD;
     P.qkvL = t; t += (size_t)XCDS * P.qkvStride;
-    P.partStride = XNH * c->pagesPerSeq * (XHD + 2);
+    P.partStride = XNH * (MLH_KV_PAGE / XTK) * c->pagesPerSeq * (XHD + 2);
     P.partL = t; t += (size_t)XCDS * P.partStride;
     P.h1P = t; t += (size_t)XCDS * hp.dim;
     P.h1L = t; t += (size_t)XCDS * hp.dim;
