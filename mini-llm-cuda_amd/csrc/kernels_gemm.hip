@@ -177,9 +177,11 @@ __global__ void __launch_bounds__(GTHREADS) k_gemm_tn(const T* __restrict__ A, i
 // flight while slice s is multiplied, and one barrier per slice separates the stages.
 //
 // A direct load puts lane i's 16 bytes at (wave-uniform base) + 16 i, so rows cannot be padded.  The
-// 8 pieces of a 128-byte row are stored permuted instead: slot j of row r holds piece j ^ (r & 7)
-// -- the lane picks which piece it fetches, not where it lands.  Eight consecutive rows reading the
-// same piece then touch eight different 16-byte bank groups (one full 128-byte LDS beat).
+// 8 pieces of a 128-byte row are stored permuted instead: slot j of row r holds piece j ^ ((r >> 1) & 7)
+// -- the lane picks which piece it fetches, not where it lands.  The LDS serves 256 bytes (64 banks) per
+// cycle, i.e. sixteen lanes of a 16-byte read; two consecutive rows fill the 64 banks once, so sixteen
+// consecutive rows reading the same piece touch sixteen different 16-byte bank groups: even and odd rows
+// lie in different halves of the banks, and rows of equal parity differ in (r >> 1) & 7.
 // ----------------------------------------------------------------------------
 #define GB_T 256
 #define GB_STAGE (2 * GB_T * GKB) // bytes per stage: A rows then B rows
@@ -206,7 +208,7 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int r = wave * 32 + q * 8 + (lane >> 3);
-        const int pc = (lane & 7) ^ (r & 7);
+        const int pc = (lane & 7) ^ ((r >> 1) & 7);
         srcA[q] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(m0 + r, M - 1) * ldaB + pc * 16;
         srcB[q] = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + r, N - 1) * ldbB + pc * 16;
     }
@@ -226,8 +228,8 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
         for (int j = 0; j < GB_BN; j++) acc[i][j] = (f32x16)(0.f);
 
     const int half = lane >> 5, lrow = lane & 31;
-    // row offsets and swizzle keys of this lane's operand rows (row & 7 does not depend on the 32-row block)
-    const int keyA = (wm * 128 + lrow) & 7, keyB = (wn * 32 * GB_BN + lrow) & 7;
+    // row offsets and swizzle keys of this lane's operand rows ((row >> 1) & 7 does not depend on the 32-row block)
+    const int keyA = ((wm * 128 + lrow) >> 1) & 7, keyB = ((wn * 32 * GB_BN + lrow) >> 1) & 7;
     const int offA = (wm * 128 + lrow) * GKB, offB = GB_T * GKB + (wn * 32 * GB_BN + lrow) * GKB;
 
     issue(0, 0);
