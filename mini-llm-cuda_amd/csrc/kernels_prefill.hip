@@ -313,26 +313,48 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
     const float inv_scale = 1.0f / sqrtf((float)HD);
     const int ntiles = (maxPos >> 6) + 1;
 
-    for (int t = 0; t < ntiles; t++) {
+    // A tile's K and V rows travel global -> registers -> LDS; the loads of tile t + 1 are issued before tile t is
+    // multiplied, so their latency runs under the MFMAs.  Rows beyond the last position any query of the workgroup
+    // may see are read from a clamped row and zeroed (every load unconditional: all of them in flight at once).
+    constexpr int NK = 64 * (HD / 4) / PWG, NV = 32 * (HD / 4) / PWG;
+    f32x4 kreg[NK], vreg[NV][2];
+    auto fetch = [&](int t) {
         const int j0 = t << 6;
         const int page = a.pageTable[seq * a.pagesPerSeq + t];
         const size_t base = ((size_t)page * MLH_KV_PAGE) * a.dim + h * HD;
+        const int rmax = maxPos - j0; // >= 0
+#pragma unroll
+        for (int n = 0; n < NK; n++) {
+            const int i = tid + n * PWG, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+            kreg[n] = *reinterpret_cast<const f32x4*>(L.K + base + (size_t)min(r, rmax) * a.dim + c4);
+        }
+#pragma unroll
+        for (int n = 0; n < NV; n++) {
+            const int i = tid + n * PWG, kp = i & 7, g = (i >> 3) % (HD / 4), ko = (i >> 3) / (HD / 4);
+            const int k = 16 * ko + 2 * kp, c4 = 4 * g;
+            vreg[n][0] = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)min(k, rmax) * a.dim + c4);
+            vreg[n][1] = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)min(k + 1, rmax) * a.dim + c4);
+        }
+    };
+    fetch(0);
+    for (int t = 0; t < ntiles; t++) {
+        const int j0 = t << 6;
+        const int rmax = maxPos - j0;
         __syncthreads(); // the previous tile has been consumed
         // ---- K tile: natural layout ----
-        for (int i = tid; i < 64 * (HD / 4); i += PWG) {
-            const int r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
-            f32x4 kk = (f32x4)(0.f);
-            if (j0 + r <= maxPos) kk = *reinterpret_cast<const f32x4*>(L.K + base + (size_t)r * a.dim + c4);
+#pragma unroll
+        for (int n = 0; n < NK; n++) {
+            const int i = tid + n * PWG, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+            const f32x4 kk = r <= rmax ? kreg[n] : (f32x4)(0.f);
             u32x2 w; w.x = pack_f16(kk.x, kk.y); w.y = pack_f16(kk.z, kk.w);
             *reinterpret_cast<u32x2*>(Kt + r * KP + c4) = w;
         }
         // ---- V tile: transposed, keys in contraction-slot order; a lane carries two keys that are neighbours there ----
-        for (int i = tid; i < 32 * (HD / 4); i += PWG) {
-            const int kp = i & 7, g = (i >> 3) % (HD / 4), ko = (i >> 3) / (HD / 4); // key pair, column chunk, group of 8 pairs
+#pragma unroll
+        for (int n = 0; n < NV; n++) {
+            const int i = tid + n * PWG, kp = i & 7, g = (i >> 3) % (HD / 4), ko = (i >> 3) / (HD / 4); // key pair, column chunk, group of 8 pairs
             const int k = 16 * ko + 2 * kp, c4 = 4 * g;
-            f32x4 v0 = (f32x4)(0.f), v1 = (f32x4)(0.f);
-            if (j0 + k <= maxPos) v0 = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)k * a.dim + c4);
-            if (j0 + k + 1 <= maxPos) v1 = *reinterpret_cast<const f32x4*>(L.V + base + (size_t)(k + 1) * a.dim + c4);
+            const f32x4 v0 = k <= rmax ? vreg[n][0] : (f32x4)(0.f), v1 = k + 1 <= rmax ? vreg[n][1] : (f32x4)(0.f);
             const int slot = pv_slot(k); // even, and pv_slot(k + 1) == slot + 1
             *reinterpret_cast<uint32_t*>(Vt + (c4 + 0) * VP + slot) = pack_f16(v0.x, v1.x);
             *reinterpret_cast<uint32_t*>(Vt + (c4 + 1) * VP + slot) = pack_f16(v0.y, v1.y);
@@ -340,6 +362,7 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
             *reinterpret_cast<uint32_t*>(Vt + (c4 + 3) * VP + slot) = pack_f16(v0.w, v1.w);
         }
         __syncthreads();
+        if (t + 1 < ntiles) fetch(t + 1);
         if (!waveActive || j0 > waveMaxPos) continue; // wave-uniform; the barriers above are still reached by every wave
         // ---- S^T = K . Q^T for the two 32-key blocks ----
         f32x16 sacc[2];
@@ -620,7 +643,10 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     {
         const float* src = P.QKV + (size_t)row0 * P.qkvLd + (sel ? L.offK : 0) + h * DK + cidx;
 #pragma unroll
-        for (int t = 0; t < GD_C; t++) colv[t] = t < nv ? src[(size_t)t * P.qkvLd] : 0.f;
+        for (int t = 0; t < GD_C; t++) { // unconditional loads of clamped rows: 64 loads in flight, no branch per row
+            const float v = src[(size_t)min(t, nv - 1) * P.qkvLd];
+            colv[t] = t < nv ? v : 0.f;
+        }
     }
     if (tid < GD_C) { // gates
         const int t = tid;
@@ -702,8 +728,11 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     float X[GD_C];
     const int col = cidx;
     if (tid < DV) {
+        const float* vsrc = P.QKV + (size_t)row0 * P.qkvLd + L.offV + h * DV + col;
 #pragma unroll
-        for (int t = 0; t < GD_C; t++) X[t] = t < nv ? beta[t] * P.QKV[(size_t)(row0 + t) * P.qkvLd + L.offV + h * DV + col] : 0.f;
+        for (int t = 0; t < GD_C; t++) X[t] = vsrc[(size_t)min(t, nv - 1) * P.qkvLd]; // all 64 loads in flight at once
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) X[t] *= beta[t]; // beta is zero for tokens past the segment end
     } else {
 #pragma unroll
         for (int t = 0; t < GD_C; t++) X[t] = beta[t] * eg[t] * colv[t];
