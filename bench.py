@@ -181,6 +181,20 @@ def prefill_leg(m, reps=2):
             "decode_after_prefill": {"sequences": nseq, "ms_per_step": dec * 1e3, "tok_s": nseq / dec}}
 
 
+def gemm_leg(m, iters=3):
+    """The gate/up product of one config-5 prefill pass alone (16384 x 11264 x 2048, half operands, plain epilogue):
+    the launch the operand-path counters of the big GEMM kernel are collected on."""
+    hp = m.config(5)
+    M = 8 * 2048
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((M, hp.dim), dtype=np.float32)
+    b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
+    _, us = m.selftest_gemm(a, b, None, f16=True, iters=iters)
+    tf = 2.0 * M * 2 * hp.ffnDim * hp.dim / us / 1e6
+    return {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "avg_us": us, "TFLOPs": tf,
+            "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
+
+
 def timed_decode(dev, prompt, K, W, persistent, maxL):
     """W untimed warm-up steps, then exactly K timed steps with the device idle on both sides.
     Returns (wall seconds, HIP-event milliseconds of a second identical run, ids)."""
@@ -213,8 +227,8 @@ def main():
     ap.add_argument("--path", choices=["xcd", "persistent", "kernels", "tagged"], default="xcd",
                     help="decode path reported as `value`")
     ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
-    ap.add_argument("--leg", choices=["all", "batched", "prefill"], default="all",
-                    help="profiler runs: run only the batched-decode or the prefill leg and print its JSON object")
+    ap.add_argument("--leg", choices=["all", "batched", "prefill", "gemm"], default="all",
+                    help="profiler runs: run only the batched-decode leg, the prefill leg or the big GEMM alone and print its JSON object")
     ap.add_argument("--only-path", action="store_true", help="time only the chosen path (for profiler runs)")
     ap.add_argument("--graph-steps", type=int, default=0,
                     help="kernels path: decode steps per hipGraph replay; 0 = plain launches (use 0 under rocprofv3)")
@@ -226,7 +240,8 @@ def main():
 
     m = entry.load_package()
     if args.leg != "all":
-        print(json.dumps({args.leg: batched_decode_leg(m) if args.leg == "batched" else prefill_leg(m, reps=1)}))
+        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=1), "gemm": gemm_leg}[args.leg]
+        print(json.dumps({args.leg: leg(m)}))
         return 0
     hp = m.config(2)
     K, W = max(1, args.steps), max(0, args.warmup)
