@@ -518,7 +518,24 @@ __global__ void __launch_bounds__(WG) k_gdn(StepArgs a, LayerDev L) {
 #pragma unroll
     for (int c = 0; c < CPT; c += 4)
         *reinterpret_cast<float4*>(Srow + c) = make_float4(S[c], S[c + 1], S[c + 2], S[c + 3]);
-    if (cg == 0) a.mix[(size_t)slot * (a.gdnHeads * DV) + h * DV + r] = oacc;
+    if (!a.mixRows) {
+        if (cg == 0) a.mix[(size_t)slot * (a.gdnHeads * DV) + h * DV + r] = oacc;
+        return;
+    }
+    // batched step: the read-out is a row segment of the output-projection GEMM's input; the workgroup of head 0 also
+    // appends the PLE columns e = silu(gate) * P[tok] behind the gdnHeads * DV read-out columns
+    const size_t row = (size_t)slot * a.mixRowsLd;
+    auto put_row = [&](size_t col, float v) {
+        if (a.mixRowsHalf) ((_Float16*)a.mixRows)[row + col] = (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f); // saturating
+        else ((float*)a.mixRows)[row + col] = v;
+    };
+    if (cg == 0) put_row((size_t)h * DV + r, oacc);
+    if (h == 0)
+        for (int j = tid; j < a.ple; j += WG) {
+            const size_t e = (size_t)a.tok[slot] * a.ple + j;
+            const float p = a.wbytes == 2 ? __uint_as_float(((uint32_t)((const uint16_t*)L.pleTable)[e]) << 16) : ((const float*)L.pleTable)[e];
+            put_row((size_t)a.gdnHeads * DV + j, siluf_ref(qkv[L.offPle + j]) * p);
+        }
 }
 
 // ----------------------------------------------------------------------------
@@ -820,6 +837,7 @@ void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr) {
     a.nseq = nseq; a.sidx = c->d_sidx; a.tok = tokPtr; a.pos = c->d_pos;
     a.pageTable = c->d_pageTable; a.pagesPerSeq = c->pagesPerSeq; a.nsplit = c->nsplit;
     a.x = c->x; a.qkv = c->qkv; a.qkvStride = c->maxRowsA; a.part = c->part; a.mix = c->mix;
+    a.mixRows = c->mixRows; a.mixRowsLd = c->mixRowsLd; a.mixRowsHalf = c->mixRowsHalf; a.wbytes = c->wbytes;
     a.h1 = c->h1; a.u = c->u; a.logits = c->logits; a.amaxVal = c->amaxVal; a.amaxIdx = c->amaxIdx;
     a.amaxParts = c->amaxParts; a.rope = c->rope; a.E = c->E; a.gF = c->gF;
     a.nextTok = c->d_next; a.outIds = c->d_outIds; a.stepCounter = c->d_stepCounter; a.outCapacity = c->outCapacity;

@@ -1402,10 +1402,18 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
             else hipLaunchKernelGGL((k_pf_rmsnorm<float>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (float*)c->pfXn, n, d_);
             GEMM(0, c->pfXn, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_);
         }
-        int rc = mlh_launch_one(c, L.kind == MLH_KIND_ATTENTION ? MLH_K_ATTN : MLH_K_GDN, t, nseq);
+        const bool gdn = L.kind != MLH_KIND_ATTENTION;
+        // The GDN kernel writes its read-out and the PLE columns straight into the GEMM's input rows (mlh_launch_one
+        // reads the step's tokens from the context's own buffer, hence the second condition).
+        const bool direct = gdn && tokPtr == c->d_tok;
+        if (direct) { c->mixRows = c->pfA; c->mixRowsLd = c->maxAd + hp.pleDim; c->mixRowsHalf = bf ? 1 : 0; }
+        int rc = mlh_launch_one(c, gdn ? MLH_K_GDN : MLH_K_ATTN, t, nseq);
+        c->mixRows = nullptr;
         if (rc) return rc;
-        if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd + hp.pleDim);
-        else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
+        if (!direct) { // attention: combine the split-KV partials, gate; PLE columns
+            if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd + hp.pleDim);
+            else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
+        }
         GEMM(0, c->pfA, c->maxAd + hp.pleDim, L.WoG, L.sWo, L.ad + hp.pleDim, c->h1, d_, c->x, d_, n, d_, L.ad + hp.pleDim);
         if (mlh_gemm_norm_fusable(dt, n, 2 * F)) {
             GEMMN(1, c->h1, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_, L.g2);

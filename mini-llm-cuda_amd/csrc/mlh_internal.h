@@ -65,6 +65,10 @@ struct StepArgs {
     int qkvStride;
     float* part;          // [slots, nsplit, heads, hd + 2] attention partials (m, l, acc)
     float* mix;           // [slots, maxAd] GDN read-out
+    void* mixRows;        // batched step: if set, the GDN read-out and the PLE columns go straight into the rows of the
+    int mixRowsLd;        //   output-projection GEMM (leading dimension in elements, fp32 or IEEE half) instead of `mix`
+    int mixRowsHalf;
+    int wbytes;           // bytes per weight element (PLE table rows)
     float* h1;            // [slots, dim]
     float* u;             // [slots, ffn]
     float* logits;        // [maxSeqs, vocab] indexed by sequence id
@@ -97,6 +101,8 @@ struct mlh_ctx {
     float* gF = nullptr;
     float* rope = nullptr;
 
+    void* mixRows = nullptr; // see StepArgs::mixRows; set by the batched step around its GDN launches
+    int mixRowsLd = 0, mixRowsHalf = 0;
     int pagesPerSeq = 0;
     int nsplit = 1;
     int maxRowsA = 0, maxAd = 0;
