@@ -301,10 +301,15 @@ def main():
         # the dominant (only) kernel: one launch = K tokens; duration from HIP events around the launch
         launch_us = chosen["event_ms_per_step"] * K * 1e3
         launch_bytes = mean_bytes * K
+        # HBM bytes per launch: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one run each), scaled by what the same
+        # counters read for the 256 MiB copy kernel (reads x 2.0, writes x 1.0), measured on a 16-token launch of the
+        # XCD-rank kernel (the profiler does not survive the 512-token launch): 381.7 MB read + 3.4 MB written per
+        # token against 370.4 MB algorithmic at those lengths.  Not measured for the barrier kernels.
+        traffic_ratio = {"xcd": 1.04}.get(args.path)
         roofline = {"kernel": {"persistent": "k_decode_persistent", "tagged": "k_decode_tagged", "xcd": "k_decode_xcd"}[args.path], "bound": "hbm", "achieved": launch_bytes / launch_us / 1e3,
                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": launch_bytes / launch_us / 1e3 / HBM_PEAK_GBPS,
-                    "traffic": None, "avg_launch_us": launch_us, "algo_bytes_per_launch": launch_bytes,
-                    "tokens_per_launch": K}
+                    "traffic": traffic_ratio * launch_bytes if traffic_ratio else None, "avg_launch_us": launch_us,
+                    "algo_bytes_per_launch": launch_bytes, "tokens_per_launch": K}
     else:
         # dominant = the kernel with the largest share of the step's time
         dom = max(kernels, key=lambda k: kernels[k]["avg_us_in_sequence"] * kernels[k]["launches_per_token"])
