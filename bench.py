@@ -140,6 +140,31 @@ def batched_decode_leg(m, steps=64):
             "last_ids": [int(x) for x in out[-1, :4]]}
 
 
+def hybrid_decode_leg(m, steps=256):
+    """Configuration 3: batch-1 greedy decode of the hybrid architecture (3 GDN : 1 attention + PLE) after a
+    128-token prompt.  Returns tok/s and the fraction of the bytes-per-token roofline (weights, GDN states read and
+    written, K/V rows of the attention layers)."""
+    hp = m.config(3)
+    hp.maxSeqs = 1
+    plen, warm = 128, 16
+    model = m.Model.generate(hp, seed=3)
+    dev = m.Device(hp, 0)
+    dev.upload(model)
+    dev.prefill(0, m.random_tokens(3, 0, hp.vocabSize, plen))
+    out = dev.decode_loop([dev.greedy_token(0)], warm)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    out = dev.decode_loop([int(out[-1, 0])], steps)
+    dev.synchronize()
+    wall = time.perf_counter() - t0
+    nbytes = float(np.mean([decode_bytes_per_token(hp, plen + warm + 1 + i) for i in range(steps)]))
+    dev.close()
+    return {"workload": "config 3: batch-1 greedy decode, hybrid 3 GDN : 1 attention + PLE at config-2 size, fp32, "
+                        "128-token prompt", "steps": steps, "ms_per_step": wall / steps * 1e3, "tok_s": steps / wall,
+            "bytes_per_token": nbytes, "achieved_GBps": nbytes / (wall / steps) / 1e9,
+            "frac_of_hbm_peak": nbytes / (wall / steps) / 1e9 / HBM_PEAK_GBPS, "last_ids": [int(x) for x in out[-4:, 0]]}
+
+
 def prefill_leg(m, reps=2):
     """Configuration 5: 8 prompts of 2048 uniform-random tokens through the bf16 model in one pass.
     MFMA utilisation = algorithmic flops (projections + causal attention, LM head on the last position
@@ -227,8 +252,9 @@ def main():
     ap.add_argument("--path", choices=["xcd", "persistent", "kernels", "tagged"], default="xcd",
                     help="decode path reported as `value`")
     ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
-    ap.add_argument("--leg", choices=["all", "batched", "prefill", "gemm"], default="all",
-                    help="profiler runs: run only the batched-decode leg, the prefill leg or the big GEMM alone and print its JSON object")
+    ap.add_argument("--leg", choices=["all", "batched", "prefill", "gemm", "hybrid"], default="all",
+                    help="profiler runs: run only the batched-decode leg, the prefill leg, the big GEMM alone or the "
+                         "batch-1 hybrid decode leg and print its JSON object")
     ap.add_argument("--only-path", action="store_true", help="time only the chosen path (for profiler runs)")
     ap.add_argument("--graph-steps", type=int, default=0,
                     help="kernels path: decode steps per hipGraph replay; 0 = plain launches (use 0 under rocprofv3)")
@@ -240,7 +266,8 @@ def main():
 
     m = entry.load_package()
     if args.leg != "all":
-        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=1), "gemm": gemm_leg}[args.leg]
+        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=1), "gemm": gemm_leg,
+               "hybrid": hybrid_decode_leg}[args.leg]
         print(json.dumps({args.leg: leg(m)}))
         return 0
     hp = m.config(2)
@@ -336,7 +363,7 @@ def main():
     dev.close()
     extras = {}
     if not args.no_extras and not args.only_path:
-        for name, leg in (("batched_decode", batched_decode_leg), ("prefill", prefill_leg)):
+        for name, leg in (("batched_decode", batched_decode_leg), ("hybrid_decode", hybrid_decode_leg), ("prefill", prefill_leg)):
             try:
                 extras[name] = leg(m)
             except Exception as e:  # reported alongside, never required for the headline line

@@ -48,6 +48,7 @@
 #define XCB 24                  // softmax partials the communicator fetches per round
 #define XSPIN (1u << 20)
 #define XHD 64
+#define XQX 16                  // extra first-phase rows per XCD in hybrid models: two gate scalars per GDN head + PLE gate rows
 #define XTK 32                  // keys per attention unit (half a KV page)
 #define XTILE (XTK * XHD)       // floats of a K or V tile
 
@@ -341,6 +342,21 @@ __device__ __forceinline__ int rowA_of(int offK, int offV, int offG, int X, int 
     return off + (X + XCDS * j) * XHD + i;
 }
 
+// The same for models with gated-delta-net layers and per-layer embeddings: behind the q | k | v | gate rows come
+// the two gate scalars of every GDN head of the XCD (alpha rows, then beta rows) and the XCD's share (pleX) of the
+// PLE gate rows.
+__device__ __forceinline__ int rowA_hyb(const LayerDev& L, int X, int nh, int np, int pleX, int rho) {
+    const int rq = np * nh * XHD;
+    if (rho < rq) return rowA_of(uni(L.offK), uni(L.offV), uni(L.offG), X, nh, rho);
+    int e = rho - rq;
+    if (uni(L.kind) != MLH_KIND_ATTENTION) {
+        if (e < nh) return uni(L.offGa) + X + XCDS * e;
+        if (e < 2 * nh) return uni(L.offGb) + X + XCDS * (e - nh);
+        e -= 2 * nh;
+    }
+    return uni(L.offPle) + X * pleX + e;
+}
+
 // Wo columns of the XCD's heads: a pass covers N rows per wave (64/N lanes per 64-column head segment).  Rows
 // and heads beyond the end are clamped to the last valid one (loaded, never used).
 template <typename WT>
@@ -397,6 +413,7 @@ __device__ __forceinline__ void issue_kv_tile(const float* Kh, const float* Vh, 
 
 struct XShared {
     float *xs, *h1s, *qkvs, *as, *us, *scratch, *bestv, *tiles;
+    float *es, *gst; // hybrid models: the XCD's PLE values of the layer; this workgroup's GDN state rows [layer][4][64]
     int *besti, *ctl;
     LayerDev* Ls;
 };
@@ -412,7 +429,7 @@ struct XShared {
     } while (0)
 
 // ------------------------------------------------------------------------------------------------ communicator
-template <typename WT>
+template <typename WT, bool HYB>
 __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
     const StepArgs& a = P.a;
     const int d = a.dim, V = a.vocab;
@@ -443,7 +460,12 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
             X_BARRIER(); // 1: x in LDS
 
             // q | k | v | gate rows of the XCD's heads, as the workers produced them; the attention waves take it from there
-            poll_vec<false, 8, false>(qkvL, RA, lt, S.qkvs, P.abortFlag, ok, P.nap[2]);
+            int RAL = RA;
+            if constexpr (HYB) {
+                const bool gdnL = uni(L.kind) != MLH_KIND_ATTENTION;
+                RAL = (gdnL ? 3 : np) * nh * XHD + (gdnL ? 2 * nh : 0) + a.ple / XCDS;
+            }
+            poll_vec<false, 8, false>(qkvL, RAL, lt, S.qkvs, P.abortFlag, ok, P.nap[2]);
             if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
             X_STAMP(ts + 2);
             X_BARRIER(); // 2: q, k, v, gate in LDS
@@ -521,7 +543,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
 }
 
 // ------------------------------------------------------------------------------------------------ workers
-template <typename WT, int NCH>
+template <typename WT, int NCH, bool HYB>
 __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
     constexpr int N = PVec<WT>::N, CPS = XHD / N;
     const StepArgs& a = P.a;
@@ -536,6 +558,18 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
     const int np = 3 + (a.gating ? 1 : 0);
     const int RA = np * nh * XHD;
+    const int pleX = HYB ? a.ple / XCDS : 0; // PLE columns of this XCD
+    // rows of the first phase in layer Lx (hybrid models: fewer parts and two gate scalars per head in a GDN layer,
+    // the PLE gate rows in every layer)
+    auto rowsA = [&](const LayerDev& Lx) {
+        if constexpr (!HYB) return RA;
+        const bool g = uni(Lx.kind) != MLH_KIND_ATTENTION;
+        return (g ? 3 : np) * nh * XHD + (g ? 2 * nh : 0) + pleX;
+    };
+    auto rowA = [&](const LayerDev& Lx, int rho) {
+        if constexpr (HYB) return rowA_hyb(Lx, X, nh, uni(Lx.kind) != MLH_KIND_ATTENTION ? 3 : np, pleX, rho);
+        else return rowA_of(uni(Lx.offK), uni(Lx.offV), uni(Lx.offG), X, nh, rho);
+    };
     u64* qkvL = P.qkvL + (size_t)X * P.qkvStride;
     u64* partL = P.partL + (size_t)X * P.partStride;
     float* tK = S.tiles + (wave < XAW ? wave : 0) * (2 * XTILE);
@@ -548,10 +582,10 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     XGain<WT, NCH> gn;
     // first-phase rows lw, lw + XLW, ... of layer Lx and its first gain vector
     auto issueA = [&](const LayerDev& Lx) {
-        const int offK = uni(Lx.offK), offV = uni(Lx.offV), offG = uni(Lx.offG);
+        const int ra = rowsA(Lx);
         int rows[XS1];
 #pragma unroll
-        for (int k = 0; k < XS1; k++) rows[k] = nh > 0 ? rowA_of(offK, offV, offG, X, nh, min(lw + XLW * k, RA - 1)) : 0;
+        for (int k = 0; k < XS1; k++) rows[k] = nh > 0 ? rowA(Lx, min(lw + XLW * k, ra - 1)) : 0;
         issue_rows<WT, XS1, NCH>(s1.r, uni_ptr((const WT*)Lx.Wa), d, rows);
         issue_gain<WT, NCH>(gn, uni_ptr(Lx.g1));
     };
@@ -575,11 +609,44 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
         for (int i = lane * 4; i < 2 * XTILE; i += 256) *reinterpret_cast<f32x4*>(tK + i) = (f32x4)(0.f);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
+    // hybrid models: the PLE up-projection columns of this XCD for the first two passes of the output projection
+    // (lane c of a row group holds column X pleX + c), fetched together with the Wo columns
+    float plw[2] = {0.f, 0.f};
+    float plv = 0.f; // wave 0, lane c < pleX: the token's PLE table value for the coming layer
+    auto issuePlw = [&](const LayerDev& Lx) {
+        if constexpr (HYB) {
+            if (pleX > 0) {
+                const int rs = lane / CPS, c = min(lane % CPS, pleX - 1);
+                const WT* up = uni_ptr((const WT*)Lx.pleUp);
+#pragma unroll
+                for (int p = 0; p < 2; p++) plw[p] = PVec<WT>::one(up + (size_t)min((p * XLW + lw) * N + rs, d - 1) * a.ple + X * pleX + c);
+            }
+        }
+    };
+    auto issuePlv = [&](const LayerDev& Lx, int token) {
+        if constexpr (HYB) {
+            if (pleX > 0 && wave == 0) plv = PVec<WT>::one(uni_ptr((const WT*)Lx.pleTable) + (size_t)token * a.ple + X * pleX + min(lane, pleX - 1));
+        }
+    };
+    // hybrid models: wave w < 2 nh owns state row r 2nh + w of the XCD's GDN heads in every GDN layer; the rows stay
+    // in LDS for the whole launch (lane = column) and go back to memory at its end
+    const int grow = r * 2 * nh + wave;         // row among the 64 nh state rows of the XCD
+    const bool gwave = HYB && wave < 2 * nh;
+    float* gst = S.gst + (size_t)wave * XHD + lane; // + layer * 4 * XHD
+    auto stateRow = [&](const LayerDev& Lx) {
+        return uni_ptr(Lx.S) + (((size_t)P.seq * a.gdnHeads + (X + XCDS * (grow >> 6))) * XHD + (grow & 63)) * XHD + lane;
+    };
+    if constexpr (HYB) {
+        if (gwave)
+            for (int t = 0; t < P.NL; t++)
+                if (uni(S.Ls[t].kind) != MLH_KIND_ATTENTION) gst[(size_t)t * 4 * XHD] = *stateRow(S.Ls[t]);
+    }
     {
         const LayerDev& L0 = S.Ls[P.NL - 1];
         issueA(L0);
         issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
-        if (wave < XAW) issueKV(L0, pos);
+        issuePlw(L0);
+        if (wave < XAW && (!HYB || uni(L0.kind) == MLH_KIND_ATTENTION)) issueKV(L0, pos);
     }
 
     float* qh = S.tiles + XAW * 2 * XTILE + (wave < XAW ? wave : 0) * 64; // this wave's query after norm and RoPE
@@ -594,10 +661,14 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             rsn = a.rope[(size_t)pos * XHD + (lane | 1)];
             pageNew = uni(a.pageTable[P.seq * a.pagesPerSeq + (pos >> 6)]);
         }
+        issuePlv(S.Ls[P.NL - 1], tok);
         for (int t = P.NL - 1; t >= 0; t--) {
             const LayerDev& L = S.Ls[t];
             const unsigned lt = tagBase + (unsigned)(step * P.NL + (P.NL - 1 - t) + 1);
             const bool lastLayer = t == 0;
+            const bool gdnL = HYB && uni(L.kind) != MLH_KIND_ATTENTION;
+            const int RAL = rowsA(L);                       // rows of the first phase in this layer
+            const int RAq = (gdnL ? 3 : np) * nh * XHD;     // of which q | k | v | gate
             const LayerDev& Ln = S.Ls[lastLayer ? P.NL - 1 : t - 1];
             X_BARRIER(); // 1
             const int ts = (P.NL - 1 - t) * 16;
@@ -611,16 +682,15 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
 #pragma unroll
                 for (int k = 0; k < XS1; k++) {
                     const int rho = lw + XLW * k;
-                    if (rho < RA) {
+                    if (rho < RAL) {
                         const float acc = pwave_sum(row_dot_reg<WT, NCH>(s1.r, k, xn));
                         if (lane == 0) lst(qkvL + rho, acc, lt);
                     }
                 }
-                if (lw + XS1 * XLW < RA) {
-                    const int offK = uni(L.offK), offV = uni(L.offV), offG = uni(L.offG);
+                if (lw + XS1 * XLW < RAL) {
                     const WT* Wa = uni_ptr((const WT*)L.Wa);
-                    for (int rho = lw + XS1 * XLW; rho < RA; rho += XLW) {
-                        const float acc = pwave_sum(row_dot_stream<WT, NCH>(Wa, d, rowA_of(offK, offV, offG, X, nh, rho), xn));
+                    for (int rho = lw + XS1 * XLW; rho < RAL; rho += XLW) {
+                        const float acc = pwave_sum(row_dot_stream<WT, NCH>(Wa, d, rowA(L, rho), xn));
                         if (lane == 0) lst(qkvL + rho, acc, lt);
                     }
                 }
@@ -628,7 +698,51 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             W_STAMP(11);
             X_BARRIER(); // 2
             // ------------------------------------------------------------------ phase B
-            if (wave < XAW) {
+            if constexpr (HYB) {
+                if (pleX > 0 && wave == 0) { // e = silu(gate) * P[tok] for the XCD's PLE columns (inference-side PLE rule of k_oproj)
+                    if (lane < pleX) S.es[lane] = psilu(S.qkvs[RAL - pleX + lane]) * plv;
+                    if (!(lastLayer)) issuePlv(Ln, tok); // the last layer's successor belongs to the next token
+                }
+                if (gdnL) {
+                    // gated delta rule on this wave's state row (k_gdn of the kernel sequence, one row per wave, lane = column):
+                    //   u = S k ; S <- alpha (S - beta u k^T) + beta v k^T ; o = S q   with q, k L2-normalised
+                    if (gwave) {
+                        const int j = grow >> 6, i = grow & 63, h = X + XCDS * j;
+                        const float* qsA = S.qkvs;
+                        const float qc = qsA[j * XHD + lane], kc = qsA[nh * XHD + j * XHD + lane];
+                        const float vr = qsA[2 * nh * XHD + j * XHD + i];
+                        const float rq = sqrtf(pwave_sum(qc * qc) + 1e-6f), rk = sqrtf(pwave_sum(kc * kc) + 1e-6f);
+                        const float za = qsA[RAq + j] + uni_ptr(L.gdnBa)[h], zb = qsA[RAq + nh + j] + uni_ptr(L.gdnBb)[h];
+                        const float sp = fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)));
+                        const float alpha = expf(-sp), beta = psigmoid(zb);
+                        const float kn = kc / rk, qn = qc / rq;
+                        float* sp_ = gst + (size_t)t * 4 * XHD;
+                        float sv = *sp_;
+                        const float u = pwave_sum(sv * kn);
+                        sv = alpha * (sv - beta * u * kn) + beta * vr * kn;
+                        const float o = pwave_sum(sv * qn);
+                        *sp_ = sv;
+                        if (lane == 0) lst(partL + grow, o, lt);
+                    }
+                    // the read-outs of a head's 64 rows come from 32 / nh workgroups: one head per wave gathers them
+                    for (int j = wave; j < nh; j += XAW) {
+                        if (wave >= XAW) break;
+                        const u64* ub = pin_uniform(partL + (size_t)j * XHD);
+                        u64 w = 0;
+                        for (unsigned spins = 0;; spins++) {
+                            asm volatile("" ::: "memory");
+                            w = ldw<false>(ub, (unsigned)lane * 8u, 0u);
+                            if (__all((unsigned)(w >> 32) == lt)) break;
+                            if (!ok || spins > XSPIN || ((spins & 255) == 255 && aldu(P.abortFlag))) { ok = false; break; }
+                        }
+                        S.as[j * XHD + lane] = __uint_as_float((unsigned)w);
+                    }
+                    if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
+                    if (wave < XAW && !(lastLayer && step == P.steps - 1) && uni(Ln.kind) == MLH_KIND_ATTENTION)
+                        issueKV(Ln, lastLayer ? pos + 1 : pos);
+                }
+            }
+            if (wave < XAW && !gdnL) {
                 const int U = nh * ntiles;
                 const float* qsAll = S.qkvs; // rows as the first phase produced them
                 const float* ksAll = qsAll + nh * XHD;
@@ -761,7 +875,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 W_STAMP(15);
                 if (!ok) { S.ctl[0] = 1; astu(P.abortFlag, 1u); }
                 // first tile of this wave for the next layer pass (the next step's first layer sees one more row)
-                if (!(lastLayer && step == P.steps - 1)) issueKV(Ln, lastLayer ? pos + 1 : pos);
+                if (!(lastLayer && step == P.steps - 1) && (!HYB || uni(Ln.kind) == MLH_KIND_ATTENTION)) issueKV(Ln, lastLayer ? pos + 1 : pos);
             }
             // gate/up rows of this wave's first two FFN units, and the second gain vector
             {
@@ -791,6 +905,13 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                                 : PVec<WT>::load(uni_ptr((const WT*)L.Wo) + (size_t)row * ad + (X + XCDS * j) * XHD + c * N);
                             acc = chunk_dot_lds<WT>(w, S.as + j * XHD + c * N, acc);
                         }
+                    if constexpr (HYB) { // + pleUp . e over the XCD's PLE columns (one column per lane of the row group)
+                        if (pleX > 0) {
+                            const float w = p == 0 ? plw[0] : p == 1 ? plw[1]
+                                                  : PVec<WT>::one(uni_ptr((const WT*)L.pleUp) + (size_t)row * a.ple + X * pleX + min(c, pleX - 1));
+                            if (c < pleX) acc = fmaf(w, S.es[c], acc);
+                        }
+                    }
                     acc = pgroup_sum<CPS>(acc);
                     if (c == 0) xst(P.h1P + (size_t)X * d + row, acc, lt);
                 }
@@ -871,6 +992,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             W_STAMP(9);
             if (!lastLayer) {
                 issue_wo<WT>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, a.heads, lw, d);
+                issuePlw(Ln);
             } else {
                 // two more LM-head rows; the second register set has room for them when a row has at most 4 chunks
                 const int rows[2] = {min(gwl + XS1 * TWL, V - 1), min(gwl + (XS1 + 1) * TWL, V - 1)};
@@ -904,16 +1026,22 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             const LayerDev& L0 = S.Ls[P.NL - 1];
             issueA(L0);
             issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
+            issuePlw(L0);
         }
         X_BARRIER(); // best logits in LDS
         X_BARRIER(); // next token in LDS
         tok = S.ctl[1];
         pos += 1;
     }
+    if constexpr (HYB) {
+        if (gwave)
+            for (int t = 0; t < P.NL; t++)
+                if (uni(S.Ls[t].kind) != MLH_KIND_ATTENTION) *const_cast<float*>(stateRow(S.Ls[t])) = gst[(size_t)t * 4 * XHD];
+    }
     (void)tok;
 }
 
-template <typename WT, int NCH>
+template <typename WT, int NCH, bool HYB>
 __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     extern __shared__ float lds[];
     const StepArgs& a = P.a;
@@ -922,7 +1050,7 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     S.xs = lds;
     S.h1s = S.xs + d;
     S.qkvs = S.h1s + d;                 // [4][nh * 64] q | k | v | gate of the XCD's heads
-    S.as = S.qkvs + 4 * XNH * XHD;      // [nh * 64] mixing output
+    S.as = S.qkvs + 4 * XNH * XHD + XQX; // [nh * 64] mixing output (XQX: room for the extra first-phase rows of hybrid models)
     S.us = S.as + XNH * XHD;            // [fs]
     S.scratch = S.us + ((P.fs + 3) & ~3); // [max(d / 4, 2 * grid)]
     S.bestv = S.scratch + 512;
@@ -930,6 +1058,8 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     S.ctl = S.besti + 16;               // [0] a wait expired, [1] next token
     S.tiles = reinterpret_cast<float*>(S.ctl + 16); // [XAW][K tile | V tile]
     S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 2 * XTILE + XAW * 64); // (after the tiles: one query vector per attention wave)
+    S.es = reinterpret_cast<float*>(S.Ls + P.NL);
+    S.gst = S.es + 16;                  // hybrid models only: [NL][4][64]
     for (int i = threadIdx.x; i < P.NL * (int)(sizeof(LayerDev) / 4); i += XWG)
         reinterpret_cast<uint32_t*>(S.Ls)[i] = reinterpret_cast<const uint32_t*>(P.layers)[i];
     if (threadIdx.x == 0) {
@@ -953,8 +1083,8 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     const int X = uni(S.ctl[2]), r = uni(S.ctl[3]);
     const int tok = uni(a.tok[0]), pos = uni(a.pos[P.seq]);
     const unsigned tagBase = *P.tagCounter; // tags never repeat from launch to launch: nothing has to be cleared
-    if (wave == XWORK) xcd_communicator<WT>(P, S, tok, pos, tagBase, X, r);
-    else xcd_worker<WT, NCH>(P, S, tok, pos, tagBase, X, r);
+    if (wave == XWORK) xcd_communicator<WT, HYB>(P, S, tok, pos, tagBase, X, r);
+    else xcd_worker<WT, NCH, HYB>(P, S, tok, pos, tagBase, X, r);
 }
 
 // before every launch: abort flag and per-XCD arrival counters
@@ -971,28 +1101,42 @@ __global__ void k_xcd_zero(unsigned* p, size_t n) {
 // ----------------------------------------------------------------------------
 // host side
 // ----------------------------------------------------------------------------
+// hybrid model: gated-delta-net layers or per-layer embeddings (the HYB instantiation of the kernel)
+static bool xcd_hybrid(const mlh_ctx* c) {
+    const mlh_hparams& hp = c->hp;
+    if (hp.pleDim > 0) return true;
+    for (int t = 0; t < hp.transformers; t++)
+        if (hp.layerKinds[t] != MLH_KIND_ATTENTION) return true;
+    return false;
+}
+
 static size_t xcd_lds_bytes(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
     const int fs = hp.ffnDim / XCDS;
-    return ((size_t)2 * hp.dim + 5 * XNH * XHD + ((fs + 3) & ~3) + 512 + 48 + XAW * 2 * XTILE + XAW * 64) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
+    return ((size_t)2 * hp.dim + 5 * XNH * XHD + XQX + ((fs + 3) & ~3) + 512 + 48 + XAW * 2 * XTILE + XAW * 64 + 16 +
+            (xcd_hybrid(c) ? (size_t)hp.transformers * 4 * XHD : 0)) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
 }
 
 // Exchange words (64-bit) the kernel needs for this model.
 size_t mlh_xcd_words(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
-    return (size_t)XCDS * (4 * XNH * XHD) + (size_t)XCDS * XNH * (MLH_KV_PAGE / XTK) * c->pagesPerSeq * (XHD + 2) + (size_t)4 * XCDS * hp.dim + hp.ffnDim +
+    return (size_t)XCDS * (4 * XNH * XHD + XQX) + (size_t)XCDS * XNH * (MLH_KV_PAGE / XTK) * c->pagesPerSeq * (XHD + 2) + (size_t)4 * XCDS * hp.dim + hp.ffnDim +
            2 * (size_t)XCDS * XPER + 64;
 }
 
-// True when the XCD-rank kernel supports this context's shape: attention layers only, head size 64, no PLE,
-// a 256-unit chip, rows that fit the register sets.
+// True when the XCD-rank kernel supports this context's shape: head size 64 (attention heads, and GDN heads with
+// 64 x 64 states, as many as attention heads), PLE columns that split evenly over the XCDs, a 256-unit chip, rows
+// that fit the register sets.
 bool mlh_xcd_supported(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
     if (c->numCUs != XCDS * XPER || !c->xcdWords) return false;
-    for (int t = 0; t < hp.transformers; t++)
-        if (hp.layerKinds[t] != MLH_KIND_ATTENTION) return false;
     const int N = hp.weightDtype == MLH_DTYPE_BF16 ? 8 : 4;
-    if (hp.headDim != XHD || hp.pleDim != 0) return false;
+    bool gdn = false;
+    for (int t = 0; t < hp.transformers; t++) gdn = gdn || hp.layerKinds[t] != MLH_KIND_ATTENTION;
+    if (gdn && (hp.gdnDk != XHD || hp.gdnDv != XHD || hp.gdnHeads != hp.attnHeads || hp.attnHeads < XCDS || hp.attnHeads > 2 * XCDS)) return false; // (four state rows per workgroup and layer)
+    if (hp.pleDim % XCDS || hp.pleDim / XCDS > XHD / N || 2 * XNH + hp.pleDim / XCDS > XQX) return false;
+    if (hp.pleDim > 0 && hp.attnHeads < XCDS) return false;
+    if (hp.headDim != XHD) return false;
     if (hp.dim != hp.attnHeads * XHD || hp.dim > 4 * 64 * N || hp.dim % (64 * N) || hp.dim % XPER) return false;
     if (hp.attnHeads > XCDS * XNH) return false;
     if (hp.ffnDim % (XCDS * N)) return false;
@@ -1000,16 +1144,20 @@ bool mlh_xcd_supported(const mlh_ctx* c) {
     return xcd_lds_bytes(c) <= 160 * 1024;
 }
 
-template <typename WT, int NCH>
-static int launch_xcd(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
-    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+template <typename WT, int NCH, bool HYB>
+static int launch_xcd_as(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
+    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH, HYB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
     int perCu = 0;
-    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH>, XWG, ldsBytes));
+    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH, HYB>, XWG, ldsBytes));
     if (perCu < 1) { c->err = "XCD-rank decode kernel does not fit on a compute unit"; return -1; }
     // one workgroup per compute unit, all resident at once (the occupancy query says each unit can hold one); waits are bounded
-    hipLaunchKernelGGL((k_decode_xcd<WT, NCH>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
+    hipLaunchKernelGGL((k_decode_xcd<WT, NCH, HYB>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
     MLH_CHECK(c, hipGetLastError());
     return 0;
+}
+template <typename WT, int NCH>
+static int launch_xcd(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
+    return xcd_hybrid(c) ? launch_xcd_as<WT, NCH, true>(c, P, ldsBytes) : launch_xcd_as<WT, NCH, false>(c, P, ldsBytes);
 }
 
 // Puts the exchange words and the tag counter back to zero (after a launch that gave up a wait).
@@ -1050,7 +1198,7 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
         }
     }
     u64* t = c->xcdBuf;
-    P.qkvStride = 4 * XNH * XHD;
+    P.qkvStride = 4 * XNH * XHD + XQX;
     P.qkvL = t; t += (size_t)XCDS * P.qkvStride;
     P.partStride = XNH * (MLH_KV_PAGE / XTK) * c->pagesPerSeq * (XHD + 2);
     P.partL = t; t += (size_t)XCDS * P.partStride;

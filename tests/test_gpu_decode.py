@@ -97,14 +97,29 @@ def test_config1_golden_horizon(pkg, orc, persistent):
     dev.close()
 
 
-@pytest.mark.parametrize("case", ["heads12", "bf16_dim512", "two_combine_batches", "shuffled_pages"])
+@pytest.mark.parametrize("case", ["heads12", "bf16_dim512", "two_combine_batches", "shuffled_pages", "hybrid12",
+                                  "hybrid8_flags", "hybrid8_bf16", "attention8_ple", "hybrid12_no_ple"])
 def test_xcd_rank_kernel_shapes(pkg, orc, case):
     """The XCD-rank kernel on the shapes its work split distinguishes: XCDs with two heads and with one
     (12 heads over 8 XCDs), bf16 weights (8 values per 16-byte chunk), more softmax partials per XCD than
-    one combine round fetches, and a shuffled page table; several launches in a row (the tags run on)."""
-    bf16 = case == "bf16_dim512"
+    one combine round fetches, and a shuffled page table; several launches in a row (the tags run on).
+    Hybrid models: gated-delta-net layers whose state rows stay in LDS from launch to launch end and return to
+    memory in between (3 GDN : 1 attention and 1 : 1, with and without the flags), PLE columns split over the XCDs
+    (with GDN layers, with attention layers only), GDN layers without PLE, bf16 weights."""
+    bf16 = case in ("bf16_dim512", "hybrid8_bf16")
     kw = dict(transformers=2, vocabSize=1024, headDim=64)
-    if bf16:
+    if case.startswith("hybrid") or case == "attention8_ple":
+        heads = 12 if "12" in case else 8
+        hkw = dict(dim=64 * heads, attnHeads=heads, gdnHeads=heads, headDim=64, ffnDim=512, transformers=4, vocabSize=1024, maxL=200)
+        if case == "hybrid8_flags":
+            hkw.update(qkRmsNorm=1, queryGating=1)
+        if case == "hybrid12_no_ple":
+            hkw.update(pleDim=0)
+        if bf16:
+            hkw.update(weightDtype=pkg.DTYPE_BF16)
+        hp = pkg.config(3, **hkw)
+        pkg.set_layer_pattern(hp, {"hybrid12": 3, "hybrid8_flags": 1, "hybrid8_bf16": 1, "attention8_ple": 0, "hybrid12_no_ple": 3}[case])
+    elif bf16:
         hp = pkg.config(1, dim=512, attnHeads=8, ffnDim=1024, maxL=200, weightDtype=pkg.DTYPE_BF16, **kw)
     elif case == "two_combine_batches":
         hp = pkg.config(1, dim=768, attnHeads=12, ffnDim=512, maxL=900, qkRmsNorm=1, queryGating=1, **kw)
