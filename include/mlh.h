@@ -181,8 +181,9 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
  * unit free; their waits are bounded, and a call whose wait expired returns -3 with a message.
  * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says.
  * Mode 3 treats each of the eight XCDs as a tensor-parallel rank (heads and FFN units are split over the
- * XCDs, exchanges inside an XCD go through its L2, only two per layer cross XCDs); it covers models of
- * attention layers with head size 64 and no per-layer embeddings on a 256-unit device
+ * XCDs, exchanges inside an XCD go through its L2, only two per layer cross XCDs); it covers models with
+ * head size 64 (attention heads; gated-delta-net heads with 64 x 64 states, as many as attention heads;
+ * per-layer embeddings of a width that is a multiple of 8) on a 256-unit device
  * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default. */
 int mlh_set_persistent(mlh_ctx* ctx, int mode);
 

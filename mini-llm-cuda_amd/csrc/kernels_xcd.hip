@@ -16,6 +16,12 @@
 //   E  W2 product over the XCD's F/8 columns                           -> partial x, across XCDs (inference.cu:675-699)
 //   LM head rows over all workgroups, argmax across XCDs                                  (inference.cu:705-743)
 //
+// Hybrid models (template flag HYB; these layer kinds have no counterpart in inference.cu, they follow the kernel
+// sequence's k_gdn and k_oproj): a gated-delta-net layer keeps the five phases; A also yields the two gate scalars
+// of each of the XCD's heads, B is the delta rule on state rows (one row per wave, lane = column, the row resident
+// in LDS for the whole launch) followed by a gather of the 64 read-outs of a head inside the XCD.  The PLE gate
+// rows are split over the XCDs in A, e = silu(gate) * P[tok] is formed in B, and C adds the XCD's pleUp columns.
+//
 // Every exchanged value is one 64-bit word (value, tag): the tag is the number of the layer pass that
 // produced it, the buffers start at zero, and a consumer reads until the tag is there, so data arrival is
 // the synchronisation and a late or stale read only costs another read.  Every exchange is all-to-all
