@@ -67,11 +67,10 @@ struct XcdArgs {
     unsigned* abortFlag;
     unsigned* tagCounter;   // tags already used by earlier launches (advanced by workgroup 0 at the end)
     unsigned* xcdCount;     // [XCDS] zero at launch: workgroups that have arrived on each XCD
-    int maxTiles;
     int fs;                 // FFN units per XCD
     // exchange words: L = read inside the XCD that wrote them ([XCDS] regions), P = partials read by every XCD
-    u64* qkvL; int qkvStride;   // [XCDS][4 * XNH * 64]
-    u64* partL; int partStride; // [XCDS][XNH * maxTiles * 66]
+    u64* qkvL; int qkvStride;   // [XCDS][4 * XNH * 64 + XQX]
+    u64* partL; int partStride; // [XCDS][XNH * (32-key tiles of the longest sequence) * 66]; GDN layers: the read-outs [64 nh]
     u64* h1P;                   // [XCDS][d]
     u64* h1L;                   // [XCDS][d]
     u64* uL;                    // [XCDS][fs]
@@ -1188,7 +1187,6 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.abortFlag = c->d_sync + 64 * 20;
     P.tagCounter = c->d_sync + 64 * 21;
     P.xcdCount = c->d_sync + 64 * 22;
-    P.maxTiles = c->pagesPerSeq;
     P.fs = hp.ffnDim / XCDS;
     P.timing = c->d_timing;
     {
