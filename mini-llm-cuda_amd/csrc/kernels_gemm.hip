@@ -625,6 +625,112 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
     }
 }
 
+// The weight-streaming kernel for M <= 32 with the RMSNorm of the activation rows fused in (one 32-row tile, no split
+// over K): A holds the fp32 residual rows; a lane multiplies its elements by the gain on the way into the operand
+// registers (rounded to half for half weights), adds up their squares, and 1 / rms scales the result:
+//   W . (g (.) x / rms(x)) = (W . (g (.) x)) / rms(x),   rms(x) = sqrt(sum x^2 / K + 1e-8)   (inference.cu:24-50, 83-95)
+// T is the weight operand type (float, or f16_t for the half mirrors of a bf16 model).
+template <typename T, int EPI>
+__global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny_norm(const float* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
+                                                               void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
+                                                               float alpha, const float* __restrict__ gain) {
+    constexpr int EPC = GKB / (int)sizeof(T), HPC = EPC / 2, NV = HPC / 4; // elements per chunk, per lane half, 16-byte loads of fp32
+    __shared__ float red[GSK_WAVES][1][16][64];
+    __shared__ float ssq[GSK_WAVES][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n0 = blockIdx.x * 32, n32 = lane & 31, half = lane >> 5;
+    const int nchunks = (int)(((size_t)K * sizeof(T)) / GKB);
+    const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n32, N - 1) * ldb * sizeof(T) + half * 64;
+    const float* arow = A + (size_t)min(n32, M - 1) * lda + half * HPC;
+    const float* grow = gain + half * HPC;
+    f32x16 acc = (f32x16)(0.f);
+    float ss = 0.f;
+    u32x4 fb[2][4];
+    f32x4 xa[2][NV], ga[2][NV];
+    auto load = [&](int c, int buf) {
+#pragma unroll
+        for (int p = 0; p < 4; p++) fb[buf][p] = *reinterpret_cast<const u32x4*>(brow + (size_t)c * GKB + p * 16);
+#pragma unroll
+        for (int q = 0; q < NV; q++) {
+            xa[buf][q] = *reinterpret_cast<const f32x4*>(arow + (size_t)c * EPC + 4 * q);
+            ga[buf][q] = *reinterpret_cast<const f32x4*>(grow + (size_t)c * EPC + 4 * q);
+        }
+    };
+    auto half2 = [](float lo, float hi) { // two floats -> two IEEE halves, saturating
+        const _Float16 a = (_Float16)fminf(fmaxf(lo, -65504.0f), 65504.0f), b = (_Float16)fminf(fmaxf(hi, -65504.0f), 65504.0f);
+        return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+    };
+    auto mul = [&](int buf) {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            u32x4 fa;
+            if constexpr (sizeof(T) == 4) {
+                const f32x4 x = xa[buf][p], g = ga[buf][p];
+                ss = fmaf(x.x, x.x, ss); ss = fmaf(x.y, x.y, ss); ss = fmaf(x.z, x.z, ss); ss = fmaf(x.w, x.w, ss);
+                fa.x = __float_as_uint(g.x * x.x); fa.y = __float_as_uint(g.y * x.y); fa.z = __float_as_uint(g.z * x.z); fa.w = __float_as_uint(g.w * x.w);
+            } else {
+                const f32x4 x0 = xa[buf][2 * p], x1 = xa[buf][2 * p + 1], g0 = ga[buf][2 * p], g1 = ga[buf][2 * p + 1];
+                ss = fmaf(x0.x, x0.x, ss); ss = fmaf(x0.y, x0.y, ss); ss = fmaf(x0.z, x0.z, ss); ss = fmaf(x0.w, x0.w, ss);
+                ss = fmaf(x1.x, x1.x, ss); ss = fmaf(x1.y, x1.y, ss); ss = fmaf(x1.z, x1.z, ss); ss = fmaf(x1.w, x1.w, ss);
+                fa.x = half2(g0.x * x0.x, g0.y * x0.y); fa.y = half2(g0.z * x0.z, g0.w * x0.w);
+                fa.z = half2(g1.x * x1.x, g1.y * x1.y); fa.w = half2(g1.z * x1.z, g1.w * x1.w);
+            }
+            GemmTraits<T>::mma(fb[buf][p], fa, acc);
+        }
+    };
+    int c = wave;
+    if (c < nchunks) load(c, 0);
+    for (; c < nchunks; c += 2 * GSK_WAVES) { // two chunks per trip so the buffers are addressed statically
+        if (c + GSK_WAVES < nchunks) load(c + GSK_WAVES, 1);
+        mul(0);
+        if (c + GSK_WAVES < nchunks) {
+            if (c + 2 * GSK_WAVES < nchunks) load(c + 2 * GSK_WAVES, 0);
+            mul(1);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) red[wave][0][i][lane] = acc[i];
+    ssq[wave][lane] = ss;
+    __syncthreads();
+    // token m = n32: the squares of its row are spread over the waves and the two lane halves (fixed summation order)
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < GSK_WAVES; w++) tot += ssq[w][n32] + ssq[w][n32 + 32];
+    const float scale = alpha / sqrtf(tot / (float)K + 1e-8f);
+    for (int g = wave; g < 4; g += GSK_WAVES) {
+        const int i4 = g;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = red_sum(red, 0, 4 * i4 + j, lane) * scale;
+        const int m = n32, n = n0 + 8 * i4 + 4 * half; // accumulator element i: weight row 8 (i / 4) + 4 half + i % 4, column m
+        if (m >= M) continue;
+        if (EPI == GEMM_EPI_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2)
+                if (n + j + 1 < N) GemmTraits<T>::put((T*)Cv + (size_t)m * ldc + ((n + j) >> 1), (v[j] / (1.0f + expf(-v[j]))) * v[j + 1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (n + j < N) {
+                    float o = v[j];
+                    if (R) o += R[(size_t)m * ldr + n + j];
+                    ((float*)Cv)[(size_t)m * ldc + n + j] = o;
+                }
+        }
+    }
+}
+
+template <typename T>
+static hipError_t launch_gemm_skinny_norm(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                                          const float* R, int ldr, int M, int N, int K, float alpha, const float* normGain) {
+    const dim3 grid((N + 31) / 32);
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_skinny_norm<T, GEMM_EPI_SWIGLU>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);
+    else
+        hipLaunchKernelGGL((k_gemm_skinny_norm<T, GEMM_EPI_PLAIN>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);
+    return hipGetLastError();
+}
+
 static hipError_t launch_gemm_skinny16(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                                        const float* R, int ldr, int M, int N, int K, void* ws, float alpha, const float* normGain) {
     const int nblocks = (N + 15) / 16;
@@ -677,6 +783,10 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
 // share a workspace must be ordered on one stream.
 // True when mlh_gemm_tn_epi can take `normGain` for this shape (the RMSNorm of A's rows fused into the product).
 bool mlh_gemm_norm_fusable(int dtype, int M, int N) {
+    // k_gemm_skinny_norm (A is the fp32 residual for both operand types).  With half weights its register need allows
+    // one workgroup per compute unit, where the plain kernel runs two: a matrix of more than 256 row blocks would
+    // take two rounds and lose more than the saved RMSNorm launch brings.
+    if (M <= 32) return dtype == MLH_DTYPE_F32 || (dtype == MLH_GEMM_F16 && (N + 31) / 32 <= 256);
     return dtype == MLH_DTYPE_F32 && M > 32 && M <= 64 && N <= 16 * GSK_COUNTERS && (N + 31) / 32 < 200;
 }
 
@@ -691,6 +801,9 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
     // fed by direct-to-LDS loads; in between: 128 x 128 tiles
 #define GEMM_BY_TYPE(call_f32, call_bf16, call_f16) \
     return dtype == MLH_DTYPE_BF16 ? (call_bf16) : dtype == MLH_GEMM_F16 ? (call_f16) : (call_f32)
+    if (M <= 32 && normGain)
+        return dtype == MLH_GEMM_F16 ? launch_gemm_skinny_norm<f16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain)
+                                     : launch_gemm_skinny_norm<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);
     if (M <= 32)
         GEMM_BY_TYPE((launch_gemm_skinny<float, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<bf16_t, 1>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),

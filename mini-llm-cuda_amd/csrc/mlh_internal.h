@@ -189,8 +189,9 @@ hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, co
 // ws: zero-initialised workspace of mlh_gemm_workspace_bytes() or null; with it, M <= 64 products of matrices
 // with few rows are split along K over workgroups (deterministically reduced).
 // alpha scales the product before the epilogue (the power of two an fp16 weight mirror was scaled by, inverted).
-// normGain (fp32, 32 < M <= 64, see mlh_gemm_norm_fusable): A holds raw rows and the product is taken of
-// gain * A / rms(A) (the RMSNorm of the rows, eps 1e-8 inside the root), without a pass that writes the normalised rows.
+// normGain (M <= 64 for fp32 operands, M <= 32 for half operands, see mlh_gemm_norm_fusable): A holds the raw fp32
+// rows -- also when the weights are half -- and the product is taken of gain * A / rms(A) (the RMSNorm of the rows,
+// eps 1e-8 inside the root), without a pass that writes the normalised rows.
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                            const float* R, int ldr, int M, int N, int K, void* ws, float alpha = 1.0f, const float* normGain = nullptr);
 bool mlh_gemm_norm_fusable(int dtype, int M, int N);
