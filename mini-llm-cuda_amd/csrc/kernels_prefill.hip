@@ -1298,9 +1298,12 @@ template <typename WT, typename AT>
 __global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix, int aLd) {
     const int slot = blockIdx.x, tid = threadIdx.x;
     const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
+    // the row is dealt to the gridDim.y workgroups of the slot in contiguous pieces (one workgroup per slot would
+    // walk every head's partials alone)
+    const int piece = (L.ad + (int)gridDim.y - 1) / (int)gridDim.y, i0 = (int)blockIdx.y * piece, i1 = min(L.ad, i0 + piece);
     if (L.kind == MLH_KIND_ATTENTION) {
         const int hd = a.hd;
-        for (int i = tid; i < L.ad; i += PWG) {
+        for (int i = i0 + tid; i < i1; i += PWG) {
             const int h = i / hd, e = i - h * hd;
             const float* pp = a.part + (((size_t)slot * a.nsplit) * a.heads + h) * (hd + 2);
             const size_t sstride = (size_t)a.heads * (hd + 2);
@@ -1317,9 +1320,10 @@ __global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix
             put<AT>(Amix + (size_t)slot * aLd + i, v);
         }
     } else {
-        for (int i = tid; i < L.ad; i += PWG) put<AT>(Amix + (size_t)slot * aLd + i, a.mix[(size_t)slot * L.ad + i]);
+        for (int i = i0 + tid; i < i1; i += PWG) put<AT>(Amix + (size_t)slot * aLd + i, a.mix[(size_t)slot * L.ad + i]);
     }
-    for (int j = tid; j < a.ple; j += PWG)
+    if (blockIdx.y == 0)
+        for (int j = tid; j < a.ple; j += PWG)
         put<AT>(Amix + (size_t)slot * aLd + L.ad + j, pf_silu(qkv[L.offPle + j]) * getw<WT>((const WT*)L.pleTable + (size_t)a.tok[slot] * a.ple + j));
 }
 
@@ -1411,8 +1415,9 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
         c->mixRows = nullptr;
         if (rc) return rc;
         if (!direct) { // attention: combine the split-KV partials, gate; PLE columns
-            if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), dim3(n), dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd + hp.pleDim);
-            else hipLaunchKernelGGL((k_bd_mix<float, float>), dim3(n), dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
+            const dim3 mg(n, std::max(1, (L.ad + PWG - 1) / PWG * (n <= 16 ? 4 : 1))); // few slots: more workgroups per row
+            if (bf) hipLaunchKernelGGL((k_bd_mix<bf16_t, f16_t>), mg, dim3(PWG), 0, st, a, L, (f16_t*)c->pfA, c->maxAd + hp.pleDim);
+            else hipLaunchKernelGGL((k_bd_mix<float, float>), mg, dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
         }
         GEMM(0, c->pfA, c->maxAd + hp.pleDim, L.WoG, L.sWo, L.ad + hp.pleDim, c->h1, d_, c->x, d_, n, d_, L.ad + hp.pleDim);
         if (mlh_gemm_norm_fusable(dt, n, 2 * F)) {
