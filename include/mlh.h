@@ -187,6 +187,16 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
  * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default. */
 int mlh_set_persistent(mlh_ctx* ctx, int mode);
 
+/* Next-token rule of the decode entry points.  temperature 0 (the default): greedy, the argmax fused into the
+ * LM-head reduction, lowest index on ties (the reference's only mode: it keeps the top entry of a qsort of the
+ * probabilities, inference_orchestrator.cu:120-165).  temperature > 0: the token is drawn on the device from
+ * softmax(logits / temperature) -- the smallest index whose cumulative probability exceeds u, with u a 53-bit
+ * uniform from a counter-based generator (SplitMix64) keyed by (seed, sequence id, position of the drawn token), so
+ * a sequence draws the same tokens alone, in a batch or from a graph.  Sampling has no counterpart in the
+ * reference.  While it is on, batch-1 decode runs as the kernel sequence (the single-launch modes fuse the argmax
+ * only).  Returns 0, or -1 for a temperature outside [0, 1e4]. */
+int mlh_set_sampling(mlh_ctx* ctx, float temperature, unsigned long long seed);
+
 /* 1 when mode 3 of mlh_set_persistent applies to this context's model and device, else 0
  * (no counterpart in the reference: its decode loop is one kernel sequence, inference_orchestrator.cu:120-165). */
 int mlh_xcd_decode_supported(mlh_ctx* ctx);

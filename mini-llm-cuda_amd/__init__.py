@@ -88,6 +88,7 @@ _sigs_dev = {
     "mlh_read_logits": (c_int, [c_void_p, c_int, c_void_p]),
     "mlh_read_probs": (c_int, [c_void_p, c_int, c_void_p]),
     "mlh_set_graph": (c_int, [c_void_p, c_int]),
+    "mlh_set_sampling": (c_int, [c_void_p, c_float, ctypes.c_ulonglong]),
     "mlh_set_persistent": (c_int, [c_void_p, c_int]),
     "mlh_xcd_decode_supported": (c_int, [c_void_p]),
     "mlh_synchronize": (c_int, [c_void_p]),
@@ -327,6 +328,10 @@ class Device:
 
     def set_graph(self, enabled):
         self._check(dev.mlh_set_graph(self._h, int(enabled)))
+
+    def set_sampling(self, temperature, seed=0):
+        """temperature 0: greedy (default); > 0: tokens are drawn from softmax(logits / temperature)."""
+        self._check(dev.mlh_set_sampling(self._h, float(temperature), int(seed)))
 
     def set_persistent(self, enabled):
         self._check(dev.mlh_set_persistent(self._h, int(enabled)))

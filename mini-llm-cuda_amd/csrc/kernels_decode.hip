@@ -14,6 +14,7 @@
 // The arithmetic follows inference.cu of the reference op for op (citations at
 // each kernel); the reduction order inside a dot product is this file's own.
 #include "mlh_internal.h"
+#include "sample.h"
 
 #define WG 256
 #define WAVES (WG / MLH_WAVE)
@@ -746,9 +747,24 @@ __global__ void __launch_bounds__(WG) k_lmhead(StepArgs a, int rowsPerWg) {
 __global__ void __launch_bounds__(WG) k_finish(StepArgs a, int* tokOut, int nparts) {
     __shared__ float sv[WG];
     __shared__ int si[WG];
+    __shared__ double sd[WG + 1];
     const int tid = threadIdx.x;
     const int step = *a.stepCounter;
     for (int slot = 0; slot < a.nseq; slot++) {
+        if (a.temperature > 0.f) { // draw instead of argmax: the row of logits is complete (k_lmhead wrote it)
+            const int seq = a.sidx[slot];
+            const int nxt = mlh_sample_row<WG>(a.logits + (size_t)seq * a.vocab, a.vocab, a.temperature,
+                                               mlh_sample_uniform(a.sampleSeed, seq, a.pos[seq] + 1), sd, si);
+            __syncthreads();
+            if (tid == 0) {
+                tokOut[slot] = nxt;
+                a.nextTok[seq] = nxt;
+                if (step < a.outCapacity) a.outIds[(size_t)step * a.nseq + slot] = nxt;
+                a.pos[seq] += 1;
+            }
+            __syncthreads();
+            continue;
+        }
         float v = -3.0e38f;
         int idx = 0x7fffffff;
         for (int i = tid; i < nparts; i += WG) {
@@ -838,6 +854,7 @@ void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr) {
     a.pageTable = c->d_pageTable; a.pagesPerSeq = c->pagesPerSeq; a.nsplit = c->nsplit;
     a.x = c->x; a.qkv = c->qkv; a.qkvStride = c->maxRowsA; a.part = c->part; a.mix = c->mix;
     a.mixRows = c->mixRows; a.mixRowsLd = c->mixRowsLd; a.mixRowsHalf = c->mixRowsHalf; a.wbytes = c->wbytes;
+    a.temperature = c->temperature; a.sampleSeed = c->sampleSeed;
     a.h1 = c->h1; a.u = c->u; a.logits = c->logits; a.amaxVal = c->amaxVal; a.amaxIdx = c->amaxIdx;
     a.amaxParts = c->amaxParts; a.rope = c->rope; a.E = c->E; a.gF = c->gF;
     a.nextTok = c->d_next; a.outIds = c->d_outIds; a.stepCounter = c->d_stepCounter; a.outCapacity = c->outCapacity;

@@ -16,6 +16,7 @@
 #include <algorithm>
 
 #include "mlh_internal.h"
+#include "sample.h"
 
 #define PWG 256
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -1332,9 +1333,23 @@ __global__ void __launch_bounds__(PWG) k_bd_mix(StepArgs a, LayerDev L, AT* Amix
 __global__ void __launch_bounds__(PWG) k_bd_finish(StepArgs a, const float* lg, int* tokOut) {
     __shared__ float sv[PWG];
     __shared__ int si[PWG];
+    __shared__ double sd[PWG + 1];
     const int slot = blockIdx.x, tid = threadIdx.x, seq = a.sidx[slot];
     const float* row = lg + (size_t)slot * a.vocab;
     float* dst = a.logits + (size_t)seq * a.vocab;
+    if (a.temperature > 0.f) { // draw instead of argmax
+        for (int i = tid; i < a.vocab; i += PWG) dst[i] = row[i];
+        const int nxt = mlh_sample_row<PWG>(row, a.vocab, a.temperature, mlh_sample_uniform(a.sampleSeed, seq, a.pos[seq] + 1), sd, si);
+        __syncthreads();
+        if (tid == 0) {
+            const int step = *a.stepCounter - 1;
+            tokOut[slot] = nxt;
+            a.nextTok[seq] = nxt;
+            if (step >= 0 && step < a.outCapacity) a.outIds[(size_t)step * a.nseq + slot] = nxt;
+            a.pos[seq] += 1;
+        }
+        return;
+    }
     float v = -3.0e38f;
     int idx = 0x7fffffff;
     for (int i = tid; i < a.vocab; i += PWG) {

@@ -576,7 +576,8 @@ static int ensure_graph(mlh_ctx* c, int slot, int nseq, int k) {
 }
 
 static bool use_persistent(const mlh_ctx* c, int nseq) {
-    return nseq == 1 && c->usePersistent && mlh_persistent_supported(c);
+    // (the single-launch kernels fuse the argmax only: sampling runs through the kernel sequence)
+    return nseq == 1 && c->usePersistent && c->temperature <= 0.f && mlh_persistent_supported(c);
 }
 
 // After the stream has drained: a persistent launch that gave up a bounded wait leaves its flag set.
@@ -806,6 +807,17 @@ extern "C" int mlh_read_probs(mlh_ctx* c, int seq, float* out) {
     if ((rc = mlh_launch_probs(c, seq))) return rc;
     MLH_CHECK(c, hipStreamSynchronize(c->stream));
     MLH_CHECK(c, hipMemcpy(out, c->probs, (size_t)c->hp.vocabSize * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+extern "C" int mlh_set_sampling(mlh_ctx* c, float temperature, unsigned long long seed) {
+    if (!c) return -1;
+    if (!(temperature >= 0.f) || temperature > 1.0e4f) { c->err = "sampling temperature must be in [0, 1e4]"; return -1; }
+    if (c->temperature != temperature || c->sampleSeed != seed)
+        for (int g = 0; g < 2; g++) // recorded launches carry the old values in their kernel arguments
+            if (c->graphExec[g]) { (void)hipGraphExecDestroy(c->graphExec[g]); c->graphExec[g] = nullptr; }
+    c->temperature = temperature;
+    c->sampleSeed = seed;
     return 0;
 }
 

@@ -69,6 +69,8 @@ struct StepArgs {
     int mixRowsLd;        //   output-projection GEMM (leading dimension in elements, fp32 or IEEE half) instead of `mix`
     int mixRowsHalf;
     int wbytes;           // bytes per weight element (PLE table rows)
+    float temperature;    // > 0: the next token is drawn from softmax(logits / temperature) instead of the argmax
+    unsigned long long sampleSeed;
     float* h1;            // [slots, dim]
     float* u;             // [slots, ffn]
     float* logits;        // [maxSeqs, vocab] indexed by sequence id
@@ -128,6 +130,8 @@ struct mlh_ctx {
     // persistent batch-1 decode kernel
     int numCUs = 0;
     bool coopLaunch = false;
+    float temperature = 0.f;       // 0: greedy; > 0: temperature sampling (kernel-sequence and batched paths)
+    unsigned long long sampleSeed = 0;
     int usePersistent = 3;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange;
                                    // 3: XCD ranks where the model and device allow it, else as 1
     unsigned long long* xcdBuf = nullptr; // (value, tag) exchange words of mode 3

@@ -188,3 +188,40 @@ def forward_full(weights, tokens, dtype="f64", last_only=True, want_probs=False,
     if rc != 0:
         raise RuntimeError(f"oracle forward failed ({rc})")
     return {"logits": logits, "probs": probs, "hidden": hidden}
+
+
+# ---------------------------------------------------------------------------------------------------------
+# Temperature sampling (test infrastructure like the rest of this package).  The reference has no sampling: its
+# loop keeps the top entry of a qsort of the probabilities (inference_orchestrator.cu:120-165).  The rule restated
+# here is the one the device documents: p_i = exp((l_i - max l) / T) / Z, pick = smallest i with
+# sum_{j <= i} p_j Z > u Z, u a 53-bit uniform from SplitMix64 keyed by (seed, sequence id, position drawn).
+# Pinned by: the published first outputs of SplitMix64 seeded with 0, the T -> 0 limit (argmax), the ends of the
+# u range, monotonicity in u, and a frequency test against the softmax (tests/test_oracle_sampling.py).
+# ---------------------------------------------------------------------------------------------------------
+_M64 = (1 << 64) - 1
+
+
+def splitmix64(x):
+    """Output function of SplitMix64 applied to x + golden gamma (Steele, Lea, Flood 2014)."""
+    x = (x + 0x9E3779B97F4A7C15) & _M64
+    z = x
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def sample_uniform(seed, seq, pos):
+    base = splitmix64(splitmix64(seed & _M64) ^ (((seq + 1) * 0xD1342543DE82EF95) & _M64))
+    return (splitmix64((base + pos) & _M64) >> 11) * (1.0 / 9007199254740992.0)
+
+
+def sample_cdf(logits, temperature):
+    """Unnormalised cumulative sums of exp((l - max l) / T) in index order, float64."""
+    l = np.asarray(logits, dtype=np.float64)
+    return np.cumsum(np.exp((l - l.max()) / float(temperature)))
+
+
+def sample_token(logits, temperature, u):
+    c = sample_cdf(logits, temperature)
+    i = int(np.searchsorted(c, u * c[-1], side="right"))  # first index whose cumulative sum exceeds the target
+    return min(i, len(c) - 1)
