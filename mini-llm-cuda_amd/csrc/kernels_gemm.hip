@@ -720,6 +720,117 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny_norm(const float
     }
 }
 
+// The same for at most GSK_WAVES rows and half weights, with the normalised-up-to-1/rms rows staged in LDS: wave w
+// turns row w into halves of g (.) x once (sum of squares from the same pass), the product then reads its token
+// operand from LDS instead of holding fp32 rows and gains in registers -- this keeps the register need of the plain
+// kernel, so two workgroups share a compute unit and a matrix of several hundred row blocks still takes one round.
+// LDS rows are K halves + 16 bytes apart (rows four banks apart: the eight rows a read touches do not collide).
+template <int EPI>
+__global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny_norm8(const float* __restrict__ A, int lda, const f16_t* __restrict__ B, int ldb,
+                                                                void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
+                                                                float alpha, const float* __restrict__ gain) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char a16[]; // [M][2 K + 16] bytes
+    __shared__ float red[GSK_WAVES][1][16][64];
+    __shared__ float rinv[GSK_WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int n0 = blockIdx.x * 32, n32 = lane & 31, half = lane >> 5;
+    const int nchunks = (int)(((size_t)K * 2) / GKB);
+    const int pitch = 2 * K + 16;
+    const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n32, N - 1) * ldb * 2 + half * 64;
+    f32x16 acc = (f32x16)(0.f);
+    u32x4 fb[2][4];
+    auto loadw = [&](int c, int buf) {
+#pragma unroll
+        for (int p = 0; p < 4; p++) fb[buf][p] = *reinterpret_cast<const u32x4*>(brow + (size_t)c * GKB + p * 16);
+    };
+    int c = wave;
+    if (c < nchunks) loadw(c, 0); // the first weights are on their way while the rows are staged
+    if (wave < M) {
+        const float* xr = A + (size_t)wave * lda;
+        float ss = 0.f;
+        for (int k = lane * 8; k < K; k += 64 * 8) {
+            const f32x4 x0 = *reinterpret_cast<const f32x4*>(xr + k), x1 = *reinterpret_cast<const f32x4*>(xr + k + 4);
+            const f32x4 g0 = *reinterpret_cast<const f32x4*>(gain + k), g1 = *reinterpret_cast<const f32x4*>(gain + k + 4);
+            ss = fmaf(x0.x, x0.x, ss); ss = fmaf(x0.y, x0.y, ss); ss = fmaf(x0.z, x0.z, ss); ss = fmaf(x0.w, x0.w, ss);
+            ss = fmaf(x1.x, x1.x, ss); ss = fmaf(x1.y, x1.y, ss); ss = fmaf(x1.z, x1.z, ss); ss = fmaf(x1.w, x1.w, ss);
+            auto h2 = [](float lo, float hi) {
+                const _Float16 a = (_Float16)fminf(fmaxf(lo, -65504.0f), 65504.0f), b = (_Float16)fminf(fmaxf(hi, -65504.0f), 65504.0f);
+                return (uint32_t)__builtin_bit_cast(uint16_t, a) | ((uint32_t)__builtin_bit_cast(uint16_t, b) << 16);
+            };
+            u32x4 w;
+            w.x = h2(g0.x * x0.x, g0.y * x0.y); w.y = h2(g0.z * x0.z, g0.w * x0.w);
+            w.z = h2(g1.x * x1.x, g1.y * x1.y); w.w = h2(g1.z * x1.z, g1.w * x1.w);
+            *reinterpret_cast<u32x4*>(a16 + (size_t)wave * pitch + 2 * k) = w;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        if (lane == 0) rinv[wave] = 1.0f / sqrtf(ss / (float)K + 1e-8f);
+    }
+    __syncthreads();
+    const unsigned char* arow = a16 + (size_t)min(n32, M - 1) * pitch + half * 64;
+    auto mul = [&](int cc, int buf) {
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            const u32x4 fa = *reinterpret_cast<const u32x4*>(arow + (size_t)cc * GKB + p * 16);
+            GemmTraits<f16_t>::mma(fb[buf][p], fa, acc);
+        }
+    };
+    for (; c < nchunks; c += 2 * GSK_WAVES) { // two chunks per trip so the buffers are addressed statically
+        if (c + GSK_WAVES < nchunks) loadw(c + GSK_WAVES, 1);
+        mul(c, 0);
+        if (c + GSK_WAVES < nchunks) {
+            if (c + 2 * GSK_WAVES < nchunks) loadw(c + 2 * GSK_WAVES, 0);
+            mul(c + GSK_WAVES, 1);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) red[wave][0][i][lane] = acc[i];
+    __syncthreads();
+    const float scale = alpha * rinv[min(n32, M - 1)];
+    for (int g = wave; g < 4; g += GSK_WAVES) {
+        const int i4 = g;
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = red_sum(red, 0, 4 * i4 + j, lane) * scale;
+        const int m = n32, n = n0 + 8 * i4 + 4 * half; // accumulator element i: weight row 8 (i / 4) + 4 half + i % 4, column m
+        if (m >= M) continue;
+        if (EPI == GEMM_EPI_SWIGLU) {
+#pragma unroll
+            for (int j = 0; j < 4; j += 2)
+                if (n + j + 1 < N) GemmTraits<f16_t>::put((f16_t*)Cv + (size_t)m * ldc + ((n + j) >> 1), (v[j] / (1.0f + expf(-v[j]))) * v[j + 1]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (n + j < N) {
+                    float o = v[j];
+                    if (R) o += R[(size_t)m * ldr + n + j];
+                    ((float*)Cv)[(size_t)m * ldc + n + j] = o;
+                }
+        }
+    }
+}
+
+// rows that k_gemm_skinny_norm8 can stage: at most one per wave, and 40 KB of LDS beside the reduction buffer (two workgroups per unit)
+static bool skinny_norm8_fits(int M, int K) { return M <= GSK_WAVES && (size_t)M * (2 * (size_t)K + 16) <= 40 * 1024 && K % 512 == 0; }
+
+static hipError_t launch_gemm_skinny_norm8(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                                           const float* R, int ldr, int M, int N, int K, float alpha, const float* normGain) {
+    const dim3 grid((N + 31) / 32);
+    const size_t lds = (size_t)M * (2 * (size_t)K + 16);
+    static bool attr = false; // static + dynamic LDS pass 64 KB
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_skinny_norm8<GEMM_EPI_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_skinny_norm8<GEMM_EPI_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_skinny_norm8<GEMM_EPI_SWIGLU>), grid, dim3(GSK_WAVES * 64), lds, stream, (const float*)A, lda, (const f16_t*)B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);
+    else
+        hipLaunchKernelGGL((k_gemm_skinny_norm8<GEMM_EPI_PLAIN>), grid, dim3(GSK_WAVES * 64), lds, stream, (const float*)A, lda, (const f16_t*)B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);
+    return hipGetLastError();
+}
+
 template <typename T>
 static hipError_t launch_gemm_skinny_norm(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                                           const float* R, int ldr, int M, int N, int K, float alpha, const float* normGain) {
@@ -782,11 +893,11 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
 // ws: optional zero-initialised workspace of mlh_gemm_workspace_bytes() (enables split-K for M <= 64); launches that
 // share a workspace must be ordered on one stream.
 // True when mlh_gemm_tn_epi can take `normGain` for this shape (the RMSNorm of A's rows fused into the product).
-bool mlh_gemm_norm_fusable(int dtype, int M, int N) {
+bool mlh_gemm_norm_fusable(int dtype, int M, int N, int K) {
     // k_gemm_skinny_norm (A is the fp32 residual for both operand types).  With half weights its register need allows
     // one workgroup per compute unit, where the plain kernel runs two: a matrix of more than 256 row blocks would
-    // take two rounds and lose more than the saved RMSNorm launch brings.
-    if (M <= 32) return dtype == MLH_DTYPE_F32 || (dtype == MLH_GEMM_F16 && (N + 31) / 32 <= 256);
+    // take two rounds and lose more than the saved RMSNorm launch brings -- unless the rows fit k_gemm_skinny_norm8's LDS.
+    if (M <= 32) return dtype == MLH_DTYPE_F32 || (dtype == MLH_GEMM_F16 && ((N + 31) / 32 <= 256 || skinny_norm8_fits(M, K)));
     return dtype == MLH_DTYPE_F32 && M > 32 && M <= 64 && N <= 16 * GSK_COUNTERS && (N + 31) / 32 < 200;
 }
 
@@ -796,11 +907,13 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
     if (M <= 0 || N <= 0 || K <= 0 || ((size_t)K * esz) % GKB != 0 || ((size_t)lda * esz) % 16 != 0 || ((size_t)ldb * esz) % 16 != 0)
         return hipErrorInvalidValue;
     if (epi == GEMM_EPI_SWIGLU && (N & 1)) return hipErrorInvalidValue;
-    if (normGain && !mlh_gemm_norm_fusable(dtype, M, N)) return hipErrorInvalidValue;
+    if (normGain && !mlh_gemm_norm_fusable(dtype, M, N, K)) return hipErrorInvalidValue;
     // M <= 64 (one row per sequence of a decode batch): weight-streaming skinny kernel; long M: 256 x 256 tiles
     // fed by direct-to-LDS loads; in between: 128 x 128 tiles
 #define GEMM_BY_TYPE(call_f32, call_bf16, call_f16) \
     return dtype == MLH_DTYPE_BF16 ? (call_bf16) : dtype == MLH_GEMM_F16 ? (call_f16) : (call_f32)
+    if (M <= 32 && normGain && dtype == MLH_GEMM_F16 && skinny_norm8_fits(M, K))
+        return launch_gemm_skinny_norm8(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);
     if (M <= 32 && normGain)
         return dtype == MLH_GEMM_F16 ? launch_gemm_skinny_norm<f16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain)
                                      : launch_gemm_skinny_norm<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha, normGain);

@@ -1414,7 +1414,7 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
     for (int t = hp.transformers - 1; t >= 0; t--) {
         const LayerDev& L = c->layers[t];
         // (fp32, 33..64 sequences: the RMSNorm rides in the product, see mlh_gemm_norm_fusable)
-        if (mlh_gemm_norm_fusable(dt, n, L.rowsA)) {
+        if (mlh_gemm_norm_fusable(dt, n, L.rowsA, d_)) {
             GEMMN(0, c->x, d_, L.WaG, L.sWa, d_, c->qkv, c->maxRowsA, nullptr, 0, n, L.rowsA, d_, L.g1);
         } else {
             if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->x, L.g1, (f16_t*)c->pfXn, n, d_);
@@ -1435,7 +1435,7 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
             else hipLaunchKernelGGL((k_bd_mix<float, float>), mg, dim3(PWG), 0, st, a, L, (float*)c->pfA, c->maxAd + hp.pleDim);
         }
         GEMM(0, c->pfA, c->maxAd + hp.pleDim, L.WoG, L.sWo, L.ad + hp.pleDim, c->h1, d_, c->x, d_, n, d_, L.ad + hp.pleDim);
-        if (mlh_gemm_norm_fusable(dt, n, 2 * F)) {
+        if (mlh_gemm_norm_fusable(dt, n, 2 * F, d_)) {
             GEMMN(1, c->h1, d_, L.W13G, L.sW13, d_, c->pfU, F, nullptr, 0, n, 2 * F, d_, L.g2);
         } else {
             if (bf) hipLaunchKernelGGL((k_pf_rmsnorm<f16_t>), dim3(cdiv(n, 4)), dim3(PWG), 0, st, c->h1, L.g2, (f16_t*)c->pfXn, n, d_);

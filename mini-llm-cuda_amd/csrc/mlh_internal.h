@@ -198,7 +198,7 @@ hipError_t mlh_gemm_tn(hipStream_t stream, int dtype, const void* A, int lda, co
 // eps 1e-8 inside the root), without a pass that writes the normalised rows.
 hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                            const float* R, int ldr, int M, int N, int K, void* ws, float alpha = 1.0f, const float* normGain = nullptr);
-bool mlh_gemm_norm_fusable(int dtype, int M, int N);
+bool mlh_gemm_norm_fusable(int dtype, int M, int N, int K);
 size_t mlh_gemm_workspace_bytes(void);
 
 // kernels_prefill.hip
