@@ -193,7 +193,7 @@ template <typename T, int EPI>
 __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
                                                             void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN, float alpha) {
     extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 2, wn = wave & 3;
     int tm, tn;
     gemm_tile_of(blockIdx.x, tilesM, tilesN, tm, tn);
@@ -202,22 +202,38 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
     const int nslices = (int)(((size_t)K * sizeof(T)) / GKB);
     const size_t ldaB = (size_t)lda * sizeof(T), ldbB = (size_t)ldb * sizeof(T);
 
-    // this wave fills rows [32 wave, 32 wave + 32) of A and of B, eight rows per load instruction
-    const unsigned char* srcA[4];
-    const unsigned char* srcB[4];
+    // This wave fills rows [32 wave, 32 wave + 32) of A and of B, eight rows per load instruction.  A load's address is
+    // a scalar base (the tile's first row, advanced by one slice per trip on the scalar unit) plus a 32-bit lane offset
+    // that never changes, and its LDS target is scalar too: issuing a slice's loads takes no vector-ALU instruction,
+    // so it does not queue behind the MFMAs of the other wave on the SIMD.
+    unsigned goffA[4], goffB[4];
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int r = wave * 32 + q * 8 + (lane >> 3);
         const int pc = (lane & 7) ^ ((r >> 1) & 7);
-        srcA[q] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(m0 + r, M - 1) * ldaB + pc * 16;
-        srcB[q] = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + r, N - 1) * ldbB + pc * 16;
+        goffA[q] = (unsigned)((size_t)(min(m0 + r, M - 1) - m0) * ldaB) + pc * 16; // rows past the end: the last row again
+        goffB[q] = (unsigned)((size_t)(min(n0 + r, N - 1) - n0) * ldbB) + pc * 16;
     }
+    auto uniform_base = [](const void* p) { // wave-uniform pointer into global memory, kept in scalar registers
+        unsigned long long v = (unsigned long long)p;
+        asm("" : "+s"(v));
+        return (const unsigned char*)(__attribute__((address_space(1))) const unsigned char*)v;
+    };
+    const unsigned char* baseA = uniform_base(reinterpret_cast<const unsigned char*>(A) + (size_t)m0 * ldaB);
+    const unsigned char* baseB = uniform_base(reinterpret_cast<const unsigned char*>(B) + (size_t)n0 * ldbB);
+    // (written as the instruction itself: through the builtin the compiler either re-forms 64-bit lane addresses or
+    // copies the offsets, one vector-ALU instruction per load either way)
+    auto dma16 = [](unsigned long long sbase, unsigned laneOff, unsigned ldsAddr) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsAddr), "v"(laneOff), "s"(sbase) : "memory", "m0");
+    };
+    const unsigned ldsBase = (unsigned)(unsigned long long)gsm + (unsigned)(wave * 32 * GKB);
     auto issue = [&](int s, int stage) {
-        unsigned char* dst = gsm + stage * GB_STAGE + wave * 32 * GKB;
+        const unsigned dst = ldsBase + (unsigned)(stage * GB_STAGE);
+        const unsigned long long sa = (unsigned long long)baseA + (unsigned long long)s * GKB, sb = (unsigned long long)baseB + (unsigned long long)s * GKB;
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            __builtin_amdgcn_global_load_lds(srcA[q] + (size_t)s * GKB, dst + q * 8 * GKB, 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(srcB[q] + (size_t)s * GKB, dst + GB_T * GKB + q * 8 * GKB, 16, 0, 0);
+            dma16(sa, goffA[q], dst + q * 8 * GKB);
+            dma16(sb, goffB[q], dst + GB_T * GKB + q * 8 * GKB);
         }
     };
 
