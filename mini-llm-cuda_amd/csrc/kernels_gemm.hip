@@ -509,50 +509,86 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny(const T* __restr
 // With NORM the rows of A are RMS-normalised on the way in (inference.cu:24-50): C = (gain * A / rms(A)) . B^T.  The gain
 // multiplies the elements as they are loaded, the sum of squares of a row is gathered from the same loads, and
 // 1 / rms scales the finished product, so the normalised activations are never written to memory (gridDim.y = 1).
+// The activation rows take the way through LDS: the operand layout wants 16 different rows in 16 neighbouring lanes,
+// and a load of that shape touches 16 cache lines for 64 bytes each -- the L1 then fills at 36 GB/s per compute unit
+// instead of 112 GB/s with eight lanes per 128-byte line (measured with a load-only probe), and at 64 tokens the
+// activation matrix is four fifths of what a workgroup reads.  So a wave fetches its chunk of A global -> LDS with
+// line-shaped loads (8 token rows per instruction, the 16-byte piece order XOR-swizzled by the fetching lane) into a
+// private buffer and reads the operands from there; only the 16 weight rows still load row per lane.
+#define SK16_ABUF (64 * GKB)                          // one chunk of A: 64 token rows x 128 bytes
+#define SK16_LDS (GSK_WAVES * SK16_ABUF)              // bytes of dynamic LDS per workgroup
 template <int EPI, bool NORM>
 __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* __restrict__ A, int lda, const float* __restrict__ B, int ldb,
                                                                    void* Cv, int ldc, const float* R, int ldr, int M, int N, int K,
                                                                    unsigned* counters, float* partials, float alpha,
                                                                    const float* __restrict__ gain) {
-    __shared__ float red[GSK_WAVES][4][4][64];
+    extern __shared__ __attribute__((aligned(16))) unsigned char sk16_lds[];
+    float (*red)[4][4][64] = reinterpret_cast<float (*)[4][4][64]>(sk16_lds); // [GSK_WAVES], over the A buffers once they are done
     __shared__ float ssred[GSK_WAVES][4][16];
     __shared__ int lastFlag;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n0 = blockIdx.x * 16, n16 = lane & 15, kq = lane >> 4;
     const int ks = gridDim.y, kslice = blockIdx.y;
     const int nchunks = (int)(((size_t)K * 4) / GKB);
     const int cbeg = (int)((long)nchunks * kslice / ks), cend = (int)((long)nchunks * (kslice + 1) / ks);
     const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n16, N - 1) * ldb * 4 + kq * 16;
-    const unsigned char* arow[4];
+    // fetch side: instruction j of a chunk brings token rows 8 j + lane / 8, this lane the piece that belongs into
+    // slot lane % 8 of its row; read side: row tb * 16 + n16, pieces kq and kq + 4 (their slots: XOR with the same key)
+    unsigned aoff[8];
 #pragma unroll
-    for (int tb = 0; tb < 4; tb++) arow[tb] = reinterpret_cast<const unsigned char*>(A) + (size_t)min(tb * 16 + n16, M - 1) * lda * 4 + kq * 16;
+    for (int j = 0; j < 8; j++) {
+        const int r = j * 8 + (lane >> 3);
+        aoff[j] = (unsigned)((size_t)min(r, M - 1) * lda * 4) + (unsigned)(((lane & 7) ^ ((r >> 1) & 7)) * 16);
+    }
+    const unsigned char* abase = reinterpret_cast<const unsigned char*>(A);
+    unsigned char* const wbuf = sk16_lds + wave * SK16_ABUF;
+    const int akey = (n16 >> 1) & 7;
+    const int ardoff = n16 * GKB;
     f32x4 acc[4];
 #pragma unroll
     for (int tb = 0; tb < 4; tb++) acc[tb] = (f32x4)(0.f);
-    f32x4 fb[2][2], fa[2][4][2], fg[2][2];
+    f32x4 fb[2][2], fa[4][2], fg[2][2];
     float ss[4] = {0.f, 0.f, 0.f, 0.f}; // NORM: this lane's share of the sums of squares of its four tokens
     const unsigned char* grow = reinterpret_cast<const unsigned char*>(gain) + kq * 16;
-    auto load = [&](int c, int buf) {
+    auto load = [&](int c, int buf) { // buf names the registers of the weight rows and the gain; A has one LDS buffer
 #pragma unroll
         for (int p = 0; p < 2; p++) fb[buf][p] = *reinterpret_cast<const f32x4*>(brow + (size_t)c * GKB + p * 64);
         if (NORM) {
 #pragma unroll
             for (int p = 0; p < 2; p++) fg[buf][p] = *reinterpret_cast<const f32x4*>(grow + (size_t)c * GKB + p * 64);
         }
+        const unsigned char* src = abase + (size_t)c * GKB;
+#pragma unroll
+        for (int j = 0; j < 8; j++) __builtin_amdgcn_global_load_lds(src + aoff[j], wbuf + j * 8 * GKB, 16, 0, 0);
+    };
+    // One chunk per wave is in flight at a time and every wait is for all of the wave's loads; the overlap comes from
+    // the registers: a chunk's operands are read out of LDS, then the next chunk's loads go out into the same buffer,
+    // then this chunk is multiplied.  (Two chunks in flight with a counted wait do not work: with register loads and
+    // direct-to-LDS loads mixed the compiler waits for all of them anyway, and loads written as instructions behind
+    // its back get their target registers copied before the data has landed.)
+    auto mul = [&](int buf, int cnext) { // cnext < 0: nothing more to fetch
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0): this chunk's weight rows, gain and A rows have landed
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned char* rd = wbuf + ardoff;
 #pragma unroll
         for (int tb = 0; tb < 4; tb++)
 #pragma unroll
-            for (int p = 0; p < 2; p++) fa[buf][tb][p] = *reinterpret_cast<const f32x4*>(arow[tb] + (size_t)c * GKB + p * 64);
-    };
-    auto mul = [&](int buf) {
+            for (int p = 0; p < 2; p++) fa[tb][p] = *reinterpret_cast<const f32x4*>(rd + tb * 16 * GKB + (((kq + 4 * p) ^ akey) * 16));
+        // the operands must be in registers before the buffer is fetched into again
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0][0]), "+v"(fa[0][1]), "+v"(fa[1][0]), "+v"(fa[1][1]), "+v"(fa[2][0]), "+v"(fa[2][1]), "+v"(fa[3][0]), "+v"(fa[3][1]) : : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        if (cnext >= 0) load(cnext, buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
         if (NORM) {
 #pragma unroll
             for (int tb = 0; tb < 4; tb++)
 #pragma unroll
                 for (int p = 0; p < 2; p++) {
-                    const f32x4 x = fa[buf][tb][p];
+                    const f32x4 x = fa[tb][p];
                     ss[tb] = fmaf(x.x, x.x, ss[tb]); ss[tb] = fmaf(x.y, x.y, ss[tb]); ss[tb] = fmaf(x.z, x.z, ss[tb]); ss[tb] = fmaf(x.w, x.w, ss[tb]);
-                    fa[buf][tb][p] = x * fg[buf][p];
+                    fa[tb][p] = x * fg[buf][p];
                 }
         }
 #pragma unroll
@@ -560,18 +596,20 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
 #pragma unroll
             for (int e = 0; e < 4; e++)
 #pragma unroll
-                for (int tb = 0; tb < 4; tb++) acc[tb] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[buf][p][e], fa[buf][tb][p][e], acc[tb], 0, 0, 0);
+                for (int tb = 0; tb < 4; tb++) acc[tb] = __builtin_amdgcn_mfma_f32_16x16x4f32(fb[buf][p][e], fa[tb][p][e], acc[tb], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     };
     int c = cbeg + wave;
-    if (c < cend) load(c, 0);
-    for (; c < cend; c += 2 * GSK_WAVES) {
-        if (c + GSK_WAVES < cend) load(c + GSK_WAVES, 1);
-        mul(0);
-        if (c + GSK_WAVES < cend) {
-            if (c + 2 * GSK_WAVES < cend) load(c + 2 * GSK_WAVES, 0);
-            mul(1);
+    if (c < cend) {
+        load(c, 0);
+        for (;;) {
+            if (c + GSK_WAVES < cend) mul(0, c + GSK_WAVES); else { mul(0, -1); break; }
+            c += GSK_WAVES;
+            if (c + GSK_WAVES < cend) mul(1, c + GSK_WAVES); else { mul(1, -1); break; }
+            c += GSK_WAVES;
         }
     }
+    __syncthreads(); // every wave is done with its A buffers: red lies over them
 #pragma unroll
     for (int tb = 0; tb < 4; tb++)
 #pragma unroll
@@ -876,8 +914,18 @@ static hipError_t launch_gemm_skinny16(hipStream_t stream, int epi, const void* 
     const dim3 grid(nblocks, ks);
     unsigned* counters = (unsigned*)ws;
     float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
+    static bool attr = false;
+    if (!attr) {
+        const void* fns[4] = {reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_PLAIN, false>), reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_PLAIN, true>),
+                              reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_SWIGLU, false>), reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_SWIGLU, true>)};
+        for (const void* f : fns) {
+            const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, SK16_LDS);
+            if (e != hipSuccess) return e;
+        }
+        attr = true;
+    }
 #define SK16(EPI_, NORM_)                                                                                                     \
-    hipLaunchKernelGGL((k_gemm_skinny16<EPI_, NORM_>), grid, dim3(GSK_WAVES * 64), 0, stream, (const float*)A, lda, (const float*)B, ldb, \
+    hipLaunchKernelGGL((k_gemm_skinny16<EPI_, NORM_>), grid, dim3(GSK_WAVES * 64), SK16_LDS, stream, (const float*)A, lda, (const float*)B, ldb, \
                        C, ldc, R, ldr, M, N, K, counters, partials, alpha, normGain)
     if (epi == GEMM_EPI_SWIGLU) { if (normGain) SK16(GEMM_EPI_SWIGLU, true); else SK16(GEMM_EPI_SWIGLU, false); }
     else { if (normGain) SK16(GEMM_EPI_PLAIN, true); else SK16(GEMM_EPI_PLAIN, false); }
