@@ -403,7 +403,9 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny(const T* __restr
     const int n0 = blockIdx.x * 32, n32 = lane & 31, half = lane >> 5;
     const int ks = gridDim.y, kslice = blockIdx.y;
     const int nchunks = (int)(((size_t)K * sizeof(T)) / GKB);
-    const int cbeg = (int)((long)nchunks * kslice / ks), cend = (int)((long)nchunks * (kslice + 1) / ks);
+    // (32-bit and skipped without split-K: a 64-bit division is some 130 instructions in front of every wave's first load)
+    const int cbeg = ks == 1 ? 0 : (int)((unsigned)nchunks * (unsigned)kslice / (unsigned)ks);
+    const int cend = ks == 1 ? nchunks : (int)((unsigned)nchunks * (unsigned)(kslice + 1) / (unsigned)ks);
     const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n32, N - 1) * ldb * sizeof(T) + half * 64;
     const unsigned char* arow[MB];
 #pragma unroll
@@ -530,7 +532,9 @@ __global__ void __launch_bounds__(GSK_WAVES * 64) k_gemm_skinny16(const float* _
     const int n0 = blockIdx.x * 16, n16 = lane & 15, kq = lane >> 4;
     const int ks = gridDim.y, kslice = blockIdx.y;
     const int nchunks = (int)(((size_t)K * 4) / GKB);
-    const int cbeg = (int)((long)nchunks * kslice / ks), cend = (int)((long)nchunks * (kslice + 1) / ks);
+    // (32-bit and skipped without split-K: a 64-bit division is some 130 instructions in front of every wave's first load)
+    const int cbeg = ks == 1 ? 0 : (int)((unsigned)nchunks * (unsigned)kslice / (unsigned)ks);
+    const int cend = ks == 1 ? nchunks : (int)((unsigned)nchunks * (unsigned)(kslice + 1) / (unsigned)ks);
     const unsigned char* brow = reinterpret_cast<const unsigned char*>(B) + (size_t)min(n0 + n16, N - 1) * ldb * 4 + kq * 16;
     // fetch side: instruction j of a chunk brings token rows 8 j + lane / 8, this lane the piece that belongs into
     // slot lane % 8 of its row; read side: row tb * 16 + n16, pieces kq and kq + 4 (their slots: XOR with the same key)
