@@ -93,6 +93,26 @@ def test_prefill_logits_vs_oracle_and_tokenwise(pkg, orc, kind, plen):
     dev.close()
 
 
+@pytest.mark.parametrize("cfg,plen", [(2, 64), (2, 41), (3, 48)])
+def test_prefill_rows_33_to_64_long_k(pkg, orc, cfg, plen):
+    """33 to 64 rows take the 16-row fp32 kernel with the RMSNorm fused in and the token rows staged through LDS;
+    at d = 768 / F = 2048 a wave of it walks several K chunks (the small shapes above give it one), and the
+    down projection splits K over workgroups."""
+    hp = pkg.config(cfg, transformers=4 if cfg == 3 else 2, maxL=128)
+    if cfg == 3:
+        pkg.set_layer_pattern(hp, 1)
+    model, dev, w = make(pkg, orc, hp, seed=27)
+    prompt = pkg.random_tokens(27, 0, hp.vocabSize, plen)
+    want = orc.forward_full(w, prompt, "f64", last_only=True)["logits"][-1]
+    dev.prefill(0, prompt)
+    got = dev.logits(0)
+    assert_logits_close(got, want, FP32_RTOL, f"config {cfg} shape, {plen} rows")
+    dev.reset()
+    dev.prefill(0, prompt)
+    assert np.array_equal(dev.logits(0), got), "a repeated prefill from reset must be bit-identical"
+    dev.close()
+
+
 def test_prefill_in_pieces(pkg, orc):
     """A prompt appended in three calls (GEMM, GEMM, short token-by-token tail) gives the logits of one call."""
     hp = small_cfg(pkg, "hybrid_flags")
