@@ -611,9 +611,9 @@ __host__ __device__ __forceinline__ int slot_of(int x) {
 template <int DK> struct GdLayout { // one chunk's operand image (bytes), rows padded by 16 bytes against LDS bank conflicts
     static constexpr int KP = (DK + 8) * 2, TP = (GD_C + 8) * 2; // row pitches of [*, DK] and [*, 64] half matrices
     static constexpr int oKt = 0, oQh = oKt + GD_C * KP, oM = oQh + GD_C * KP, oKhT = oM + GD_C * TP;
-    static constexpr int image = oKhT + DK * TP;                  // 62464 (DK 128), 36864 (DK 64): multiples of 1024
-    static constexpr int oVt = image;                             // half [64, DV], read straight from global
-    static constexpr int total = image + GD_C * DK * 2;
+    static constexpr int oVt = oKhT + DK * TP;                    // half [DV, 64]: a column's 64 tokens contiguous
+    static constexpr int image = oVt + DK * TP;                   // 80896 (DK 128), 46080 (DK 64): multiples of 1024
+    static constexpr int total = image;
 };
 __device__ __forceinline__ uint16_t f16_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 
@@ -760,10 +760,13 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     if (tid < DV) { // holds the q column
         uint16_t* Vt = reinterpret_cast<uint16_t*>(img + Lay::oVt);
 #pragma unroll
-        for (int t = 0; t < GD_C; t++) {
-            Vt[t * DV + col] = f16_bits(X[t]);
-            q16[t * (DK + 8) + sl] = f16_bits(eg[t] * colv[t]);
+        for (int t = 0; t < GD_C; t += 8) { // this column's 64 tokens in a row: the scan reads four at a time
+            u32x4 w;
+            w.x = pack_f16(X[t], X[t + 1]); w.y = pack_f16(X[t + 2], X[t + 3]); w.z = pack_f16(X[t + 4], X[t + 5]); w.w = pack_f16(X[t + 6], X[t + 7]);
+            *reinterpret_cast<u32x4*>(Vt + col * (GD_C + 8) + t) = w;
         }
+#pragma unroll
+        for (int t = 0; t < GD_C; t++) q16[t * (DK + 8) + sl] = f16_bits(eg[t] * colv[t]);
     } else { // holds the k column
 #pragma unroll
         for (int t = 0; t < GD_C; t++) {
@@ -790,6 +793,13 @@ __device__ __forceinline__ void gd_issue_image(const unsigned char* src, unsigne
     for (int q = wave; q < IMG / 1024; q += NW) __builtin_amdgcn_global_load_lds(src + q * 1024 + lane * 16, dst + q * 1024, 16, 0, 0);
 }
 
+// The same, one instruction at a time: load k of this wave (k < ceil(IMG / 1024 / NW)), to be spread over other work.
+template <int IMG, int NW>
+__device__ __forceinline__ void gd_issue_image_one(const unsigned char* src, unsigned char* dst, int wave, int lane, int k) {
+    const int q = wave + k * NW;
+    if (q < IMG / 1024) __builtin_amdgcn_global_load_lds(src + q * 1024 + lane * 16, dst + q * 1024, 16, 0, 0);
+}
+
 template <int DK>
 __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const int* __restrict__ chunkBase, const unsigned char* __restrict__ ws,
                                                       const float* __restrict__ gCexp) {
@@ -810,21 +820,27 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
         for (int i = 0; i < 16; i++) St[j][i] = Sg[(size_t)dv * DK + 32 * j + 8 * (i >> 2) + 4 * half + (i & 3)];
     auto image_of = [&](int c) { return ws + ((size_t)(cb + c) * a.gdnHeads + h) * Lay::total; };
     auto issue = [&](int c, int stage) { gd_issue_image<Lay::image, NW>(image_of(c), sls + stage * Lay::image, wave, lane); };
-    f32x16 Vt[2];
-    auto load_vt = [&](int c) {
-        const _Float16* v = reinterpret_cast<const _Float16*>(image_of(c) + Lay::oVt);
+    constexpr int NIMG = (Lay::image / 1024 + NW - 1) / NW; // loads per wave and image
+    auto issue_one = [&](int c, int stage, int k) { gd_issue_image_one<Lay::image, NW>(image_of(c), sls + stage * Lay::image, wave, lane, k); };
+    // V^T - (what the state predicts) needs tokens 8 g + 4 half + e, e = 0..3, of column dv: eight bytes of the image
+    auto vt_of = [&](const unsigned char* im, int tt, int st, float (&v)[8]) { // elements 8 st .. 8 st + 7 of tile tt
+        const unsigned char* p = im + Lay::oVt + dv * Lay::TP + (32 * tt + 16 * st + 4 * half) * 2;
 #pragma unroll
-        for (int tt = 0; tt < 2; tt++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) Vt[tt][i] = (float)v[(32 * tt + 8 * (i >> 2) + 4 * half + (i & 3)) * DV + dv];
+        for (int g = 0; g < 2; g++) {
+            const u32x2 w = *reinterpret_cast<const u32x2*>(p + 16 * g);
+            v[4 * g + 0] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w.x & 0xffff));
+            v[4 * g + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w.x >> 16));
+            v[4 * g + 2] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w.y & 0xffff));
+            v[4 * g + 3] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w.y >> 16));
+        }
     };
     issue(0, 0);
-    load_vt(0);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+    asm volatile("" ::: "memory");
     __syncthreads();
     for (int c = 0; c < nch; c++) {
         const unsigned char* im = sls + (c & 1) * Lay::image;
-        if (c + 1 < nch) issue(c + 1, (c + 1) & 1);
+        const bool more = c + 1 < nch;
         const float gC = gCexp[(size_t)(cb + c) * a.gdnHeads + h];
         // S0^T as B operands: step (j, st) = elements 8 st .. 8 st + 7 of tile j, rounded to half
         u32x4 sop[JT][2];
@@ -835,7 +851,9 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
                 sop[j][st].x = pack_f16(St[j][8 * st + 0], St[j][8 * st + 1]); sop[j][st].y = pack_f16(St[j][8 * st + 2], St[j][8 * st + 3]);
                 sop[j][st].z = pack_f16(St[j][8 * st + 4], St[j][8 * st + 5]); sop[j][st].w = pack_f16(St[j][8 * st + 6], St[j][8 * st + 7]);
             }
-        // X = Kt S0^T, Y = diag(e^g) Q S0^T : [64 tokens, 32 dv]
+        // X = Kt S0^T : [64 tokens, 32 dv] (lane = dv), Y^T = S0 (diag(e^g) Q)^T : [32 dv, 64 tokens] (lane = token: the
+        // operands swapped), so that an output row leaves as four neighbouring columns per store.  The next image's
+        // loads go out between the MFMAs, one per pair: issued in one go they hold the wave for a microsecond.
         f32x16 X[2], Y[2];
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
@@ -850,9 +868,13 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
                     const u32x4 ka = *reinterpret_cast<const u32x4*>(kr + 32 * (2 * j + st));
                     const u32x4 qa = *reinterpret_cast<const u32x4*>(qr + 32 * (2 * j + st));
                     X[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ka), __builtin_bit_cast(f16x8, sop[j][st]), X[tt], 0, 0, 0);
-                    Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, qa), __builtin_bit_cast(f16x8, sop[j][st]), Y[tt], 0, 0, 0);
+                    Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, sop[j][st]), __builtin_bit_cast(f16x8, qa), Y[tt], 0, 0, 0);
+                    if (more && (tt * JT + j) * 2 + st < NIMG) issue_one(c + 1, (c + 1) & 1, (tt * JT + j) * 2 + st);
                 }
         }
+#pragma unroll
+        for (int k = 2 * JT * 2; k < NIMG; k++) // (more loads than MFMA pairs: the rest goes out here)
+            if (more) issue_one(c + 1, (c + 1) & 1, k);
         // W^T = Vt - X, as B operands (token axis in slot order by construction)
         u32x4 wop[2][2];
 #pragma unroll
@@ -860,12 +882,12 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
 #pragma unroll
             for (int st = 0; st < 2; st++) {
                 float w[8];
+                vt_of(im, tt, st, w);
 #pragma unroll
-                for (int e = 0; e < 8; e++) w[e] = Vt[tt][8 * st + e] - X[tt][8 * st + e];
+                for (int e = 0; e < 8; e++) w[e] -= X[tt][8 * st + e];
                 wop[tt][st].x = pack_f16(w[0], w[1]); wop[tt][st].y = pack_f16(w[2], w[3]);
                 wop[tt][st].z = pack_f16(w[4], w[5]); wop[tt][st].w = pack_f16(w[6], w[7]);
             }
-        if (c + 1 < nch) load_vt(c + 1); // Vt of this chunk has been consumed
         // O = Y + M W^T (M is lower triangular: tokens of tile 0 see only tile 0)
 #pragma unroll
         for (int tt = 0; tt < 2; tt++) {
@@ -875,13 +897,19 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
 #pragma unroll
                 for (int st = 0; st < 2; st++) {
                     const u32x4 ma = *reinterpret_cast<const u32x4*>(mr + 32 * (2 * t2 + st));
-                    Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ma), __builtin_bit_cast(f16x8, wop[t2][st]), Y[tt], 0, 0, 0);
+                    Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, wop[t2][st]), __builtin_bit_cast(f16x8, ma), Y[tt], 0, 0, 0);
                 }
-            const int nvalid = len - (c * GD_C + 32 * tt);
+            // lane = token n32 of this tile; element i = column 32 wave + 8 (i / 4) + 4 half + i % 4
+            if (n32 < len - (c * GD_C + 32 * tt)) {
+                f16_t* orow = (f16_t*)P.Amix + (size_t)(row0 + c * GD_C + 32 * tt + n32) * P.aLd + h * DV + 32 * wave + 4 * half;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int tk = 8 * (i >> 2) + 4 * half + (i & 3);
-                if (tk < nvalid) put<f16_t>((f16_t*)P.Amix + (size_t)(row0 + c * GD_C + 32 * tt + tk) * P.aLd + h * DV + dv, Y[tt][i]);
+                for (int g = 0; g < 4; g++) {
+                    float o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = fminf(fmaxf(Y[tt][4 * g + e], -65504.0f), 65504.0f); // saturating: an overflow must not become inf
+                    u32x2 w; w.x = pack_f16(o[0], o[1]); w.y = pack_f16(o[2], o[3]);
+                    *reinterpret_cast<u32x2*>(orow + 8 * g) = w;
+                }
             }
         }
         // S^T <- e^{g_C} S^T + Kh^T W^T
@@ -898,7 +926,8 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
                     St[j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, ha), __builtin_bit_cast(f16x8, wop[t2][st]), St[j], 0, 0, 0);
                 }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the next chunk's image (and Vt) has landed
+        __builtin_amdgcn_s_waitcnt(0x0F70);              // vmcnt(0): the next chunk's image has landed -- as a builtin, so that
+        asm volatile("" ::: "memory");                   // the compiler knows and does not wait again among the next loads
         __syncthreads();                                  // ... for every wave; everyone is done with this image
     }
 #pragma unroll
