@@ -757,13 +757,14 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
     // needed: the MFMAs are done) and leave as 16-byte rows; element-wise 2-byte stores to global would touch a
     // different cache line per lane.
     uint16_t* khs = q16 + GD_C * (DK + 8); // [DK][64 + 8]
+    __syncthreads();                       // every column is solved: the triangular matrix has been read for the last time
+    uint16_t* vts = reinterpret_cast<uint16_t*>(Am); // V^T [DV][64] takes its place (the same 64 * DV * 2 bytes)
     if (tid < DV) { // holds the q column
-        uint16_t* Vt = reinterpret_cast<uint16_t*>(img + Lay::oVt);
 #pragma unroll
         for (int t = 0; t < GD_C; t += 8) { // this column's 64 tokens in a row: the scan reads four at a time
             u32x4 w;
             w.x = pack_f16(X[t], X[t + 1]); w.y = pack_f16(X[t + 2], X[t + 3]); w.z = pack_f16(X[t + 4], X[t + 5]); w.w = pack_f16(X[t + 6], X[t + 7]);
-            *reinterpret_cast<u32x4*>(Vt + col * (GD_C + 8) + t) = w;
+            *reinterpret_cast<u32x4*>(vts + col * GD_C + t) = w;
         }
 #pragma unroll
         for (int t = 0; t < GD_C; t++) q16[t * (DK + 8) + sl] = f16_bits(eg[t] * colv[t]);
@@ -782,6 +783,8 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
         const u32x4* s2 = reinterpret_cast<const u32x4*>(khs);
         u32x4* d2 = reinterpret_cast<u32x4*>(img + Lay::oKhT);
         for (int i = tid; i < DK * Lay::TP / 16; i += NT) d2[i] = s2[i];
+        const u32x4* s3 = reinterpret_cast<const u32x4*>(vts); // rows of eight 16-byte pieces to rows of pitch TP
+        for (int i = tid; i < DV * 8; i += NT) *reinterpret_cast<u32x4*>(img + Lay::oVt + (i >> 3) * Lay::TP + (i & 7) * 16) = s3[i];
     }
     if (tid == 0) gCexp[(size_t)chunk * a.gdnHeads + h] = expf(gC);
 }
