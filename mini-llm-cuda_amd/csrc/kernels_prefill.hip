@@ -902,16 +902,36 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_scan(PfArgs P, LayerDev L, const
                     const u32x4 ma = *reinterpret_cast<const u32x4*>(mr + 32 * (2 * t2 + st));
                     Y[tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, wop[t2][st]), __builtin_bit_cast(f16x8, ma), Y[tt], 0, 0, 0);
                 }
-            // lane = token n32 of this tile; element i = column 32 wave + 8 (i / 4) + 4 half + i % 4
-            if (n32 < len - (c * GD_C + 32 * tt)) {
-                f16_t* orow = (f16_t*)P.Amix + (size_t)(row0 + c * GD_C + 32 * tt + n32) * P.aLd + h * DV + 32 * wave + 4 * half;
+            // lane = token n32 of this tile; element i = column 32 wave + 8 (i / 4) + 4 half + i % 4.  The two lanes of a
+            // token (half 0 and 1) swap two of their four 8-byte pieces so that each holds two whole 16-byte pieces:
+            // half as many store instructions, and the address unit works through a store per lane and instruction.
+            {
+                u32x2 w[4];
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     float o[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) o[e] = fminf(fmaxf(Y[tt][4 * g + e], -65504.0f), 65504.0f); // saturating: an overflow must not become inf
-                    u32x2 w; w.x = pack_f16(o[0], o[1]); w.y = pack_f16(o[2], o[3]);
-                    *reinterpret_cast<u32x2*>(orow + 8 * g) = w;
+                    w[g].x = pack_f16(o[0], o[1]); w[g].y = pack_f16(o[2], o[3]);
+                }
+                // half 0 keeps pieces g = 0, 2 (and gets the partner's upper halves of them), half 1 keeps g = 1, 3
+                u32x2 give[2], got[2];
+                give[0] = half ? w[0] : w[1]; give[1] = half ? w[2] : w[3];
+#pragma unroll
+                for (int k = 0; k < 2; k++) {
+                    got[k].x = (uint32_t)__shfl_xor((int)give[k].x, 32, 64);
+                    got[k].y = (uint32_t)__shfl_xor((int)give[k].y, 32, 64);
+                }
+                if (n32 < len - (c * GD_C + 32 * tt)) {
+                    f16_t* orow = (f16_t*)P.Amix + (size_t)(row0 + c * GD_C + 32 * tt + n32) * P.aLd + h * DV + 32 * wave + 8 * half;
+#pragma unroll
+                    for (int k = 0; k < 2; k++) { // columns 16 k + 8 half .. + 7: lower four from the half-0 lane, upper four from the half-1 lane
+                        const u32x2 mine = w[2 * k + half];
+                        u32x4 v;
+                        v.x = half ? got[k].x : mine.x; v.y = half ? got[k].y : mine.y;
+                        v.z = half ? mine.x : got[k].x; v.w = half ? mine.y : got[k].y;
+                        *reinterpret_cast<u32x4*>(orow + 16 * k) = v;
+                    }
                 }
             }
         }
