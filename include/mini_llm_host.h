@@ -106,6 +106,30 @@ unsigned int mll_hash_token(const char* str);
 int mll_load_story_context(const char* storiesPath, int storyIndex, int percentage, const mll_vocab* v,
                            int maxL, int32_t* out);
 
+/* loadStoriesFromFile (training_orchestrator.cu:103-273): ALL stories of a tokenised-stories file.
+ * Story i that loads occupies tokens[i*(maxL+1) .. (i+1)*(maxL+1)): its first min(count, maxL+1) ids, then
+ * MLL_PADDING_TOKEN_INDEX; rightEnd[i] = ids loaded - 2 (the last position with a known next token, so the
+ * forward runs over L = rightEnd[i]+1 positions).  At most maxStories stories of the file are looked at
+ * (the reference's MAX_TRAINING_STORIES); stories that are not arrays, are empty, have fewer than two
+ * tokens, or hold a non-string or out-of-vocabulary token are skipped with a warning.  Returns the number
+ * of stories loaded, 0 for an empty file, -1 on error (missing file, not JSON, not an array). */
+#define MLL_PADDING_TOKEN_INDEX 89   /* training_orchestrator.h:11 */
+#define MLL_MAX_TRAINING_STORIES 2000 /* training_orchestrator.h:6 */
+int mll_load_stories(const char* filePath, const mll_vocab* v, int maxL, int maxStories, int32_t* tokens,
+                     int32_t* rightEnd);
+
+/* Feeds `count` loaded stories (slab and rightEnd as mll_load_stories fills them, first story `first`) to
+ * the device in ONE batched prefill: story first+i is appended to sequence i (which the call empties first)
+ * over its L = rightEnd+1 positions.  The context needs maxSeqs >= count.  Returns 0, or -1 on error. */
+int mll_prefill_stories(mlh_ctx* ctx, const int32_t* tokens, const int32_t* rightEnd, int maxL, int first,
+                        int count);
+
+/* The forward half of processSequence (training_orchestrator.cu:289-359) for one loaded story: a
+ * teacher-forced forward over L = rightEnd+1 positions on sequence 0, then for every position whose next
+ * token is not the padding token: loss += -logf(max(p(next), 1e-4)).  story points at the story's maxL+1
+ * ids.  Returns 0 and fills totalLoss / numPredictions (either may be null); non-zero on error. */
+int mll_story_loss(mlh_ctx* ctx, const int32_t* story, int rightEnd, float* totalLoss, int* numPredictions);
+
 /* ---- token loop --------------------------------------------------------- */
 
 typedef struct {

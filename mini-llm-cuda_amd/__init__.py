@@ -120,6 +120,9 @@ _sigs_host = {
     "mll_vocab_lookup": (c_int, [c_void_p, c_char_p]),
     "mll_hash_token": (ctypes.c_uint, [c_char_p]),
     "mll_load_story_context": (c_int, [c_char_p, c_int, c_int, c_void_p, c_int, c_void_p]),
+    "mll_load_stories": (c_int, [c_char_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    "mll_prefill_stories": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int]),
+    "mll_story_loss": (c_int, [c_void_p, c_void_p, c_int, _P(c_float), _P(c_int)]),
     "mll_generate": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, _P(c_double)]),
     "mll_top_k": (c_int, [c_void_p, c_int, c_int, _P(TokenProb)]),
 }
@@ -366,6 +369,20 @@ class Device:
             raise MlhError(f"generate failed: {dev.mlh_last_error(self._h).decode()}")
         return out[:n].copy(), ms.value
 
+    def prefill_stories(self, tokens, right_end, first, count):
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        r = np.ascontiguousarray(right_end, dtype=np.int32)
+        if host.mll_prefill_stories(self._h, t.ctypes.data, r.ctypes.data, t.shape[1] - 1, first, count) != 0:
+            raise MlhError(f"prefill_stories failed: {dev.mlh_last_error(self._h).decode()}")
+
+    def story_loss(self, story, right_end):
+        """(total loss, predictions) of one loaded story: the forward half of the reference's processSequence."""
+        t = np.ascontiguousarray(story, dtype=np.int32)
+        loss, n = c_float(), c_int()
+        if host.mll_story_loss(self._h, t.ctypes.data, int(right_end), byref(loss), byref(n)) != 0:
+            raise MlhError(f"story_loss failed: {dev.mlh_last_error(self._h).decode()}")
+        return float(loss.value), int(n.value)
+
     def top_k(self, k, seq=0):
         buf = (TokenProb * k)()
         n = host.mll_top_k(self._h, seq, k, buf)
@@ -404,6 +421,15 @@ class Vocab:
         out = np.zeros(max_l + 1, dtype=np.int32)
         n = host.mll_load_story_context(os.fsencode(path), story_index, percentage, self._h, max_l, out.ctypes.data)
         return out[:n].copy()
+
+    def load_stories(self, path, max_l, max_stories=2000):
+        """All stories of a tokenised-stories file: (tokens [n, max_l+1], rightEnd [n]), or None on error."""
+        toks = np.zeros((max(max_stories, 1), max_l + 1), dtype=np.int32)
+        right = np.zeros(max(max_stories, 1), dtype=np.int32)
+        n = host.mll_load_stories(os.fsencode(path), self._h, max_l, max_stories, toks.ctypes.data, right.ctypes.data)
+        if n < 0:
+            return None
+        return toks[:n].copy(), right[:n].copy()
 
     def close(self):
         if self._h:

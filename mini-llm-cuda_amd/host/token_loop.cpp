@@ -1,6 +1,7 @@
 // Greedy token loop over the device layer, and the reference-named C++ surface
 // (mini_llm_reference_api.h) that makes the library a drop-in for the
 // reference's inference path.
+#include <math.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -54,6 +55,44 @@ extern "C" int mll_top_k(mlh_ctx* ctx, int seq, int k, mll_token_prob* out) {
     });
     for (int i = 0; i < k; i++) { out[i].tokenIdx = idx[i]; out[i].prob = probs[idx[i]]; }
     return k;
+}
+
+extern "C" int mll_prefill_stories(mlh_ctx* ctx, const int32_t* tokens, const int32_t* rightEnd, int maxL_,
+                                   int first, int count) {
+    if (!ctx || !tokens || !rightEnd || first < 0 || count <= 0 || maxL_ != mlh_max_len(ctx)) return -1;
+    std::vector<int32_t> seqs(count), lens(count), ids;
+    for (int i = 0; i < count; i++) {
+        const int L = rightEnd[first + i] + 1;
+        if (L < 1 || L > maxL_) return -1;
+        seqs[i] = i;
+        lens[i] = L;
+        const int32_t* story = tokens + (size_t)(first + i) * (maxL_ + 1);
+        ids.insert(ids.end(), story, story + L);
+        if (mlh_reset(ctx, i)) return -1;
+    }
+    return mlh_prefill_batch(ctx, count, seqs.data(), ids.data(), lens.data()) ? -1 : 0;
+}
+
+extern "C" int mll_story_loss(mlh_ctx* ctx, const int32_t* story, int rightEnd, float* totalLoss, int* numPredictions) {
+    if (!ctx || !story || rightEnd < 0 || rightEnd + 1 > mlh_max_len(ctx)) return 1;
+    const int L = rightEnd + 1, V = mlh_vocab_size(ctx);
+    std::vector<float> probs((size_t)L * V);
+    if (mlh_reset(ctx, 0)) return 1;
+    if (mlh_forward_full(ctx, 0, story, L, nullptr, probs.data(), nullptr)) return 1;
+    float loss = 0.0f;
+    int n = 0;
+    for (int pos = 0; pos <= rightEnd; pos++) { // training_orchestrator.cu:330-352
+        const int next = story[pos + 1];
+        if (next == MLL_PADDING_TOKEN_INDEX) continue;
+        if (next < 0 || next >= V) return 1;
+        float p = probs[(size_t)pos * V + next];
+        if (p < 0.0001f) p = 0.0001f;
+        loss += -logf(p);
+        n++;
+    }
+    if (totalLoss) *totalLoss = loss;
+    if (numPredictions) *numPredictions = n;
+    return 0;
 }
 
 // ---------------------------------------------------------------------------

@@ -151,3 +151,62 @@ extern "C" int mll_load_story_context(const char* storiesPath, int storyIndex, i
     printf("--- Story context loaded successfully. ---\n\n");
     return contextLength;
 }
+
+// loadStoriesFromFile (training_orchestrator.cu:103-273): every story of a file into one slab of
+// maxL+1 ids per story, padded with the padding token; rightEnd[i] = (tokens loaded) - 2, the last
+// position whose next token is known.  Stories that are not arrays, are empty, hold fewer than two
+// tokens, a non-string or a token outside the vocabulary are skipped with the reference's warnings.
+extern "C" int mll_load_stories(const char* filePath, const mll_vocab* v, int maxL_, int maxStories, int32_t* tokens,
+                                int32_t* rightEnd) {
+    const int perStory = maxL_ + 1; // TOKENS_PER_STORY, training_orchestrator.h:9
+    printf("--- Loading stories from %s ---\n", filePath ? filePath : "(null)");
+    std::string text;
+    if (!filePath || !read_file(filePath, text)) {
+        printf("Error: Stories file not found at '%s'\n", filePath ? filePath : "(null)");
+        return -1;
+    }
+    if (!tokens || !rightEnd || maxStories < 0 || maxL_ < 1) return -1;
+    Json root;
+    std::string err;
+    if (!mll::parseJson(text.data(), text.size(), root, err)) { printf("Error: Failed to parse stories JSON.\n"); return -1; }
+    if (!root.isArray()) { printf("Error: Stories JSON is not an array.\n"); return -1; }
+    int numStories = (int)root.arr.size();
+    if (numStories == 0) { printf("Warning: Stories file is empty.\n"); return 0; }
+    if (numStories > maxStories) {
+        printf("Warning: File contains %d stories, truncating to %d.\n", numStories, maxStories);
+        numStories = maxStories;
+    }
+    printf("Processing %d stories...\n", numStories);
+    int loaded = 0;
+    for (int s = 0; s < numStories; s++) {
+        const Json& story = root.arr[s];
+        if (!story.isArray()) { printf("Warning: Story at index %d is not an array, skipping.\n", s); continue; }
+        const int count = (int)story.arr.size();
+        if (count == 0) { printf("Warning: Story at index %d has no tokens, skipping.\n", s); continue; }
+        const int toLoad = count > perStory ? perStory : count;
+        if (toLoad - 2 < 0) { printf("Warning: Story at index %d has fewer than 2 tokens, skipping.\n", s); continue; }
+        int32_t* slot = tokens + (size_t)loaded * perStory;
+        bool bad = false;
+        for (int pos = 0; pos < toLoad; pos++) {
+            const Json& item = story.arr[pos];
+            if (!item.isString()) {
+                printf("Warning: Token at position %d in story %d is not a string.\n", pos, s);
+                bad = true;
+                break;
+            }
+            const int idx = mll_vocab_lookup(v, item.str.c_str());
+            if (idx < 0) {
+                printf("Warning: Token '%s' not found in vocabulary (story %d, pos %d).\n", item.str.c_str(), s, pos);
+                bad = true;
+                break;
+            }
+            slot[pos] = idx;
+        }
+        if (bad) continue; // the slot is reused by the next story
+        for (int pos = toLoad; pos < perStory; pos++) slot[pos] = MLL_PADDING_TOKEN_INDEX;
+        rightEnd[loaded] = toLoad - 2;
+        loaded++;
+    }
+    printf("Successfully processed %d stories (out of %d in file).\n", loaded, numStories);
+    return loaded;
+}

@@ -50,6 +50,7 @@ def _lib():
         g("orc_head_rmsnorm").argtypes = [c_void_p, c_void_p, c_int, c_int]
         g("orc_rope").argtypes = [c_void_p, c_void_p, c_int, c_int, c_int]
         g("orc_matvec").argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p]
+        g("orc_matmat").argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_int]
         g("orc_attend").argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
         g("orc_gdn_step").argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, real, real, c_int, c_int, c_void_p]
         g("orc_state_new").restype = c_void_p

@@ -26,7 +26,12 @@
  * Parity status: the reference ships no numeric golden outputs, and its GEMMs
  * go through cuBLAS in TF32 mode (main.cu:179), so agreement with the CUDA
  * binary's numbers is "parity unpinned".  Every function here is pinned
- * against closed forms / brute force / an independent NumPy restatement.
+ * against closed forms / brute force / an independent NumPy restatement
+ * (tests/test_oracle_pins.py): the per-layer-embedding branch by
+ * x + Wpu (silu(Wpg xn) * P[tok]) on a one-block model plus a table-row swap,
+ * the gated-delta-net gates and update by their matrix form on two tokens,
+ * the blocked product of the full-sequence forward by bit-equality with the
+ * one-vector product.
  *
  * Every function exists twice: suffix _f32 computes in float (the reference's
  * type), suffix _f64 in double (the arbiter for tolerance decisions).
@@ -102,6 +107,8 @@ void orc_round_bf16(float* w, long n);
     void orc_head_rmsnorm_##SFX(REAL* q, const float* gamma, int heads, int hd);       \
     void orc_rope_##SFX(REAL* q, const float* tab, int pos, int heads, int hd);        \
     void orc_matvec_##SFX(const float* W, const REAL* x, int rows, int cols, REAL* y); \
+    void orc_matmat_##SFX(const float* W, const REAL* X, int ldx, int rows, int cols, int L, \
+                          REAL* Y, int ldy);                                           \
     void orc_attend_##SFX(const REAL* q, const REAL* K, const REAL* V, int T, int dim, \
                           int heads, int hd, REAL* out);                               \
     void orc_gdn_step_##SFX(REAL* S, const REAL* q, const REAL* k, const REAL* v,      \

@@ -27,6 +27,55 @@ void FN(orc_matvec)(const float* W, const REAL* x, int rows, int cols, REAL* y) 
     }
 }
 
+/* Y[l] = W X[l] for L vectors at once (X: [L, ldx], Y: [L, ldy], one vector per row).  Every output
+ * element is accumulated exactly as orc_matvec does it (one accumulator, columns in ascending order, a
+ * multiply and an add per term), so the result is bit-identical to L calls of orc_matvec; only the loop
+ * nest differs: ORC_TB vectors are transposed into a block so that a weight row is read once per block
+ * and the independent accumulators of the block's vectors fill the SIMD lanes. */
+#define ORC_TB 16
+__attribute__((target_clones("avx512f", "avx2", "default"), optimize("O3")))
+static void FN(orc_mm_tile)(const float* w0, const float* w1, const float* w2, const float* w3, int cols,
+                            const REAL* xT, REAL* out) {
+    REAL a0[ORC_TB], a1[ORC_TB], a2[ORC_TB], a3[ORC_TB];
+    for (int l = 0; l < ORC_TB; l++) a0[l] = a1[l] = a2[l] = a3[l] = 0;
+    for (int c = 0; c < cols; c++) {
+        const REAL* xc = xT + (size_t)c * ORC_TB;
+        REAL v0 = (REAL)w0[c], v1 = (REAL)w1[c], v2 = (REAL)w2[c], v3 = (REAL)w3[c];
+        for (int l = 0; l < ORC_TB; l++) {
+            a0[l] += v0 * xc[l];
+            a1[l] += v1 * xc[l];
+            a2[l] += v2 * xc[l];
+            a3[l] += v3 * xc[l];
+        }
+    }
+    for (int l = 0; l < ORC_TB; l++) {
+        out[l] = a0[l];
+        out[ORC_TB + l] = a1[l];
+        out[2 * ORC_TB + l] = a2[l];
+        out[3 * ORC_TB + l] = a3[l];
+    }
+}
+
+void FN(orc_matmat)(const float* W, const REAL* X, int ldx, int rows, int cols, int L, REAL* Y, int ldy) {
+    REAL* xT = (REAL*)malloc(sizeof(REAL) * (size_t)cols * ORC_TB);
+    for (int l0 = 0; l0 < L; l0 += ORC_TB) {
+        int nl = L - l0 < ORC_TB ? L - l0 : ORC_TB;
+        for (int c = 0; c < cols; c++)
+            for (int l = 0; l < ORC_TB; l++)
+                xT[(size_t)c * ORC_TB + l] = l < nl ? X[(size_t)(l0 + l) * ldx + c] : (REAL)0;
+#pragma omp parallel for schedule(static)
+        for (int r0 = 0; r0 < rows; r0 += 4) {
+            REAL out[4 * ORC_TB];
+            const float* w[4];
+            for (int i = 0; i < 4; i++) w[i] = W + (size_t)(r0 + i < rows ? r0 + i : rows - 1) * cols;
+            FN(orc_mm_tile)(w[0], w[1], w[2], w[3], cols, xT, out);
+            for (int i = 0; i < 4 && r0 + i < rows; i++)
+                for (int l = 0; l < nl; l++) Y[(size_t)(l0 + l) * ldy + r0 + i] = out[i * ORC_TB + l];
+        }
+    }
+    free(xT);
+}
+
 /* inference.cu:24-50 + 83-95: r = sqrt(mean(x^2) + eps); y = gamma * (x / r).
  * Division first, then the gain, as the reference's two kernels do. */
 void FN(orc_rmsnorm)(const REAL* x, const float* gamma, int n, REAL* y) {
@@ -201,14 +250,12 @@ void FN(orc_state_free)(void* p) {
  *   q,k,v = Wq xn, Wk xn, Wv xn ; q_h,k_h L2-normalised per head ;
  *   alpha_h = exp(-softplus(wa_h.xn + ba_h)) ; beta_h = sigmoid(wb_h.xn + bb_h) ;
  *   state update and read-out as orc_gdn_step.  No RoPE, no QK RMSNorm, no query gating. */
-static void FN(orc_gdn_mix)(const orc_hparams* hp, const orc_layer* lw, const REAL* xn, REAL* S,
-                            REAL* q, REAL* k, REAL* v, REAL* a) {
+static void FN(orc_gdn_recur)(const orc_hparams* hp, const orc_layer* lw, const REAL* xn, REAL* S,
+                              REAL* q, REAL* k, const REAL* v, REAL* a) {
     int Hg = hp->gdnHeads, dk = hp->gdnDk, dv = hp->gdnDv, d = hp->dim;
-    FN(orc_matvec)(lw->Wq, xn, Hg * dk, d, q);
-    FN(orc_matvec)(lw->Wk, xn, Hg * dk, d, k);
-    FN(orc_matvec)(lw->Wv, xn, Hg * dv, d, v);
     FN(orc_l2norm_heads)(q, Hg, dk);
     FN(orc_l2norm_heads)(k, Hg, dk);
+#pragma omp parallel for schedule(static) if ((long)Hg * dk * dv > 65536)
     for (int h = 0; h < Hg; h++) {
         REAL za, zb;
         FN(orc_matvec)(lw->gdnWa + (size_t)h * d, xn, 1, d, &za);
@@ -218,6 +265,15 @@ static void FN(orc_gdn_mix)(const orc_hparams* hp, const orc_layer* lw, const RE
         FN(orc_gdn_step)(S + (size_t)h * dv * dk, q + h * dk, k + h * dk, v + h * dv, alpha, beta, dk,
                          dv, a + h * dv);
     }
+}
+
+static void FN(orc_gdn_mix)(const orc_hparams* hp, const orc_layer* lw, const REAL* xn, REAL* S,
+                            REAL* q, REAL* k, REAL* v, REAL* a) {
+    int Hg = hp->gdnHeads, dk = hp->gdnDk, dv = hp->gdnDv, d = hp->dim;
+    FN(orc_matvec)(lw->Wq, xn, Hg * dk, d, q);
+    FN(orc_matvec)(lw->Wk, xn, Hg * dk, d, k);
+    FN(orc_matvec)(lw->Wv, xn, Hg * dv, d, v);
+    FN(orc_gdn_recur)(hp, lw, xn, S, q, k, v, a);
 }
 
 /* Per-layer-embedding branch for one position (no reference counterpart):
@@ -327,26 +383,30 @@ int FN(orc_forward_full)(const orc_hparams* hp, const orc_weights* w, const int*
             int Hg = hp->gdnHeads, dk = hp->gdnDk, dv = hp->gdnDv;
             ad = Hg * dv;
             memset(St, 0, sizeof(REAL) * (size_t)Hg * dk * dv);
+            FN(orc_matmat)(lw->Wq, xn, d, Hg * dk, d, L, Q, qd);
+            FN(orc_matmat)(lw->Wk, xn, d, Hg * dk, d, L, K, qd);
+            FN(orc_matmat)(lw->Wv, xn, d, Hg * dv, d, L, Vv, qd);
             for (int l = 0; l < L; l++) /* recurrence from the zero state, position by position */
-                FN(orc_gdn_mix)(hp, lw, xn + (size_t)l * d, St, Q + (size_t)l * qd, K + (size_t)l * qd,
-                                Vv + (size_t)l * qd, A + (size_t)l * ad);
+                FN(orc_gdn_recur)(hp, lw, xn + (size_t)l * d, St, Q + (size_t)l * qd, K + (size_t)l * qd,
+                                  Vv + (size_t)l * qd, A + (size_t)l * ad);
         } else {
             ad = d;
+            FN(orc_matmat)(lw->Wq, xn, d, d, d, L, Q, d);
+            FN(orc_matmat)(lw->Wk, xn, d, d, d, L, K, d);
+            FN(orc_matmat)(lw->Wv, xn, d, d, d, L, Vv, d);
+            if (hp->queryGating) FN(orc_matmat)(lw->Wg, xn, d, d, d, L, G, d);
             for (int l = 0; l < L; l++) {
-                FN(orc_matvec)(lw->Wq, xn + (size_t)l * d, d, d, Q + (size_t)l * d);
-                FN(orc_matvec)(lw->Wk, xn + (size_t)l * d, d, d, K + (size_t)l * d);
-                FN(orc_matvec)(lw->Wv, xn + (size_t)l * d, d, d, Vv + (size_t)l * d);
                 if (hp->qkRmsNorm) {
                     FN(orc_head_rmsnorm)(Q + (size_t)l * d, lw->qRms, H, hd);
                     FN(orc_head_rmsnorm)(K + (size_t)l * d, lw->kRms, H, hd);
                 }
                 FN(orc_rope)(Q + (size_t)l * d, rope, l, H, hd);
                 FN(orc_rope)(K + (size_t)l * d, rope, l, H, hd);
-                if (hp->queryGating) FN(orc_matvec)(lw->Wg, xn + (size_t)l * d, d, d, G + (size_t)l * d);
             }
             /* KtQ per head, S[h][qcol][krow] at h*L*L + qcol*L + krow (inference.cu:511-535),
              * then scale+mask (136-155), column max (157-186), exp+sum (188-218), normalise (220-239). */
             REAL scale = R_SQRT((REAL)hd);
+#pragma omp parallel for collapse(2) schedule(dynamic, 8) if (L >= 64)
             for (int h = 0; h < H; h++) {
                 for (int qc = 0; qc < L; qc++) {
                     REAL* col = Sc + ((size_t)h * L + qc) * L;
@@ -376,30 +436,39 @@ int FN(orc_forward_full)(const orc_hparams* hp, const orc_weights* w, const int*
             if (hp->queryGating)
                 for (size_t i = 0; i < (size_t)d * L; i++) A[i] = A[i] * FN(orc_sigmoid)(G[i]);
         }
+        FN(orc_matmat)(lw->Wo, A, ad, d, ad, L, h1, d);
         for (int l = 0; l < L; l++) {
-            FN(orc_matvec)(lw->Wo, A + (size_t)l * ad, d, ad, h1 + (size_t)l * d);
             for (int r = 0; r < d; r++) h1[(size_t)l * d + r] += x[(size_t)l * d + r];
             if (hp->pleDim > 0) {
                 FN(orc_ple_branch)(hp, lw, xn + (size_t)l * d, tokens[l], ple, tmp);
                 for (int r = 0; r < d; r++) h1[(size_t)l * d + r] += tmp[r];
             }
             FN(orc_rmsnorm)(h1 + (size_t)l * d, lw->rms2, d, hn + (size_t)l * d);
-            FN(orc_matvec)(lw->W1A, hn + (size_t)l * d, F, d, g1 + (size_t)l * F);
-            FN(orc_matvec)(lw->W1B, hn + (size_t)l * d, F, d, g2 + (size_t)l * F);
-            for (int i = 0; i < F; i++)
-                u[(size_t)l * F + i] = FN(orc_silu)(g1[(size_t)l * F + i]) * g2[(size_t)l * F + i];
-            FN(orc_matvec)(lw->W2, u + (size_t)l * F, d, F, tmp);
-            for (int r = 0; r < d; r++) x[(size_t)l * d + r] = tmp[r] + h1[(size_t)l * d + r];
         }
+        FN(orc_matmat)(lw->W1A, hn, d, F, d, L, g1, F);
+        FN(orc_matmat)(lw->W1B, hn, d, F, d, L, g2, F);
+        for (size_t i = 0; i < (size_t)F * L; i++) u[i] = FN(orc_silu)(g1[i]) * g2[i];
+        FN(orc_matmat)(lw->W2, u, F, d, F, L, x, d); /* x is free from here on: h1 holds the residual */
+        for (size_t i = 0; i < (size_t)d * L; i++) x[i] = x[i] + h1[i];
     }
 
     if (finalHidden) memcpy(finalHidden, x, sizeof(REAL) * (size_t)d * L);
     if (logits || probs) {
         REAL* lg = (REAL*)malloc(sizeof(REAL) * (size_t)V);
+        REAL* all = NULL;
+        if (!lastOnly) { /* every position: one blocked product over the final-normed columns */
+            all = (REAL*)malloc(sizeof(REAL) * (size_t)V * L);
+            for (int l = 0; l < L; l++) FN(orc_rmsnorm)(x + (size_t)l * d, w->gammaF, d, xn + (size_t)l * d);
+            FN(orc_matmat)(w->E, xn, d, V, d, L, all, V);
+        }
         for (int l = lastOnly ? L - 1 : 0; l < L; l++) {
             size_t o = lastOnly ? 0 : (size_t)l * V;
-            FN(orc_rmsnorm)(x + (size_t)l * d, w->gammaF, d, tmp);
-            FN(orc_matvec)(w->E, tmp, V, d, lg);
+            if (all) {
+                memcpy(lg, all + (size_t)l * V, sizeof(REAL) * (size_t)V);
+            } else {
+                FN(orc_rmsnorm)(x + (size_t)l * d, w->gammaF, d, tmp);
+                FN(orc_matvec)(w->E, tmp, V, d, lg);
+            }
             if (logits) memcpy(logits + o, lg, sizeof(REAL) * (size_t)V);
             if (probs) { /* inference.cu:293-362 */
                 REAL m = (REAL)-1.0e20f, sum = 0;
@@ -413,6 +482,7 @@ int FN(orc_forward_full)(const orc_hparams* hp, const orc_weights* w, const int*
             }
         }
         free(lg);
+        free(all);
     }
     free(rope); free(x); free(xn); free(Q); free(K); free(Vv); free(G); free(A); free(h1); free(hn);
     free(g1); free(g2); free(u); free(tmp); free(ple); free(Sc); free(St);

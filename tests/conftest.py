@@ -77,7 +77,10 @@ def check_greedy_against_oracle(decoder, prompt, gpu_ids, gap_tol, gpu_logits_pe
     exact = tolerated = 0
     for i, gid in enumerate(gpu_ids):
         best = int(np.argmax(lg))
-        if gpu_logits_per_step is not None:
+        if isinstance(gpu_logits_per_step, dict):  # logits recorded at some steps only
+            if i in gpu_logits_per_step:
+                assert_logits_close(gpu_logits_per_step[i], lg, rtol, f"{what} step {i}")
+        elif gpu_logits_per_step is not None:
             assert_logits_close(gpu_logits_per_step[i], lg, rtol, f"{what} step {i}")
         if int(gid) == best:
             exact += 1

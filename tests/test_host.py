@@ -307,6 +307,52 @@ def test_story_context_rules(pkg, tmp_path):
     assert len(v.story_context(str(notarr), 0, 100, 1280)) == 0
 
 
+def test_load_all_stories_of_a_file(pkg, tmp_path, capfd):
+    """The multi-story loader (reference: loadStoriesFromFile, training_orchestrator.cu:103-273): slab of
+    maxL+1 ids per loaded story padded with token 89, rightEnd = ids loaded - 2, bad stories skipped with
+    the slot reused, file truncated to the story limit."""
+    v = pkg.Vocab(VOCAB_PV)
+    sample = json.load(open(SAMPLE))
+    want = [v.lookup(t) for t in sample]
+    stories = tmp_path / "stories.json"
+    docs = [sample, "not an array", [], ["Once"], sample[:2], ["Once", 5], ["Once", " upon", "zzzz-not-in-vocab"],
+            sample[:41], sample[:40], sample[:100]]
+    stories.write_text(json.dumps(docs))
+    maxL = 40
+    flush = lambda: ctypes.CDLL(None).fflush(None)  # the library prints through C stdio
+    toks, right = v.load_stories(str(stories), maxL)
+    flush()
+    out = capfd.readouterr().out
+    assert toks.shape == (5, maxL + 1)
+    assert right.tolist() == [39, 0, 39, 38, 39]        # 166 -> 41 loaded; 2; 41; 40; 100 -> 41
+    assert toks[0].tolist() == want[:41] and toks[2].tolist() == want[:41] and toks[4].tolist() == want[:41]
+    assert toks[1].tolist() == want[:2] + [89] * 39      # padded with the padding token
+    assert toks[3].tolist() == want[:40] + [89]
+    for msg in ("Processing 10 stories...", "Story at index 1 is not an array, skipping.",
+                "Story at index 2 has no tokens, skipping.", "Story at index 3 has fewer than 2 tokens, skipping.",
+                "Token at position 1 in story 5 is not a string.",
+                "Token 'zzzz-not-in-vocab' not found in vocabulary (story 6, pos 2).",
+                "Successfully processed 5 stories (out of 10 in file)."):
+        assert msg in out, msg
+    # the story limit truncates the FILE (stories looked at), as the reference's MAX_TRAINING_STORIES does
+    toks2, right2 = v.load_stories(str(stories), maxL, max_stories=5)
+    flush()
+    assert right2.tolist() == [39, 0] and "File contains 10 stories, truncating to 5." in capfd.readouterr().out
+    # a long maxL loads whole stories; rightEnd follows the story length
+    toks3, right3 = v.load_stories(str(stories), 1280)
+    assert right3.tolist() == [164, 0, 39, 38, 98] and toks3[0, :166].tolist() == want and np.all(toks3[0, 166:] == 89)
+    # errors: missing file, not JSON, not an array -> -1; empty array -> 0 stories
+    assert v.load_stories(str(tmp_path / "none.json"), maxL) is None
+    bad = tmp_path / "bad.json"
+    bad.write_text("[[")
+    assert v.load_stories(str(bad), maxL) is None
+    bad.write_text('{"a": []}')
+    assert v.load_stories(str(bad), maxL) is None
+    bad.write_text("[]")
+    t0, r0 = v.load_stories(str(bad), maxL)
+    assert t0.shape[0] == 0 and r0.shape[0] == 0
+
+
 # --------------------------------------------------------------------------- generator and presets
 M64 = (1 << 64) - 1
 

@@ -135,6 +135,24 @@ def test_matvec_row_major(orc):
     assert np.allclose(yf, y, rtol=1e-4, atol=1e-5)
 
 
+def test_blocked_product_is_bit_identical_to_matvec(orc):
+    """The full-sequence forward multiplies all columns at once (blocked over tokens); each element must be
+    accumulated exactly as the one-vector routine does it, in float and in double, for ragged shapes."""
+    rng = np.random.default_rng(33)
+    for rows, cols, L in ((37, 96, 1), (6, 50, 16), (130, 64, 45)):
+        W = rng.normal(size=(rows, cols)).astype(np.float32)
+        for sfx, real in (("f32", np.float32), ("f64", np.float64)):
+            X = np.ascontiguousarray(rng.normal(size=(L, cols + 3)).astype(real))  # rows padded: ldx > cols
+            Y = np.full((L, rows + 2), 7.0, dtype=real)
+            getattr(orc.lib, f"orc_matmat_{sfx}")(_p(W), _p(X), cols + 3, rows, cols, L, _p(Y), rows + 2)
+            for l in range(L):
+                y = np.empty(rows, dtype=real)
+                x = np.ascontiguousarray(X[l, :cols])
+                getattr(orc.lib, f"orc_matvec_{sfx}")(_p(W), _p(x), rows, cols, _p(y))
+                assert np.array_equal(Y[l, :rows], y)
+            assert np.all(Y[:, rows:] == 7.0)
+
+
 def test_attend_brute_force_and_special_cases(orc):
     H, hd, T = 3, 64, 29
     d = H * hd
@@ -358,6 +376,65 @@ def test_gdn_gates_closed_form(pkg, orc):
         x_out = S @ q + x
     hid = orc.forward_full(w, np.array(toks, np.int32), "f64", want_hidden=True)["hidden"]
     assert np.allclose(hid[-1], x_out, rtol=1e-9, atol=1e-12)
+
+
+def test_ple_branch_closed_form(pkg, orc):
+    """Per-layer embeddings: h1 = Wo a + x + Wpu (silu(Wpg xn) * P[tok]), xn the RMS1-normed input.  One
+    attention block with Wo = 0 and the FFN switched off leaves hidden = x + the PLE branch, which is
+    compared with an independent NumPy statement; a wrong activation, x in place of xn, a wrong table
+    row or a missing gain each fail it."""
+    hp = pkg.config(3, dim=64, attnHeads=1, headDim=64, ffnDim=64, transformers=1, vocabSize=32, gdnHeads=1,
+                    pleDim=16, maxL=4)
+    pkg.set_layer_pattern(hp, 1)
+    hp.layerKinds[0] = 0
+    model = pkg.Model.generate(hp, 5)
+    rng = np.random.default_rng(5)
+    model.tensor(0, 6)[:] = 0                                    # Wo = 0: attention adds nothing
+    model.tensor(0, 8)[:] = 0                                    # gate rows 0: silu(0) * up = 0, FFN adds nothing
+    model.tensor(0, 2)[:] = 1 + 0.3 * rng.normal(size=hp.dim)    # RMS1 gain: xn, not x / rms
+    model.tensor(0, 18)[:] = rng.normal(size=(32, 16))           # table rows of visible size
+    model.tensor(0, 19)[:] = rng.normal(size=(16, 64))           # gate pre-activations O(1): silu != sigmoid != id
+    model.tensor(0, 20)[:] = rng.normal(size=(64, 16))
+    E = model.tensor(0, 0).astype(np.float64)
+    g1 = model.tensor(0, 2).astype(np.float64)
+    P, Wpg, Wpu = (model.tensor(0, t).astype(np.float64) for t in (18, 19, 20))
+
+    def want(tok):
+        x = E[tok]
+        xn = g1 * (x / np.sqrt(np.mean(x * x) + 1e-8))
+        z = Wpg @ xn
+        return x + Wpu @ ((z / (1 + np.exp(-z))) * P[tok])
+
+    toks = np.array([3, 7], np.int32)
+    hid = orc.forward_full(orc.Weights.from_model(model), toks, "f64", want_hidden=True)["hidden"]
+    for i, t in enumerate(toks):
+        assert np.allclose(hid[i], want(t), rtol=1e-9, atol=1e-12)
+    # the branch is not small here: leaving it out, or using the wrong row, would be far outside the bound
+    assert np.max(np.abs(hid[0] - E[3])) > 1e-2 and np.max(np.abs(want(3) - (want(7) - E[7] + E[3]))) > 1e-2
+    # row selection: swapping two table rows swaps what the two tokens receive from the table
+    model.tensor(0, 18)[[3, 7]] = model.tensor(0, 18)[[7, 3]]
+    P[[3, 7]] = P[[7, 3]]
+    hid2 = orc.forward_full(orc.Weights.from_model(model), toks, "f64", want_hidden=True)["hidden"]
+    for i, t in enumerate(toks):
+        assert np.allclose(hid2[i], want(t), rtol=1e-9, atol=1e-12)
+    assert np.max(np.abs(hid2 - hid)) > 1e-2
+    # the cached decode path uses the same branch: its logits equal the full recompute's
+    w = orc.Weights.from_model(model)
+    dec = orc.Decoder(w, "f64")
+    for t in toks:
+        _, lg = dec.step(int(t))
+    full = orc.forward_full(w, toks, "f64")["logits"][0]
+    assert np.allclose(lg, full, rtol=1e-12, atol=1e-14)
+    # and the branch joins the residual with the output projection (before RMS2 / the FFN): with the FFN on,
+    # the FFN must see x + branch
+    model.tensor(0, 8)[:] = rng.normal(size=(64, 64)) * 0.2
+    W1A, W1B, W2 = (model.tensor(0, t).astype(np.float64) for t in (8, 9, 10))
+    g2 = model.tensor(0, 7).astype(np.float64)
+    hid3 = orc.forward_full(orc.Weights.from_model(model), toks, "f64", want_hidden=True)["hidden"]
+    h1 = want(3)
+    hn = g2 * (h1 / np.sqrt(np.mean(h1 * h1) + 1e-8))
+    a = W1A @ hn
+    assert np.allclose(hid3[0], h1 + W2 @ ((a / (1 + np.exp(-a))) * (W1B @ hn)), rtol=1e-9, atol=1e-12)
 
 
 def test_greedy_pick_takes_lowest_index_on_ties(pkg, orc):
