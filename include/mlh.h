@@ -76,7 +76,7 @@ enum {
 
 typedef struct mlh_ctx mlh_ctx;
 
-/* Last error text of a context (ctx == NULL: of the last failed mlh_create on this thread). */
+/* Last error text of a context (ctx == NULL: of the last failed mlh_create or context-free call on this thread). */
 const char* mlh_last_error(const mlh_ctx* ctx);
 
 /* Number of visible HIP devices (0 when there is none; never fails). */
@@ -242,6 +242,22 @@ int mlh_time_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps,
  * cublasGemmEx calls of inference.cu:401-743 so that it can be checked and measured alone. */
 int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A, const float* B, const float* R, float* C,
                       int iters, double* avg_us);
+
+/* The same product, C[M,N] = A[M,K] . B[N,K]^T (+ R[M,N]), for callers that cannot allocate -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose GEMMs are
+ * cuBLAS calls on buffers from allocateMemory).  dA, dB, dR (may be null) and dC are DEVICE pointers on the current
+ * device: A and B in the operand type (MLH_DTYPE_F32 float, MLH_DTYPE_BF16 bf16, 2 = IEEE half), R and C fp32, all
+ * dense row-major; the launch is enqueued on `stream` (a hipStream_t; null = the default stream) and the call returns
+ * without synchronising.  The call allocates and frees nothing: the split-K workspace (tile counters and partial
+ * tiles) that mlh_selftest_gemm allocates per call lives here in a static device array of 4 KiB + 2 MiB, which every GPU
+ * the library runs on holds until the process ends.  Limits: M <= 64, N <= 32768, K <= 65536, K * element size a
+ * multiple of 128 bytes; anything else returns -1 with a message in mlh_last_error(NULL).  All calls on one GPU share
+ * that array: calls that may overlap on one GPU (different streams or threads) race and must be ordered by the caller.
+ * mlh_gemm_device_init(device) looks up the array's address on that device ahead of time (mlh_create does it too);
+ * otherwise the first call on a device does. */
+int mlh_gemm_device_init(int device);
+int mlh_gemm_device(int dtype, int M, int N, int K, const void* dA, const void* dB, const float* dR, float* dC,
+                    void* stream);
 
 #ifdef __cplusplus
 }

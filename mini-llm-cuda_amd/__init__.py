@@ -96,6 +96,8 @@ _sigs_dev = {
     "mlh_kernel_name": (c_char_p, [c_int]),
     "mlh_time_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double)]),
     "mlh_selftest_gemm": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, _P(c_double)]),
+    "mlh_gemm_device_init": (c_int, [c_int]),
+    "mlh_gemm_device": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "mlh_profile_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double), _P(c_int32)]),
 }
 _sigs_host = {

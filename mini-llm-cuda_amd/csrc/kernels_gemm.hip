@@ -15,6 +15,8 @@
 #include <string.h>
 
 #include <algorithm>
+#include <mutex>
+#include <string>
 
 #include "mlh_internal.h"
 
@@ -1082,4 +1084,80 @@ done:
     if (e1) (void)hipEventDestroy(e1);
     (void)hipFree(dA); (void)hipFree(dB); (void)hipFree(dC); (void)hipFree(dR); (void)hipFree(dW);
     return rc;
+}
+
+// ----------------------------------------------------------------------------
+// The same product for callers that cannot allocate (code under graph capture, serving loops that forbid
+// hipMalloc): device pointers in and out, the launch enqueued on the caller's stream, and the split-K workspace
+// (tile counters + partial tiles) in a file-scope device array instead of a hipMalloc'ed buffer.  Every GPU holds
+// its own copy of the array at its own address; the address is looked up once per device and kept.  All calls on
+// one GPU share the array: calls that overlap on one GPU (two streams, two threads) race on it.
+// ----------------------------------------------------------------------------
+#define NOALLOC_MAX_M 64           // rows of A (one per sequence of a decode batch): the skinny kernels' range
+#define NOALLOC_MAX_N 32768        // rows of B
+#define NOALLOC_MAX_K 65536        // contraction length
+#define NOALLOC_MAX_TILES 256      // partial tiles of a split-K launch (launch_gemm_skinny*: nblocks * ks <= 256)
+#define NOALLOC_TILE_BYTES (2 * 16 * 64 * 4) // largest partial tile: 64 activation rows x 32 weight rows, fp32
+#define NOALLOC_SCRATCH_BYTES (GSK_COUNTERS * 4 + NOALLOC_MAX_TILES * NOALLOC_TILE_BYTES) // 4 KiB + 2 MiB
+#define NOALLOC_MAX_DEVICES 64
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+static void* g_scratchPtr[NOALLOC_MAX_DEVICES]; // per device: the device address of that GPU's copy of `scratch`
+static std::mutex g_scratchMutex;
+
+__global__ void k_fill_u32(unsigned* p, unsigned v, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
+// Looks up the address of this device's copy of the scratch array (once per device, that device current).
+static int noalloc_setup(int device, void** out) {
+    if (device < 0 || device >= NOALLOC_MAX_DEVICES) { mlh_set_thread_error("device index out of range"); return -1; }
+    std::lock_guard<std::mutex> lock(g_scratchMutex);
+    if (!g_scratchPtr[device]) {
+        int cur = -1;
+        hipError_t e = hipGetDevice(&cur);
+        if (e == hipSuccess && cur != device) e = hipSetDevice(device);
+        void* p = nullptr;
+        if (e == hipSuccess) e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (cur >= 0 && cur != device) (void)hipSetDevice(cur);
+        if (e != hipSuccess || !p) {
+            mlh_set_thread_error(std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+            return -2;
+        }
+        g_scratchPtr[device] = p;
+    }
+    *out = g_scratchPtr[device];
+    return 0;
+}
+
+extern "C" int mlh_gemm_device_init(int device) {
+    void* p;
+    return noalloc_setup(device, &p);
+}
+
+extern "C" int mlh_gemm_device(int dtype, int M, int N, int K, const void* dA, const void* dB, const float* dR, float* dC,
+                               void* stream) {
+    if (!dA || !dB || !dC) { mlh_set_thread_error("null operand pointer"); return -1; }
+    if (dtype != MLH_DTYPE_F32 && dtype != MLH_DTYPE_BF16 && dtype != MLH_GEMM_F16) { mlh_set_thread_error("unknown operand type"); return -1; }
+    if (M <= 0 || N <= 0 || K <= 0) { mlh_set_thread_error("M, N and K must be positive"); return -1; }
+    if (M > NOALLOC_MAX_M || N > NOALLOC_MAX_N || K > NOALLOC_MAX_K) {
+        mlh_set_thread_error("shape beyond the static workspace: this entry point takes M <= 64, N <= 32768, K <= 65536 "
+                         "(got M " + std::to_string(M) + ", N " + std::to_string(N) + ", K " + std::to_string(K) + ")");
+        return -1;
+    }
+    const size_t esz = dtype == MLH_DTYPE_F32 ? 4 : 2;
+    if (((size_t)K * esz) % GKB != 0) { mlh_set_thread_error("K * element size must be a multiple of 128 bytes"); return -1; }
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess) { mlh_set_thread_error("hipGetDevice failed"); return -2; }
+    void* ws = nullptr;
+    int rc = noalloc_setup(device, &ws);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    // The counters must start at zero.  A finished launch leaves them at zero, a launch that was cut short may not;
+    // a fill kernel rather than hipMemsetAsync, so that the call can be recorded into a graph.
+    hipLaunchKernelGGL(k_fill_u32, dim3((GSK_COUNTERS + 255) / 256), dim3(256), 0, st, (unsigned*)ws, 0u, GSK_COUNTERS);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess) e = mlh_gemm_tn_epi(st, dtype, GEMM_EPI_PLAIN, dA, K, dB, K, dC, N, dR, N, M, N, K, ws, 1.0f);
+    if (e != hipSuccess) { mlh_set_thread_error(std::string("launch failed: ") + hipGetErrorString(e)); return -2; }
+    return 0;
 }

@@ -10,6 +10,8 @@
 
 static thread_local std::string g_create_error;
 
+void mlh_set_thread_error(const std::string& msg) { g_create_error = msg; }
+
 extern "C" const char* mlh_last_error(const mlh_ctx* ctx) {
     return ctx ? ctx->err.c_str() : g_create_error.c_str();
 }
@@ -95,6 +97,7 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
     if (ndev <= 0) return fail_create("no HIP device is visible: the MI355X path cannot run without a GPU");
     if (device < 0 || device >= ndev) return fail_create("device index out of range");
     if (hipSetDevice(device) != hipSuccess) return fail_create("hipSetDevice failed");
+    if (mlh_gemm_device_init(device)) return -2; // address of this device's static workspace (mlh_gemm_device); message already set
 
     mlh_ctx* c = new mlh_ctx();
     c->hp = *hpIn;

@@ -200,6 +200,10 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
                            const float* R, int ldr, int M, int N, int K, void* ws, float alpha = 1.0f, const float* normGain = nullptr);
 bool mlh_gemm_norm_fusable(int dtype, int M, int N, int K);
 size_t mlh_gemm_workspace_bytes(void);
+extern "C" int mlh_gemm_device_init(int device);
+
+// mlh_api.hip: message returned by mlh_last_error(NULL) on this thread (context-free entry points)
+void mlh_set_thread_error(const std::string& msg);
 
 // kernels_prefill.hip
 bool mlh_prefill_gemm_supported(const mlh_ctx* c);
