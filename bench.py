@@ -11,13 +11,15 @@ HBM), the roofline of the dominant kernel measured live with HIP events on the c
 whole-step bytes-per-token roofline, and the CPU baseline (PyTorch restatement of the reference's
 pytorch_verification model on this host's cores) timed on a bounded sample of the same workload.
 
-Four decode paths exist and all are timed; `value` is the one named in config.decode_path:
+Three decode paths exist and all are timed; `value` is the one named in config.decode_path:
   xcd         one launch covers all K steps; every XCD is a tensor-parallel rank (its heads, its FFN units),
               exchanges inside an XCD go through its L2, two per layer cross XCDs (default)
   persistent  one launch of the persistent kernel covers all K steps, phases separated by a grid barrier
               built from agent-scope atomics
-  tagged      the same kernel without barriers: consumers spin on (value, tag) words
   kernels     a sequence of per-phase kernels per step (plain launches or hipGraph replays)
+
+Protocol: every figure is the median of REPS (5) timed repetitions of the same work, each with the device idle on
+both sides; minimum and maximum are reported beside it.
 """
 import argparse
 import json
@@ -34,6 +36,32 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
 MFMA_BF16_PEAK = 2.5e15  # MI355X dense bf16 MFMA, published peak (flop/s)
 PROMPT_LEN = 64
+REPS = 5  # timed repetitions per figure; the median is reported
+
+
+def stats(xs):
+    xs = sorted(float(x) for x in xs)
+    return {"median": xs[len(xs) // 2], "min": xs[0], "max": xs[-1], "reps": len(xs)}
+
+
+def physical_cores():
+    """Physical cores of this host: distinct (physical id, core id) pairs of /proc/cpuinfo (logical CPUs if absent)."""
+    try:
+        pairs, phys, core = set(), None, None
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("physical id"):
+                phys = line.split(":")[1].strip()
+            elif line.startswith("core id"):
+                core = line.split(":")[1].strip()
+            elif not line.strip():
+                if phys is not None and core is not None:
+                    pairs.add((phys, core))
+                phys = core = None
+        if phys is not None and core is not None:
+            pairs.add((phys, core))
+        return len(pairs) or (os.cpu_count() or 1)
+    except OSError:
+        return os.cpu_count() or 1
 
 
 def decode_bytes_per_token(hp, T, wbytes=4):
@@ -61,7 +89,9 @@ def cpu_baseline(model, hp, prompt, seconds_budget=20.0):
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import cpu_model
 
-    threads = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(os.cpu_count() or 1, 16)
+    # one thread per physical core, within the share of the host this job has (OMP_NUM_THREADS is set to it on the box)
+    share = int(os.environ.get("OMP_NUM_THREADS", "0")) or (os.cpu_count() or 1)
+    threads = max(1, min(physical_cores(), share))
     tensors = {("E",): model.tensor(0, 0), ("gammaF",): model.tensor(0, 1)}
     for l in range(hp.transformers):
         for tid in range(2, 11):
@@ -89,6 +119,7 @@ def cpu_baseline(model, hp, prompt, seconds_budget=20.0):
                    f"positions per token as the reference's runInferenceLoop does; PyTorch {torch.__version__} CPU fp32"),
         "with_kv_cache_tok_s": 128 / t_cached,
         "host_cpu_count": os.cpu_count(),
+        "host_physical_cores": physical_cores(),
         "first_ids": ids_full[:8],
         "first_ids_cached": ids_cached[:8],
     }
@@ -108,7 +139,7 @@ def matrix_params(hp):
     return total
 
 
-def batched_decode_leg(m, steps=64):
+def batched_decode_leg(m, steps=48):
     """Configuration 4: 64 concurrent sequences of the hybrid architecture, prompt lengths uniform in
     [32, 512] (seeded), greedy decode.  Returns tok/s and the fraction of the bytes-per-step roofline
     (weights once per step + every sequence's K/V rows and GDN states)."""
@@ -122,25 +153,29 @@ def batched_decode_leg(m, steps=64):
     dev.prefill_batch(list(range(nseq)), prompts)
     firsts = [dev.greedy_token(s) for s in range(nseq)]
     out = dev.decode_loop(firsts, 8)  # warm-up
-    dev.synchronize()
-    t0 = time.perf_counter()
-    out = dev.decode_loop([int(t) for t in out[-1]], steps)
-    dev.synchronize()
-    wall = time.perf_counter() - t0
+    walls = []
+    for _ in range(REPS):
+        dev.synchronize()
+        t0 = time.perf_counter()
+        out = dev.decode_loop([int(t) for t in out[-1]], steps)
+        dev.synchronize()
+        walls.append(time.perf_counter() - t0)
+    wall = stats(walls)["median"]
     wb = 2 if hp.weightDtype == m.DTYPE_BF16 else 4
     weights = decode_bytes_per_token(hp, 0, wb) - sum(
         (2 * hp.dim * 4 if hp.layerKinds[t] == 0 else 2 * hp.gdnHeads * hp.gdnDk * hp.gdnDv * 4) for t in range(hp.transformers))
-    per_seq = [decode_bytes_per_token(hp, int(n) + 8 + steps // 2, wb) - weights for n in lens]
+    per_seq = [decode_bytes_per_token(hp, int(n) + 8 + (REPS * steps) // 2, wb) - weights for n in lens]
     step_bytes = weights + float(np.sum(per_seq))
     dev.close()
     return {"workload": "config 4: 64 sequences, prompts uniform in [32, 512], hybrid 3 GDN : 1 attention + PLE, fp32",
             "steps": steps, "ms_per_step": wall / steps * 1e3, "tok_s": nseq * steps / wall,
+            "ms_per_step_stats": stats([w / steps * 1e3 for w in walls]),
             "bytes_per_step": step_bytes, "achieved_GBps": step_bytes / (wall / steps) / 1e9,
             "frac_of_hbm_peak": step_bytes / (wall / steps) / 1e9 / HBM_PEAK_GBPS,
             "last_ids": [int(x) for x in out[-1, :4]]}
 
 
-def hybrid_decode_leg(m, steps=256):
+def hybrid_decode_leg(m, steps=192):
     """Configuration 3: batch-1 greedy decode of the hybrid architecture (3 GDN : 1 attention + PLE) after a
     128-token prompt.  Returns tok/s and the fraction of the bytes-per-token roofline (weights, GDN states read and
     written, K/V rows of the attention layers)."""
@@ -152,95 +187,110 @@ def hybrid_decode_leg(m, steps=256):
     dev.upload(model)
     dev.prefill(0, m.random_tokens(3, 0, hp.vocabSize, plen))
     out = dev.decode_loop([dev.greedy_token(0)], warm)
-    dev.synchronize()
-    t0 = time.perf_counter()
-    out = dev.decode_loop([int(out[-1, 0])], steps)
-    dev.synchronize()
-    wall = time.perf_counter() - t0
-    nbytes = float(np.mean([decode_bytes_per_token(hp, plen + warm + 1 + i) for i in range(steps)]))
+    walls = []
+    steps = min(steps, (hp.maxL - plen - warm) // REPS)
+    for _ in range(REPS):
+        dev.synchronize()
+        t0 = time.perf_counter()
+        out = dev.decode_loop([int(out[-1, 0])], steps)
+        dev.synchronize()
+        walls.append(time.perf_counter() - t0)
+    wall = stats(walls)["median"]
+    nbytes = float(np.mean([decode_bytes_per_token(hp, plen + warm + 1 + i) for i in range(REPS * steps)]))
     dev.close()
     return {"workload": "config 3: batch-1 greedy decode, hybrid 3 GDN : 1 attention + PLE at config-2 size, fp32, "
                         "128-token prompt", "steps": steps, "ms_per_step": wall / steps * 1e3, "tok_s": steps / wall,
+            "ms_per_step_stats": stats([w / steps * 1e3 for w in walls]),
             "bytes_per_token": nbytes, "achieved_GBps": nbytes / (wall / steps) / 1e9,
             "frac_of_hbm_peak": nbytes / (wall / steps) / 1e9 / HBM_PEAK_GBPS, "last_ids": [int(x) for x in out[-4:, 0]]}
 
 
-def prefill_leg(m, reps=2):
+def prefill_leg(m, reps=REPS):
     """Configuration 5: 8 prompts of 2048 uniform-random tokens through the bf16 model in one pass.
     MFMA utilisation = algorithmic flops (projections + causal attention, LM head on the last position
-    only) / time / the published dense bf16 peak; the GEMM kernel alone is also timed on the layer's
-    gate/up shape."""
+    only) / time / the published dense bf16 peak; the GEMM kernel alone is also timed on the pass's own
+    gate/up shape (M = 16384 rows)."""
     hp = m.config(5)
     nseq, plen = hp.maxSeqs, 2048
     model = m.Model.generate(hp, seed=5)
     dev = m.Device(hp, 0)
     dev.upload(model)
     prompts = [m.random_tokens(5, s, hp.vocabSize, plen) for s in range(nseq)]
-    best = None
-    for _ in range(reps + 1):  # the first pass allocates the work buffers
+    times = []
+    for i in range(reps + 1):  # the first pass allocates the work buffers and is not counted
         dev.reset()
         dev.synchronize()
         t0 = time.perf_counter()
         dev.prefill_batch(list(range(nseq)), prompts)
         dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
+        if i > 0:
+            times.append(dt)
+    med = stats(times)["median"]
     tokens = nseq * plen
     n_attn = sum(1 for t in range(hp.transformers) if hp.layerKinds[t] == 0)
     flops = 2.0 * tokens * matrix_params(hp) + n_attn * nseq * (4.0 * plen * plen * hp.dim) / 2 + 2.0 * nseq * hp.vocabSize * hp.dim
     firsts = [dev.greedy_token(s) for s in range(nseq)]
-    t0 = time.perf_counter()
-    dev.decode_loop(firsts, 32)
-    dec = (time.perf_counter() - t0) / 32
+    decs = []
+    for _ in range(REPS):
+        dev.synchronize()
+        t0 = time.perf_counter()
+        firsts = [int(t) for t in dev.decode_loop(firsts, 16)[-1]]
+        decs.append((time.perf_counter() - t0) / 16)
+    dec = stats(decs)["median"]
     dev.close()
-    rng = np.random.default_rng(5)
-    a = rng.standard_normal((4096, hp.dim), dtype=np.float32)
-    b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
-    _, us = m.selftest_gemm(a, b, None, f16=True, iters=20)  # the operand type the bf16 model's MFMA path multiplies
-    gemm_tflops = 2.0 * 4096 * 2 * hp.ffnDim * hp.dim / us / 1e6
+    gemm = gemm_leg(m, iters=10, reps=REPS)
     return {"workload": "config 5: 8 x 2048-token prompts, d2048 x 24 layers (3 GDN : 1 attention), 16 heads x 128, "
                         "ffn 5632, vocab 32000, PLE 64, bf16 weights, fp32 accumulation",
-            "tokens": tokens, "ms": best * 1e3, "tok_s": tokens / best, "algo_tflop": flops / 1e12,
-            "achieved_TFLOPs": flops / best / 1e12, "mfma_frac_of_bf16_peak": flops / best / MFMA_BF16_PEAK,
-            "gemm_kernel": {"shape": [4096, 2 * hp.ffnDim, hp.dim], "avg_us": us, "TFLOPs": gemm_tflops,
-                            "frac_of_bf16_peak": gemm_tflops * 1e12 / MFMA_BF16_PEAK},
-            "decode_after_prefill": {"sequences": nseq, "ms_per_step": dec * 1e3, "tok_s": nseq / dec}}
+            "tokens": tokens, "ms": med * 1e3, "ms_stats": stats([t * 1e3 for t in times]), "tok_s": tokens / med,
+            "algo_tflop": flops / 1e12,
+            "achieved_TFLOPs": flops / med / 1e12, "mfma_frac_of_bf16_peak": flops / med / MFMA_BF16_PEAK,
+            "gemm_kernel": gemm,
+            "decode_after_prefill": {"sequences": nseq, "ms_per_step": dec * 1e3, "tok_s": nseq / dec,
+                                     "ms_per_step_stats": stats([d * 1e3 for d in decs])}}
 
 
-def gemm_leg(m, iters=3):
-    """The gate/up product of one config-5 prefill pass alone (16384 x 11264 x 2048, half operands, plain epilogue):
-    the launch the operand-path counters of the big GEMM kernel are collected on."""
+def gemm_leg(m, iters=3, reps=1):
+    """The gate/up product of one config-5 prefill pass alone (16384 x 11264 x 2048, half operands -- what the bf16
+    model's MFMA path multiplies --, plain epilogue, N(0,1) data): mean launch time over `iters` back-to-back
+    launches from HIP events, median of `reps` such runs.  Also the launch the operand-path counters of the big GEMM
+    kernel are collected on."""
     hp = m.config(5)
     M = 8 * 2048
     rng = np.random.default_rng(5)
     a = rng.standard_normal((M, hp.dim), dtype=np.float32)
     b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
-    _, us = m.selftest_gemm(a, b, None, f16=True, iters=iters)
+    runs = [m.selftest_gemm(a, b, None, f16=True, iters=iters)[1] for _ in range(reps)]
+    us = stats(runs)["median"]
     tf = 2.0 * M * 2 * hp.ffnDim * hp.dim / us / 1e6
-    return {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "avg_us": us, "TFLOPs": tf,
+    return {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "avg_us": us, "avg_us_stats": stats(runs), "TFLOPs": tf,
             "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
 
 
 def timed_decode(dev, prompt, K, W, persistent, maxL):
-    """W untimed warm-up steps, then exactly K timed steps with the device idle on both sides.
-    Returns (wall seconds, HIP-event milliseconds of a second identical run, ids)."""
+    """W untimed warm-up steps, then REPS repetitions of exactly K timed steps from the same starting state (prompt
+    prefilled anew each time), the device idle on both sides of each.  Returns (wall seconds per repetition, HIP-event
+    milliseconds per repetition of a second series timed on the context's stream, ids)."""
     dev.set_persistent(persistent)
     dev.reset()
     dev.prefill(0, prompt)
     first = dev.greedy_token(0)
     if W:
         dev.decode_loop([first], min(W, maxL - PROMPT_LEN))
-    dev.reset()
-    dev.prefill(0, prompt)
-    first = dev.greedy_token(0)
-    dev.synchronize()
-    t0 = time.perf_counter()
-    ids = dev.decode_loop([first], K)
-    dev.synchronize()
-    wall = time.perf_counter() - t0
-    dev.reset()
-    dev.prefill(0, prompt)
-    ev_ms = dev.time_decode([first], K)
-    return wall, ev_ms, ids
+    walls, events, ids = [], [], None
+    for _ in range(REPS):
+        dev.reset()
+        dev.prefill(0, prompt)
+        first = dev.greedy_token(0)
+        dev.synchronize()
+        t0 = time.perf_counter()
+        ids = dev.decode_loop([first], K)
+        dev.synchronize()
+        walls.append(time.perf_counter() - t0)
+    for _ in range(REPS):
+        dev.reset()
+        dev.prefill(0, prompt)
+        events.append(dev.time_decode([first], K))
+    return walls, events, ids
 
 
 def main():
@@ -249,7 +299,7 @@ def main():
     ap.add_argument("--steps", type=int, default=512)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU-baseline leg")
-    ap.add_argument("--path", choices=["xcd", "persistent", "kernels", "tagged"], default="xcd",
+    ap.add_argument("--path", choices=["xcd", "persistent", "kernels"], default="xcd",
                     help="decode path reported as `value`")
     ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
     ap.add_argument("--leg", choices=["all", "batched", "prefill", "gemm", "hybrid"], default="all",
@@ -266,7 +316,7 @@ def main():
 
     m = entry.load_package()
     if args.leg != "all":
-        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=1), "gemm": gemm_leg,
+        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=2), "gemm": gemm_leg,
                "hybrid": hybrid_decode_leg}[args.leg]
         print(json.dumps({args.leg: leg(m)}))
         return 0
@@ -284,12 +334,18 @@ def main():
     if args.path == "xcd" and not dev.xcd_decode_supported():
         print("bench.py: the XCD-rank kernel does not cover this device; use --path persistent", file=sys.stderr)
         return 4
-    order = [args.path] if args.only_path else ["kernels", "persistent", "tagged", "xcd"]
+    order = [args.path] if args.only_path else ["kernels", "persistent", "xcd"]
     ids_by_path = {}
     for name in order:
-        wall, ev_ms, ids = timed_decode(dev, prompt, K, W, {"kernels": 0, "persistent": 1, "tagged": 2, "xcd": 3}[name], hp.maxL)
-        paths[name] = {"tok_s": K / wall, "ms_per_step": wall / K * 1e3, "event_ms_per_step": ev_ms / K}
+        walls, events, ids = timed_decode(dev, prompt, K, W, {"kernels": 0, "persistent": 1, "xcd": 3}[name], hp.maxL)
+        wall = stats(walls)["median"]
+        paths[name] = {"tok_s": K / wall, "ms_per_step": wall / K * 1e3, "ms_per_step_stats": stats([w / K * 1e3 for w in walls]),
+                       "event_ms_per_step": stats(events)["median"] / K,
+                       "event_ms_per_step_stats": stats([e / K for e in events])}
         ids_by_path[name] = ids[:, 0]
+        if dev.persistent_fallbacks():
+            print(f"bench.py: path {name} gave up a wait and fell back to the kernel sequence: {m.dev.mlh_last_error(dev._h).decode()}", file=sys.stderr)
+            return 5
     if any(not np.array_equal(v, ids_by_path[args.path]) for v in ids_by_path.values()):
         print("bench.py: the decode paths produced different ids", file=sys.stderr)
         return 3
@@ -324,18 +380,34 @@ def main():
                          "GBps": round(algo.get(name, 0.0) / us / 1e3, 1) if us > 0 else None}
     copy_us, copy_bytes = dev.time_kernel(m.K_COPY, iters=20)
 
-    if args.path in ("persistent", "tagged", "xcd"):
-        # the dominant (only) kernel: one launch = K tokens; duration from HIP events around the launch
+    hops = None
+    try:
+        h = dev.probe_hops(2000)
+        # A layer of the XCD-rank kernel is 2 exchanges across XCDs, each followed by a gather inside the XCD, plus 3
+        # exchanges inside the XCD, plus its five compute phases: the floor these hop times put under a layer pass.
+        hops = {"in_xcd_us": h[0], "cross_xcd_us": h[1], "grid_barrier_us": h[2], "rounds": 2000,
+                "what": "one all-to-all of dim tagged words among the 32 workgroups of an XCD / among all 256 / one grid barrier",
+                "layer_floor_us_xcd_kernel": 2 * (h[1] + h[0]) + 3 * h[0] if min(h[0], h[1]) > 0 else None,
+                "layer_floor_formula": "2 x (cross + in-XCD gather) + 3 x in-XCD, compute phases not counted"}
+    except Exception as e:  # a probe, never required
+        hops = {"failed": repr(e)}
+
+    if args.path in ("persistent", "xcd"):
+        # the dominant (only) kernel: one launch = K tokens; duration from HIP events around the launch (median of REPS)
         launch_us = chosen["event_ms_per_step"] * K * 1e3
         launch_bytes = mean_bytes * K
-        # HBM bytes per launch: rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE (one run each), scaled by what the same
-        # counters read for the 256 MiB copy kernel (reads x 2.0, writes x 1.0), measured on a 16-token launch of the
-        # XCD-rank kernel (the profiler does not survive the 512-token launch): 381.7 MB read + 3.4 MB written per
-        # token against 370.4 MB algorithmic at those lengths.  Not measured for the barrier kernels.
+        # HBM bytes per launch are not counted in this run: the ratio of counted to algorithmic bytes comes from the
+        # tracked profile (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE, one run each, scaled by what the same counters read
+        # for the 256 MiB copy kernel: reads x 2.0, writes x 1.0), taken on a 16-token launch of the XCD-rank kernel:
+        # 381.7 MB read + 3.4 MB written per token against 370.4 MB algorithmic at those lengths.
         traffic_ratio = {"xcd": 1.04}.get(args.path)
-        roofline = {"kernel": {"persistent": "k_decode_persistent", "tagged": "k_decode_tagged", "xcd": "k_decode_xcd"}[args.path], "bound": "hbm", "achieved": launch_bytes / launch_us / 1e3,
+        roofline = {"kernel": {"persistent": "k_decode_persistent", "xcd": "k_decode_xcd"}[args.path], "bound": "hbm", "achieved": launch_bytes / launch_us / 1e3,
                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": launch_bytes / launch_us / 1e3 / HBM_PEAK_GBPS,
-                    "traffic": traffic_ratio * launch_bytes if traffic_ratio else None, "avg_launch_us": launch_us,
+                    "traffic": traffic_ratio * launch_bytes if traffic_ratio else None,
+                    "traffic_source": ("profiles/decode_config2_hbm_traffic.md: counter ratio 1.04 from a 16-token launch under "
+                                       "rocprofv3 --pmc, applied to this run's algorithmic bytes; not counted in this run") if traffic_ratio else None,
+                    "avg_launch_us": launch_us,
+                    "avg_launch_us_stats": {k: (v * K * 1e3 if k != "reps" else v) for k, v in chosen["event_ms_per_step_stats"].items()},
                     "algo_bytes_per_launch": launch_bytes, "tokens_per_launch": K}
     else:
         # dominant = the kernel with the largest share of the step's time
@@ -392,6 +464,8 @@ def main():
                             "weights_resident_in_infinity_cache": False,
                             "note": "365 MB of fp32 weights exceed the 256 MB Infinity Cache"},
         "paths": paths,
+        "protocol": f"median of {REPS} timed repetitions per figure (min and max beside it)",
+        "exchange_latency": hops,
         "kernels": kernels,
         "copy_kernel": {"avg_us": round(copy_us, 2), "GBps": round(copy_bytes / copy_us / 1e3, 1)},
         "cpu_baseline": cpu,

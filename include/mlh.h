@@ -176,16 +176,31 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
 
 /* Batch-1 decode (nseq = 1): mode 1 runs, when the shape allows it, as ONE launch of a
  * persistent kernel (one workgroup per compute unit) that decodes all requested steps: the ~60
- * dependent phases of a token are separated by grid barriers instead of kernel launches.  Mode 2 is
- * the same kernel without barriers (consumers spin on tagged data words).  Both need every compute
- * unit free; their waits are bounded, and a call whose wait expired returns -3 with a message.
- * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says.
+ * dependent phases of a token are separated by grid barriers instead of kernel launches.
  * Mode 3 treats each of the eight XCDs as a tensor-parallel rank (heads and FFN units are split over the
  * XCDs, exchanges inside an XCD go through its L2, only two per layer cross XCDs); it covers models with
  * head size 64 (attention heads; gated-delta-net heads with 64 x 64 states, as many as attention heads;
  * per-layer embeddings of a width that is a multiple of 8) on a 256-unit device
- * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default. */
+ * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default.
+ * Both need every compute unit for themselves and all their waits are bounded: when a launch gives up (units held
+ * by other work), nothing of the sequence has advanced, and the call redoes its steps as the kernel sequence and
+ * leaves the context at mode 0 (mlh_get_persistent, mlh_persistent_fallbacks).
+ * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says. */
 int mlh_set_persistent(mlh_ctx* ctx, int mode);
+
+/* The mode in effect (it differs from what mlh_set_persistent was given after a fallback), and how many decode
+ * calls so far were started as a single launch, gave up a wait and were redone as the kernel sequence.  After such
+ * a call the context stays at mode 0; mlh_last_error keeps the reason. */
+int mlh_get_persistent(mlh_ctx* ctx);
+int mlh_persistent_fallbacks(mlh_ctx* ctx);
+
+/* Test hooks (no counterpart in the reference).  mlh_debug_inject_abort: the next `launches` single-launch decode
+ * launches find their bounded wait already given up (XCD-rank kernel: arrival counters that start full; barrier
+ * kernel: an abort flag that starts raised), so every workgroup leaves at once and the fallback path runs without
+ * any wait having to expire.  mlh_debug_set_xcd_tag: sets the XCD-rank kernel's running tag count (device word and
+ * host mirror), to exercise the reset that precedes a wrap of the 32-bit tags. */
+int mlh_debug_inject_abort(mlh_ctx* ctx, int launches);
+int mlh_debug_set_xcd_tag(mlh_ctx* ctx, unsigned tagsUsed);
 
 /* Next-token rule of the decode entry points.  temperature 0 (the default): greedy, the argmax fused into the
  * LM-head reduction, lowest index on ties (the reference's only mode: it keeps the top entry of a qsort of the
@@ -229,6 +244,14 @@ const char* mlh_kernel_name(int kernel);
  * the launches per step in launches_per_step[MLH_K_COUNT].  The sequences advance by `steps`. */
 int mlh_profile_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, double* us_per_launch,
                        int32_t* launches_per_step);
+
+/* Latency of one dependent exchange between workgroups on this device, the quantity that bounds batch-1 decode
+ * (a token is a chain of about 60 all-to-all exchanges): microseconds per round, over `iters` dependent rounds in
+ * one launch of one workgroup per compute unit, of us[0] an all-to-all of `dim` tagged words among the workgroups
+ * of one XCD through its L2, us[1] the same among all workgroups through the memory side, us[2] a two-level grid
+ * barrier of relaxed atomics.  A figure of -1 means that probe's bounded wait expired.  Measurement support; no
+ * counterpart in the reference. */
+int mlh_probe_hops(mlh_ctx* ctx, int iters, double* us);
 
 /* Times `steps` decode steps (graph replays, argmax fed back on the device)
  * with HIP events on the context's stream: total milliseconds. */

@@ -90,6 +90,10 @@ _sigs_dev = {
     "mlh_set_graph": (c_int, [c_void_p, c_int]),
     "mlh_set_sampling": (c_int, [c_void_p, c_float, ctypes.c_ulonglong]),
     "mlh_set_persistent": (c_int, [c_void_p, c_int]),
+    "mlh_get_persistent": (c_int, [c_void_p]),
+    "mlh_persistent_fallbacks": (c_int, [c_void_p]),
+    "mlh_debug_inject_abort": (c_int, [c_void_p, c_int]),
+    "mlh_debug_set_xcd_tag": (c_int, [c_void_p, ctypes.c_uint]),
     "mlh_xcd_decode_supported": (c_int, [c_void_p]),
     "mlh_synchronize": (c_int, [c_void_p]),
     "mlh_time_kernel": (c_int, [c_void_p, c_int, c_int, c_int, c_int, _P(c_double), _P(c_double)]),
@@ -98,6 +102,7 @@ _sigs_dev = {
     "mlh_selftest_gemm": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, _P(c_double)]),
     "mlh_gemm_device_init": (c_int, [c_int]),
     "mlh_gemm_device": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "mlh_probe_hops": (c_int, [c_void_p, c_int, _P(c_double)]),
     "mlh_profile_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double), _P(c_int32)]),
 }
 _sigs_host = {
@@ -341,6 +346,18 @@ class Device:
     def set_persistent(self, enabled):
         self._check(dev.mlh_set_persistent(self._h, int(enabled)))
 
+    def get_persistent(self):
+        return dev.mlh_get_persistent(self._h)
+
+    def persistent_fallbacks(self):
+        return dev.mlh_persistent_fallbacks(self._h)
+
+    def debug_inject_abort(self, launches):
+        self._check(dev.mlh_debug_inject_abort(self._h, int(launches)))
+
+    def debug_set_xcd_tag(self, tags_used):
+        self._check(dev.mlh_debug_set_xcd_tag(self._h, int(tags_used)))
+
     def xcd_decode_supported(self):
         return bool(dev.mlh_xcd_decode_supported(self._h))
 
@@ -351,6 +368,12 @@ class Device:
         us, nbytes = c_double(), c_double()
         self._check(dev.mlh_time_kernel(self._h, kernel, layer, nseq, iters, byref(us), byref(nbytes)))
         return us.value, nbytes.value
+
+    def probe_hops(self, iters=2000):
+        """Microseconds per dependent exchange: (inside one XCD, across XCDs, grid barrier); -1 where a wait expired."""
+        us = (c_double * 3)()
+        self._check(dev.mlh_probe_hops(self._h, iters, us))
+        return tuple(us)
 
     def profile_decode(self, first_ids, steps):
         """In-sequence mean microseconds per launch (run time plus the launch gap before it) and

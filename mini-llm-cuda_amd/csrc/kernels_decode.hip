@@ -1040,6 +1040,11 @@ int mlh_launch_one(mlh_ctx* c, int kernel, int layer, int nseq) {
 }
 
 int mlh_launch_copy(mlh_ctx* c) {
+    if (!c->copySrc) { // the calibration buffers exist only once the copy has been asked for
+        int rc;
+        if ((rc = mlh_dev_alloc_bytes(c, &c->copySrc, c->copyBytes)) || (rc = mlh_dev_alloc_bytes(c, &c->copyDst, c->copyBytes))) return rc;
+        MLH_CHECK(c, hipMemsetAsync(c->copySrc, 0, c->copyBytes, c->stream));
+    }
     hipLaunchKernelGGL(k_copy, dim3(2048), dim3(256), 0, c->stream, (const float4*)c->copySrc,
                        (float4*)c->copyDst, c->copyBytes / 16);
     hipError_t e = hipGetLastError();

@@ -161,8 +161,6 @@ struct PersistArgs {
     int maxTiles;
     int stageFloats;     // LDS staging vector length
     unsigned long long* timing; // optional (may be null): phase timestamps of workgroup 0 during the last step
-    // tagged-exchange variant: (value, tag) words
-    unsigned long long *tx, *tqkv, *tpart, *tmix, *th1, *tu, *tamax;
 };
 
 // Diagnostic: workgroup 0 records the constant-rate clock at phase boundaries of the last step.
@@ -197,9 +195,14 @@ __device__ __forceinline__ bool grid_wait(const PersistArgs& P, unsigned epoch) 
     if (threadIdx.x == 0) {
         const unsigned* rel = P.sync + 64 * (9 + (blockIdx.x & 7));
         unsigned spins = 0, ok = 1;
-        while (aldu(rel) < epoch) {
-            if (++spins > P_SPIN_LIMIT || ((spins & 1023) == 0 && aldu(P.abortFlag))) { astu(P.abortFlag, 1u); ok = 0; break; }
-        }
+        // the first look takes the abort flag along (both loads are in flight together): a launch whose flag is already
+        // raised is left by every workgroup at its first wait, before anything of the sequence has been written
+        const unsigned r0 = aldu(rel), ab0 = aldu(P.abortFlag);
+        if (ab0) ok = 0;
+        else if (r0 < epoch)
+            while (aldu(rel) < epoch) {
+                if (++spins > P_SPIN_LIMIT || ((spins & 1023) == 0 && aldu(P.abortFlag))) { astu(P.abortFlag, 1u); ok = 0; break; }
+            }
         s_ok = ok;
     }
     lds_barrier();
@@ -655,485 +658,7 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
     }
 }
 
-// ----------------------------------------------------------------------------
-// Tagged-exchange variant: no grid barrier at all.  Every value that another workgroup reads
-// travels as one 64-bit word (value, tag) written with an agent-scope atomic store; the tag is the
-// number of the phase that produced it (phases count up through the launch, the buffers start at
-// zero).  A consumer simply loads the words it needs until they carry the tag it expects: data
-// arrival IS the synchronisation, one memory round trip per phase instead of store-acknowledge +
-// barrier + load.  A workgroup cannot run more than one phase ahead of the slowest one (every phase
-// needs the previous phase's output of ALL workgroups), and each buffer is rewritten only five phases
-// later, so a word is never overwritten before its readers are done.  Waits are bounded; an expired
-// wait raises the abort flag and every workgroup leaves.
-// ----------------------------------------------------------------------------
-#define T_SPIN_LIMIT (1u << 20)
-__device__ __forceinline__ unsigned long long ald64(const unsigned long long* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void tst(unsigned long long* p, float v, unsigned tag) {
-    __hip_atomic_store(p, ((unsigned long long)tag << 32) | __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// one tagged value; ok turns false (and stays) when the wait expires
-__device__ __forceinline__ float tld(const unsigned long long* p, unsigned tag, bool& ok) {
-    for (unsigned spins = 0;; spins++) {
-        const unsigned long long w = ald64(p);
-        if ((unsigned)(w >> 32) == tag) return __uint_as_float((unsigned)w);
-        if (!ok || spins > T_SPIN_LIMIT) { ok = false; return 0.f; }
-    }
-}
-// a whole vector into LDS, four words per thread in flight at a time
-__device__ __forceinline__ void tld_vec(const unsigned long long* src, int n, unsigned tag, float* dst, bool& ok) {
-    for (int i0 = threadIdx.x; i0 < n; i0 += 4 * PWG) {
-        unsigned long long w[4];
-        for (unsigned spins = 0;; spins++) {
-            bool all = true;
-#pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const int i = i0 + k * PWG;
-                w[k] = i < n ? ald64(src + i) : ((unsigned long long)tag << 32);
-                all = all && (unsigned)(w[k] >> 32) == tag;
-            }
-            if (all) break;
-            if (!ok || spins > T_SPIN_LIMIT) { ok = false; break; }
-        }
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int i = i0 + k * PWG;
-            if (i < n) dst[i] = __uint_as_float((unsigned)w[k]);
-        }
-    }
-}
-// after a section of waits: the workgroup agrees on whether anyone gave up, and leaves together if so
-#define T_FAILCHECK()                                            \
-    do {                                                         \
-        if (!ok) { s_fail = 1; astu(P.abortFlag, 1u); }          \
-        lds_barrier();                                           \
-        if (s_fail) return;                                      \
-    } while (0)
-
-template <typename WT, int HD, int GDK>
-__global__ void __launch_bounds__(PWG) k_decode_tagged(PersistArgs P) {
-    extern __shared__ float lds[];
-    const StepArgs& a = P.a;
-    const int d = a.dim, F = a.ffn, V = a.vocab;
-    float* xres = lds;                 // [d] residual stream entering the layer
-    float* h1res = xres + d;           // [d] residual after the mixing block
-    float* stage = h1res + d;          // [stageFloats] normed input / mixing output / FFN activations
-    float* red = stage + P.stageFloats; // [PWAVES + 2*PWAVES] reductions and argmax scratch
-    float* g1s = red + 4 * PWAVES;     // [d] rms1 gain of the current layer (final gain during the LM head)
-    float* g2s = g1s + d;              // [d] rms2 gain
-    float* gqs = g2s + d;              // [d] per-head q gain
-    float* gks = gqs + d;              // [d] per-head k gain
-    float* tiles = gks + d;            // attention tiles, PAttn<HD>::NW x TILE_FLOATS
-    LayerDev* Ls = reinterpret_cast<LayerDev*>(tiles + PAttn<HD>::NW * PAttn<HD>::TILE_FLOATS); // the layer table (8-byte aligned: all lengths above are even)
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    for (int i = tid; i < P.NL * (int)(sizeof(LayerDev) / 4); i += PWG)
-        reinterpret_cast<uint32_t*>(Ls)[i] = reinterpret_cast<const uint32_t*>(P.layers)[i];
-    lds_barrier();
-    const int G = gridDim.x, wg = blockIdx.x;
-    const int TW = G * PWAVES;         // waves in the grid
-    const int gw = wave * G + wg;      // consecutive rows land on different workgroups
-    const int seq = P.seq;
-    __shared__ int s_fail;
-    if (tid == 0) s_fail = 0;
-    lds_barrier();
-    bool ok = true;   // false once a bounded wait of this thread has expired
-    unsigned ph = 0;  // tag of the last phase whose outputs have been written (phases count up from 1)
-    int tok = a.tok[0];
-    int pos = a.pos[seq];
-    RowPf<WT> pf;
-
-    for (int step = 0; step < P.steps; step++) {
-        // embedding gather (inference.cu:9-22): every workgroup keeps its own copy of the residual stream
-        for (int i = tid; i < d; i += PWG) xres[i] = PVec<WT>::one((const WT*)a.E + (size_t)tok * d + i);
-        pf_first<WT>(pf, (const WT*)Ls[P.NL - 1].Wa, d, Ls[P.NL - 1].rowsA, d, gw, TW);
-
-        for (int t = P.NL - 1; t >= 0; t--) { // file block 0 is the top of the stack (inference.cu:384-385)
-            // The layer table sits in LDS (copied once at kernel start): no dependent global loads for the
-            // pointers, and no registers held for them; gains and the residual stream arrive in one round of loads.
-            const LayerDev& L = Ls[t];
-            const LayerDev& Lnext = Ls[t > 0 ? t - 1 : P.NL - 1];
-            const int ts = (P.NL - 1 - t) * 16;
-            P_STAMP(ts + 0);
-            {
-                const bool qk = a.qkNorm && L.kind == MLH_KIND_ATTENTION;
-                if (t != P.NL - 1) tld_vec(P.tx, d, ph, xres, ok); // written by phase E of the layer below
-                for (int i = tid; i < d; i += PWG) {
-                    g1s[i] = L.g1[i];
-                    g2s[i] = L.g2[i];
-                    if (qk) { gqs[i] = L.gq[i]; gks[i] = L.gk[i]; }
-                }
-                T_FAILCHECK();
-            }
-            P_STAMP(ts + 1);
-            // ------------------------------------------------------------------ phase A
-            lds_rmsnorm(xres, g1s, d, stage, red);
-            P_STAMP(ts + 2);
-            rows_phase<WT>(pf, (const WT*)L.Wa, d, L.rowsA, d, stage, (const WT*)nullptr, 0, nullptr, gw, TW,
-                           [&](int row, float v) { tst(P.tqkv + row, v, ph + 1); });
-            P_STAMP(ts + 3);
-
-            // ------------------------------------------------------------------ phase B
-            if (L.kind == MLH_KIND_ATTENTION) {
-                constexpr int NW = PAttn<HD>::NW, LDK = PAttn<HD>::LDK, EPL = PAttn<HD>::EPL;
-                constexpr int LPR = HD / 4, RPI = 64 / LPR, NLD = 64 / RPI;
-                const int T = pos + 1, ntiles = (T + 63) >> 6, newTile = pos >> 6;
-                const int nunits = a.heads * ntiles;
-                if (wave < NW) {
-                    float* tile = tiles + wave * PAttn<HD>::TILE_FLOATS;
-                    float* qs = tile + 64 * LDK;
-                    float* ks = qs + HD;
-                    float* vn = ks + HD;
-                    const int lrow = lane / LPR, c4 = (lane % LPR) * 4;
-                    for (int u = wave * G + wg; u < nunits; u += NW * G) {
-                        const int h = u % a.heads, tl = u / a.heads, j0 = tl << 6;
-                        const int page = a.pageTable[seq * a.pagesPerSeq + tl];
-                        const size_t base = ((size_t)page * MLH_KV_PAGE) * d + h * HD;
-                        // one staging set of registers: K tile first, reused for the V tile once K sits in LDS
-                        f32x4 kreg[NLD];
-#pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            kreg[it] = (j0 + row < pos) ? *reinterpret_cast<const f32x4*>(L.K + base + (size_t)row * d + c4) : (f32x4)(0.f);
-                        }
-                        const float rc0 = a.rope[(size_t)pos * HD + (EPL == 1 ? (lane & ~1) : 2 * lane)];
-                        const float rs0 = a.rope[(size_t)pos * HD + (EPL == 1 ? (lane | 1) : 2 * lane + 1)];
-                        // q (and, for the tile that receives this step's row, k and v): per-head RMSNorm
-                        // (inference.cu:52-81, 97-111) then RoPE on adjacent pairs (inference.cu:113-134)
-                        const bool own = tl == newTile;
-                        float qv[EPL], kv[EPL], vv[EPL];
-#pragma unroll
-                        for (int e = 0; e < EPL; e++) {
-                            const int i = lane * EPL + e;
-                            qv[e] = tld(P.tqkv + h * HD + i, ph + 1, ok);
-                            kv[e] = own ? tld(P.tqkv + L.offK + h * HD + i, ph + 1, ok) : 0.f;
-                            vv[e] = own ? tld(P.tqkv + L.offV + h * HD + i, ph + 1, ok) : 0.f;
-                        }
-                        if (a.qkNorm) {
-                            float sq = 0.f, sk = 0.f;
-#pragma unroll
-                            for (int e = 0; e < EPL; e++) { sq = fmaf(qv[e], qv[e], sq); sk = fmaf(kv[e], kv[e], sk); }
-                            sq = pwave_sum(sq); sk = pwave_sum(sk);
-                            const float rq = sqrtf(sq / (float)HD + 1e-8f), rk = sqrtf(sk / (float)HD + 1e-8f);
-#pragma unroll
-                            for (int e = 0; e < EPL; e++) {
-                                const int i = lane * EPL + e;
-                                qv[e] = gqs[h * HD + i] * (qv[e] / rq);
-                                kv[e] = gks[h * HD + i] * (kv[e] / rk);
-                            }
-                        }
-                        if (EPL == 1) { // pair (2i, 2i+1) sits in lanes (2i, 2i+1)
-                            const float c = rc0, s = rs0;
-                            const float qo = __shfl_xor(qv[0], 1, MLH_WAVE), ko = __shfl_xor(kv[0], 1, MLH_WAVE);
-                            if (lane & 1) { qv[0] = s * qo + c * qv[0]; kv[0] = s * ko + c * kv[0]; }
-                            else { qv[0] = c * qv[0] - s * qo; kv[0] = c * kv[0] - s * ko; }
-                        } else { // the lane holds the pair (2*lane, 2*lane+1)
-                            const float c = rc0, s = rs0;
-                            const float q0 = qv[0], q1 = qv[EPL - 1], k0 = kv[0], k1 = kv[EPL - 1];
-                            qv[0] = c * q0 - s * q1; qv[EPL - 1] = s * q0 + c * q1;
-                            kv[0] = c * k0 - s * k1; kv[EPL - 1] = s * k0 + c * k1;
-                        }
-#pragma unroll
-                        for (int e = 0; e < EPL; e++) {
-                            const int i = lane * EPL + e;
-                            qs[i] = qv[e]; ks[i] = kv[e]; vn[i] = vv[e];
-                            if (own) { // append this step's row to the cache (write-through: read next step by any XCD)
-                                const size_t o = base + (size_t)(pos - j0) * d + i;
-                                ast(L.K + o, kv[e]);
-                                ast(L.V + o, vv[e]);
-                            }
-                        }
-                        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            f32x4 v = kreg[it];
-                            if (j0 + row == pos) v = *reinterpret_cast<const f32x4*>(ks + c4);
-                            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
-                        }
-                        // V tile loads go out now, into the same registers, and fly during the score computation
-#pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            kreg[it] = (j0 + row < pos) ? *reinterpret_cast<const f32x4*>(L.V + base + (size_t)row * d + c4) : (f32x4)(0.f);
-                        }
-                        __builtin_amdgcn_wave_barrier();
-                        float s = 0.f;
-                        {
-                            const float* kr = tile + lane * LDK;
-#pragma unroll
-                            for (int i = 0; i < HD; i += 4) {
-                                const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + i);
-                                const f32x4 qq = *reinterpret_cast<const f32x4*>(qs + i);
-                                s = fmaf(kk.x, qq.x, s); s = fmaf(kk.y, qq.y, s); s = fmaf(kk.z, qq.z, s); s = fmaf(kk.w, qq.w, s);
-                            }
-                        }
-                        const bool valid = j0 + lane < T;
-                        s = valid ? s / sqrtf((float)HD) : -1.0e30f; // inference.cu:154
-                        const float m = pwave_max(s);
-                        const float e = valid ? expf(s - m) : 0.f;
-                        const float l = pwave_sum(e);
-                        __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            f32x4 v = kreg[it];
-                            if (j0 + row == pos) v = *reinterpret_cast<const f32x4*>(vn + c4);
-                            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
-                        }
-                        __builtin_amdgcn_wave_barrier();
-                        float acc[EPL];
-#pragma unroll
-                        for (int ee = 0; ee < EPL; ee++) acc[ee] = 0.f;
-#pragma unroll
-                        for (int j = 0; j < 64; j++) {
-                            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), j));
-#pragma unroll
-                            for (int ee = 0; ee < EPL; ee++) acc[ee] = fmaf(pj, tile[j * LDK + lane + 64 * ee], acc[ee]);
-                        }
-                        // the appended K/V row must have landed before anyone can see this partial (the next
-                        // token's readers are ordered after it through the chain of tagged exchanges)
-                        if (own) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-                        unsigned long long* out = P.tpart + ((size_t)h * P.maxTiles + tl) * (HD + 2);
-#pragma unroll
-                        for (int ee = 0; ee < EPL; ee++) tst(out + lane + 64 * ee, acc[ee], ph + 2);
-                        if (lane == 0) { tst(out + HD, m, ph + 2); tst(out + HD + 1, l, ph + 2); }
-                        __builtin_amdgcn_wave_barrier();
-                    }
-                }
-            } else if (GDK > 0) {
-                // gated-delta-net: one head's state per workgroup; S <- alpha (S - beta (S k) k^T) + beta v k^T ; o = S q
-                constexpr int DK = GDK > 0 ? GDK : 64, DV = DK;
-                constexpr int EPT = DK * DV / PWG; // state elements per thread, contiguous in a row
-                constexpr int TPR = DK / EPT;      // threads per state row
-                float* qs = stage;                 // the normed input in `stage` is no longer needed
-                float* ks = stage + DK;
-                for (int h = wg; h < a.gdnHeads; h += G) {
-                    lds_barrier();
-                    for (int i = tid; i < DK; i += PWG) { qs[i] = tld(P.tqkv + h * DK + i, ph + 1, ok); ks[i] = tld(P.tqkv + L.offK + h * DK + i, ph + 1, ok); }
-                    lds_barrier();
-                    float sq = 0.f, sk = 0.f;
-#pragma unroll 8
-                    for (int i = 0; i < DK; i++) { sq = fmaf(qs[i], qs[i], sq); sk = fmaf(ks[i], ks[i], sk); }
-                    const float rq = sqrtf(sq + 1e-6f), rk = sqrtf(sk + 1e-6f);
-                    const float za = tld(P.tqkv + L.offGa + h, ph + 1, ok) + L.gdnBa[h];
-                    const float zb = tld(P.tqkv + L.offGb + h, ph + 1, ok) + L.gdnBb[h];
-                    const float alpha = expf(-(fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)))));
-                    const float beta = psigmoid(zb);
-                    const int r = tid / TPR, c0 = (tid % TPR) * EPT;
-                    const float vr = tld(P.tqkv + L.offV + h * DV + r, ph + 1, ok);
-                    float* Srow = L.S + (((size_t)seq * a.gdnHeads + h) * DV + r) * DK + c0;
-                    float S[EPT];
-#pragma unroll
-                    for (int c = 0; c < EPT; c += 4) {
-                        const f32x4 v = *reinterpret_cast<const f32x4*>(Srow + c);
-                        S[c] = v.x; S[c + 1] = v.y; S[c + 2] = v.z; S[c + 3] = v.w;
-                    }
-                    float u = 0.f;
-#pragma unroll
-                    for (int c = 0; c < EPT; c++) u = fmaf(S[c], ks[c0 + c] / rk, u);
-#pragma unroll
-                    for (int o = TPR / 2; o > 0; o >>= 1) u += __shfl_xor(u, o, MLH_WAVE);
-                    float oacc = 0.f;
-#pragma unroll
-                    for (int c = 0; c < EPT; c++) {
-                        const float kn = ks[c0 + c] / rk;
-                        S[c] = alpha * (S[c] - beta * u * kn) + beta * vr * kn;
-                        oacc = fmaf(S[c], qs[c0 + c] / rq, oacc);
-                    }
-#pragma unroll
-                    for (int o = TPR / 2; o > 0; o >>= 1) oacc += __shfl_xor(oacc, o, MLH_WAVE);
-                    // the state of a head is always handled by the same workgroup, so ordinary stores do:
-                    // the only other readers come after the end of the kernel
-#pragma unroll
-                    for (int c = 0; c < EPT; c += 4) {
-                        f32x4 v; v.x = S[c]; v.y = S[c + 1]; v.z = S[c + 2]; v.w = S[c + 3];
-                        *reinterpret_cast<f32x4*>(Srow + c) = v;
-                    }
-                    if ((tid % TPR) == 0) tst(P.tmix + h * DV + r, oacc, ph + 2);
-                }
-            }
-            pf_first<WT>(pf, (const WT*)L.Wo, L.ad, d, L.ad, gw, TW);
-            P_STAMP(ts + 4);
-            // the GDN phase keeps q and k in `stage`, which the next phase overwrites: every wave must be done with them
-            // (there is no grid barrier here to do that as a side effect)
-            lds_barrier();
-
-            // ------------------------------------------------------------------ phase C
-            {
-                const int ad = L.ad, pl = a.ple;
-                float* as = stage;
-                float* es = stage + ad;
-                if (L.kind == MLH_KIND_ATTENTION) {
-                    const int ntiles = (pos + 64) >> 6;
-                    for (int i = tid; i < ad; i += PWG) {
-                        const int h = i / HD, e = i - h * HD;
-                        const unsigned long long* pp = P.tpart + ((size_t)h * P.maxTiles) * (HD + 2);
-                        // partials are fetched eight tiles at a time, all loads of a batch in flight together
-                        float M = -1.0e30f, num = 0.f, den = 0.f;
-                        for (int t0 = 0; t0 < ntiles; t0 += 8) {
-                            float pm[8], pl_[8], pa[8];
-                            for (unsigned spins = 0;; spins++) { // all 24 loads of the batch in flight together, again until every tag is there
-                                bool all = true;
-#pragma unroll
-                                for (int k = 0; k < 8; k++) {
-                                    const bool in = t0 + k < ntiles;
-                                    const unsigned long long* q = pp + (in ? t0 + k : 0) * (HD + 2);
-                                    const unsigned long long w0 = ald64(q + HD), w1 = ald64(q + HD + 1), w2 = ald64(q + e);
-                                    all = all && (!in || ((unsigned)(w0 >> 32) == ph + 2 && (unsigned)(w1 >> 32) == ph + 2 && (unsigned)(w2 >> 32) == ph + 2));
-                                    pm[k] = in ? __uint_as_float((unsigned)w0) : -1.0e30f;
-                                    pl_[k] = in ? __uint_as_float((unsigned)w1) : 0.f;
-                                    pa[k] = in ? __uint_as_float((unsigned)w2) : 0.f;
-                                }
-                                if (all) break;
-                                if (!ok || spins > T_SPIN_LIMIT || ((spins & 1023) == 1023 && aldu(P.abortFlag))) { ok = false; break; }
-                            }
-                            float Mb = M;
-#pragma unroll
-                            for (int k = 0; k < 8; k++) Mb = fmaxf(Mb, pm[k]);
-                            const float corr = expf(M - Mb);
-                            num *= corr; den *= corr;
-#pragma unroll
-                            for (int k = 0; k < 8; k++) {
-                                const float w = expf(pm[k] - Mb);
-                                num = fmaf(w, pa[k], num);
-                                den = fmaf(w, pl_[k], den);
-                            }
-                            M = Mb;
-                        }
-                        float v = num / den;
-                        if (a.gating) v = v * psigmoid(tld(P.tqkv + L.offG + i, ph + 1, ok)); // inference.cu:241-250
-                        as[i] = v;
-                    }
-                } else {
-                    tld_vec(P.tmix, ad, ph + 2, as, ok);
-                }
-                for (int j = tid; j < pl; j += PWG)
-                    es[j] = psilu(tld(P.tqkv + L.offPle + j, ph + 1, ok)) * PVec<WT>::one((const WT*)L.pleTable + (size_t)tok * pl + j);
-                T_FAILCHECK();
-                P_STAMP(ts + 5);
-                rows_phase<WT>(pf, (const WT*)L.Wo, ad, d, ad, as, (const WT*)L.pleUp, pl, es, gw, TW,
-                               [&](int row, float v) { tst(P.th1 + row, v + xres[row], ph + 3); }); // inference.cu:252-260
-            P_STAMP(ts + 6);
-            }
-            {
-                const int pr = gw < F ? gw : -1;
-                pf_rows<WT>(pf, (const WT*)L.W13, d, pr < 0 ? -1 : 2 * pr, pr < 0 ? -1 : 2 * pr + 1, d);
-            }
-
-            // ------------------------------------------------------------------ phase D
-            tld_vec(P.th1, d, ph + 3, h1res, ok);
-            T_FAILCHECK();
-            P_STAMP(ts + 7);
-            lds_rmsnorm(h1res, g2s, d, stage, red);
-            P_STAMP(ts + 8);
-            for (int pr = gw; pr < F; pr += TW) {
-                float g = 0.f, up = 0.f;
-                if (pr == gw) dot_pf<WT, true>(pf, (const WT*)L.W13, d, 2 * pr, 2 * pr + 1, d, stage, g, up);
-                else { g = dot_stream<WT>((const WT*)L.W13, d, 2 * pr, d, stage); up = dot_stream<WT>((const WT*)L.W13, d, 2 * pr + 1, d, stage); }
-                g = pwave_sum(g); up = pwave_sum(up);
-                if (lane == 0) tst(P.tu + pr, psilu(g) * up, ph + 4); // inference.cu:262-281
-            }
-            P_STAMP(ts + 9);
-            pf_first<WT>(pf, (const WT*)L.W2, F, d, F, gw, TW);
-
-            // ------------------------------------------------------------------ phase E
-            lds_barrier(); // every wave is done with the normed input in `stage`
-            tld_vec(P.tu, F, ph + 4, stage, ok);
-            T_FAILCHECK();
-            P_STAMP(ts + 10);
-            rows_phase<WT>(pf, (const WT*)L.W2, F, d, F, stage, (const WT*)nullptr, 0, nullptr, gw, TW,
-                           [&](int row, float v) { tst(P.tx + row, v + h1res[row], ph + 5); }); // inference.cu:283-291
-            P_STAMP(ts + 11);
-            ph += 5;
-            P_STAMP(ts + 12); P_STAMP(ts + 13); P_STAMP(ts + 14); P_STAMP(ts + 15);
-            if (t > 0) pf_first<WT>(pf, (const WT*)Lnext.Wa, d, Lnext.rowsA, d, gw, TW);
-            else pf_first<WT>(pf, (const WT*)a.E, d, V, d, gw, TW);
-        }
-
-        // ---------------------------------------------------------------------- LM head + argmax
-        tld_vec(P.tx, d, ph, xres, ok);
-        for (int i = tid; i < d; i += PWG) g1s[i] = a.gF[i];
-        T_FAILCHECK();
-        lds_rmsnorm(xres, g1s, d, stage, red); // inference.cu:705-715
-        float best = -3.0e38f;
-        int bidx = 0x7fffffff;
-        for (int row = gw; row < V; row += 2 * TW) { // rows ascend per wave: ties keep the lower index
-            const int row2 = row + TW < V ? row + TW : -1;
-            float a0 = 0.f, a1 = 0.f;
-            if (row == gw) {
-                if (row2 >= 0) dot_pf<WT, true>(pf, (const WT*)a.E, d, row, row2, d, stage, a0, a1);
-                else dot_pf<WT, false>(pf, (const WT*)a.E, d, row, -1, d, stage, a0, a1);
-            } else {
-                a0 = dot_stream<WT>((const WT*)a.E, d, row, d, stage);
-                if (row2 >= 0) a1 = dot_stream<WT>((const WT*)a.E, d, row2, d, stage);
-            }
-            a0 = pwave_sum(a0);
-            if (lane == 0) a.logits[(size_t)seq * V + row] = a0;
-            if (a0 > best) { best = a0; bidx = row; }
-            if (row2 >= 0) {
-                a1 = pwave_sum(a1);
-                if (lane == 0) a.logits[(size_t)seq * V + row2] = a1;
-                if (a1 > best) { best = a1; bidx = row2; }
-            }
-        }
-        {
-            float* bv = red + PWAVES;
-            int* bi = (int*)(red + 2 * PWAVES);
-            lds_barrier();
-            if (lane == 0) { bv[wave] = best; bi[wave] = bidx; }
-            lds_barrier();
-            if (tid == 0) {
-                float v = bv[0];
-                int i = bi[0];
-                for (int w = 1; w < PWAVES; w++)
-                    if (bv[w] > v || (bv[w] == v && bi[w] < i)) { v = bv[w]; i = bi[w]; }
-                tst(P.tamax + 2 * wg, v, ph + 1);
-                tst(P.tamax + 2 * wg + 1, __uint_as_float((unsigned)i), ph + 1);
-            }
-        }
-        {
-            float v = -3.0e38f;
-            int i = 0x7fffffff;
-            for (int k = tid; k < G; k += PWG) {
-                const float v2 = tld(P.tamax + 2 * k, ph + 1, ok);
-                const int i2 = (int)__float_as_uint(tld(P.tamax + 2 * k + 1, ph + 1, ok));
-                if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
-            }
-            // reduce (v, i) over the block: value max, lowest index on ties
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) {
-                const float v2 = __shfl_xor(v, o, MLH_WAVE);
-                const int i2 = __shfl_xor(i, o, MLH_WAVE);
-                if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
-            }
-            float* bv = red + PWAVES;
-            int* bi = (int*)(red + 2 * PWAVES);
-            ph += 1;
-            T_FAILCHECK();
-            if (lane == 0) { bv[wave] = v; bi[wave] = i; }
-            lds_barrier();
-            v = bv[0]; i = bi[0];
-#pragma unroll
-            for (int w = 1; w < PWAVES; w++)
-                if (bv[w] > v || (bv[w] == v && bi[w] < i)) { v = bv[w]; i = bi[w]; }
-            if (i < 0 || i >= V) i = 0; // only reachable with non-finite logits
-            tok = i;
-            pos += 1;
-            if (wg == 0 && tid == 0) { // the append of inference_orchestrator.cu:149-151, kept on the device
-                const int sc = *a.stepCounter;
-                if (sc + step < a.outCapacity) a.outIds[sc + step] = tok;
-            }
-            lds_barrier();
-        }
-    }
-    if (wg == 0 && tid == 0) {
-        *a.stepCounter += P.steps;
-        a.pos[seq] = pos;
-        ((int*)a.tok)[0] = tok;
-        a.nextTok[seq] = tok;
-    }
-}
+__global__ void k_set_word(unsigned* p, unsigned v) { *p = v; }
 
 __global__ void k_zero_words(unsigned* p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -1145,12 +670,15 @@ __global__ void k_zero_words(unsigned* p, int n) {
 // ----------------------------------------------------------------------------
 template <typename WT, int HD, int GDK>
 static int launch_persistent(mlh_ctx* c, PersistArgs& P, size_t ldsBytes) {
-    const bool tagged = c->usePersistent == 2;
-    void* fn = tagged ? reinterpret_cast<void*>(&k_decode_tagged<WT, HD, GDK>) : reinterpret_cast<void*>(&k_decode_persistent<WT, HD, GDK>);
-    MLH_CHECK(c, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
-    int perCu = 0;
-    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, fn, PWG, ldsBytes));
-    if (perCu < 1) { c->err = "persistent decode kernel does not fit on a compute unit"; return -1; }
+    void* fn = reinterpret_cast<void*>(&k_decode_persistent<WT, HD, GDK>);
+    if (!c->persistentPrepared) { // once per context
+        MLH_CHECK(c, hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+        int perCu = 0;
+        MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, fn, PWG, ldsBytes));
+        if (perCu < 1) { c->err = "persistent decode kernel does not fit on a compute unit"; return -1; }
+        c->persistentPrepared = true;
+    }
+    if (P.steps <= 0) return 0; // preparation only
     void* args[] = {&P};
     // All workgroups must be resident at once: the grid is one workgroup per compute unit and the
     // occupancy query above says each unit can hold one.  A plain launch then behaves like a
@@ -1160,8 +688,7 @@ static int launch_persistent(mlh_ctx* c, PersistArgs& P, size_t ldsBytes) {
     if (coop) {
         MLH_CHECK(c, hipLaunchCooperativeKernel(fn, dim3(c->numCUs), dim3(PWG), args, (unsigned)ldsBytes, c->stream));
     } else {
-        if (tagged) hipLaunchKernelGGL((k_decode_tagged<WT, HD, GDK>), dim3(c->numCUs), dim3(PWG), ldsBytes, c->stream, P);
-        else hipLaunchKernelGGL((k_decode_persistent<WT, HD, GDK>), dim3(c->numCUs), dim3(PWG), ldsBytes, c->stream, P);
+        hipLaunchKernelGGL((k_decode_persistent<WT, HD, GDK>), dim3(c->numCUs), dim3(PWG), ldsBytes, c->stream, P);
         MLH_CHECK(c, hipGetLastError());
     }
     return 0;
@@ -1203,20 +730,11 @@ int mlh_launch_persistent(mlh_ctx* c, int steps) {
     const size_t tileFloats = hd == 64 ? (size_t)PAttn<64>::NW * PAttn<64>::TILE_FLOATS : (size_t)PAttn<128>::NW * PAttn<128>::TILE_FLOATS;
     const size_t ldsBytes = ((size_t)6 * hp.dim + stage + 4 * PWAVES + tileFloats) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
     if (ldsBytes > 160 * 1024) { c->err = "model too wide for the persistent decode kernel"; return -1; }
-    hipLaunchKernelGGL(k_zero_words, dim3(6), dim3(256), 0, c->stream, c->d_sync, 64 * 24); // barrier words and abort flag
-    if (c->usePersistent == 2) { // tagged exchange words start at tag 0 (phases count from 1)
-        const int words32 = (int)(c->taggedWords * 2);
-        hipLaunchKernelGGL(k_zero_words, dim3((words32 + 255) / 256), dim3(256), 0, c->stream, (unsigned*)c->tagged, words32);
-        unsigned long long* t = c->tagged;
-        P.tx = t; t += hp.dim;
-        P.th1 = t; t += hp.dim;
-        P.tqkv = t; t += c->maxRowsA;
-        P.tpart = t; t += (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2);
-        P.tmix = t; t += c->maxAd;
-        P.tu = t; t += hp.ffnDim;
-        P.tamax = t;
-    } else {
-        P.tx = P.th1 = P.tqkv = P.tpart = P.tmix = P.tu = P.tamax = nullptr;
+    if (steps > 0) {
+        hipLaunchKernelGGL(k_zero_words, dim3(5), dim3(256), 0, c->stream, c->d_sync, 64 * 20); // barrier words
+        // abort flag; test hook: a flag that starts raised makes every workgroup leave at its first wait
+        hipLaunchKernelGGL(k_set_word, dim3(1), dim3(1), 0, c->stream, P.abortFlag, c->injectAbort > 0 ? 1u : 0u);
+        if (c->injectAbort > 0) c->injectAbort--;
     }
     const bool bf = hp.weightDtype == MLH_DTYPE_BF16;
     if (hd == 64) {

@@ -1087,15 +1087,15 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     if (uni(S.ctl[0])) return;
     const int X = uni(S.ctl[2]), r = uni(S.ctl[3]);
     const int tok = uni(a.tok[0]), pos = uni(a.pos[P.seq]);
-    const unsigned tagBase = *P.tagCounter; // tags never repeat from launch to launch: nothing has to be cleared
+    const unsigned tagBase = *P.tagCounter; // tags do not repeat from launch to launch (the host clears everything before the count wraps)
     if (wave == XWORK) xcd_communicator<WT, HYB>(P, S, tok, pos, tagBase, X, r);
     else xcd_worker<WT, NCH, HYB>(P, S, tok, pos, tagBase, X, r);
 }
 
 // before every launch: abort flag and per-XCD arrival counters
-__global__ void k_xcd_prep(unsigned* abortFlag, unsigned* xcdCount) {
+__global__ void k_xcd_prep(unsigned* abortFlag, unsigned* xcdCount, unsigned startCount) {
     if (threadIdx.x == 0) *abortFlag = 0u;
-    if (threadIdx.x < XCDS) xcdCount[threadIdx.x] = 0u;
+    if (threadIdx.x < XCDS) xcdCount[threadIdx.x] = startCount;
 }
 
 __global__ void k_xcd_zero(unsigned* p, size_t n) {
@@ -1151,10 +1151,14 @@ bool mlh_xcd_supported(const mlh_ctx* c) {
 
 template <typename WT, int NCH, bool HYB>
 static int launch_xcd_as(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
-    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH, HYB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
-    int perCu = 0;
-    MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH, HYB>, XWG, ldsBytes));
-    if (perCu < 1) { c->err = "XCD-rank decode kernel does not fit on a compute unit"; return -1; }
+    if (!c->xcdPrepared) { // once per context (mlh_finalize does it; a context has one model, hence one instantiation)
+        MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH, HYB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+        int perCu = 0;
+        MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH, HYB>, XWG, ldsBytes));
+        if (perCu < 1) { c->err = "XCD-rank decode kernel does not fit on a compute unit"; return -1; }
+        c->xcdPrepared = true;
+    }
+    if (P.steps <= 0) return 0; // preparation only
     // one workgroup per compute unit, all resident at once (the occupancy query says each unit can hold one); waits are bounded
     hipLaunchKernelGGL((k_decode_xcd<WT, NCH, HYB>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
     MLH_CHECK(c, hipGetLastError());
@@ -1165,9 +1169,11 @@ static int launch_xcd(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
     return xcd_hybrid(c) ? launch_xcd_as<WT, NCH, true>(c, P, ldsBytes) : launch_xcd_as<WT, NCH, false>(c, P, ldsBytes);
 }
 
-// Puts the exchange words and the tag counter back to zero (after a launch that gave up a wait).
+// Puts the exchange words and the tag counter back to zero (after a launch that gave up a wait, and before the
+// 32-bit tags would wrap).
 int mlh_xcd_reset(mlh_ctx* c) {
     if (!c->xcdBuf) return 0;
+    c->xcdTagNext = 0;
     const size_t words32 = c->xcdWords * 2;
     hipLaunchKernelGGL(k_xcd_zero, dim3((unsigned)((words32 + 255) / 256)), dim3(256), 0, c->stream, (unsigned*)c->xcdBuf, words32);
     hipLaunchKernelGGL(k_xcd_zero, dim3(1), dim3(64), 0, c->stream, c->d_sync + 64 * 21, (size_t)1);
@@ -1189,18 +1195,9 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.xcdCount = c->d_sync + 64 * 22;
     P.fs = hp.ffnDim / XCDS;
     P.timing = c->d_timing;
-    {
-        static const int dflt[5] = {44, 0, 0, 0, 0};
-        const char* ew = getenv("MLH_XCD_WIDE");
-        P.wide = ew ? atoi(ew) : 1;
-        const char* er = getenv("MLH_XCD_NAP_ROUND");
-        P.napRound = er ? std::max(0, std::min(400, atoi(er))) : 3;
-        static const char* names[5] = {"MLH_XCD_NAP_CROSS", "MLH_XCD_NAP_GATHER", "MLH_XCD_NAP_QKV", "MLH_XCD_NAP_U", "MLH_XCD_NAP_PART"};
-        for (int k = 0; k < 5; k++) {
-            const char* e = getenv(names[k]);
-            P.nap[k] = e ? std::max(0, std::min(400, atoi(e))) : dflt[k];
-        }
-    }
+    P.wide = c->xcdWide;
+    P.napRound = c->xcdNapRound;
+    for (int k = 0; k < 5; k++) P.nap[k] = c->xcdNap[k];
     u64* t = c->xcdBuf;
     P.qkvStride = 4 * XNH * XHD + XQX;
     P.qkvL = t; t += (size_t)XCDS * P.qkvStride;
@@ -1213,7 +1210,20 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.uL = t; t += hp.ffnDim;
     P.amax = t;
     const size_t ldsBytes = xcd_lds_bytes(c);
-    hipLaunchKernelGGL(k_xcd_prep, dim3(1), dim3(64), 0, c->stream, P.abortFlag, P.xcdCount);
+    if (steps > 0) {
+        // Tags are a 32-bit running count of layer passes and a word whose tag matches is taken as fresh: before the
+        // count could wrap (and meet tag 0 of cleared words, or a stale word), everything goes back to zero.
+        const unsigned long long need = (unsigned long long)steps * hp.transformers + 1;
+        if (c->xcdTagNext + need >= 0xFFFFFFFFull) {
+            int rc = mlh_xcd_reset(c);
+            if (rc) return rc;
+        }
+        c->xcdTagNext += need; // (a launch that gives up is followed by mlh_xcd_reset, which puts this back to zero)
+        // test hook: arrival counters that start full make every workgroup give up before it touches anything
+        const unsigned startCount = c->injectAbort > 0 ? (unsigned)XPER : 0u;
+        if (c->injectAbort > 0) c->injectAbort--;
+        hipLaunchKernelGGL(k_xcd_prep, dim3(1), dim3(64), 0, c->stream, P.abortFlag, P.xcdCount, startCount);
+    }
     if (hp.weightDtype == MLH_DTYPE_BF16) {
         switch (hp.dim / 512) { // chunks of 8 values per lane and row
             case 1: return launch_xcd<bf16_t, 1>(c, P, ldsBytes);

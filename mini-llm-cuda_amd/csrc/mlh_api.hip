@@ -33,6 +33,14 @@ extern "C" const char* mlh_kernel_name(int kernel) {
     return (kernel >= 0 && kernel < MLH_K_COUNT) ? kKernelNames[kernel] : "";
 }
 
+int mlh_dev_alloc_bytes(mlh_ctx* c, void** p, size_t bytes) {
+    void* q = nullptr;
+    MLH_CHECK(c, hipMalloc(&q, bytes));
+    c->allocs.push_back(q);
+    *p = q;
+    return 0;
+}
+
 static int fail_create(const std::string& msg) {
     g_create_error = msg;
     return -1;
@@ -201,9 +209,6 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         (rc = dev_alloc(c, &c->pamaxVal, (size_t)c->numCUs)) || (rc = dev_alloc(c, &c->pamaxIdx, (size_t)c->numCUs)) ||
         (rc = dev_alloc(c, &c->kvPart, (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2))))
         return bail(rc);
-    c->taggedWords = (size_t)2 * d + c->maxRowsA + (size_t)hp.attnHeads * c->pagesPerSeq * (hp.headDim + 2) + c->maxAd + F + 2 * (size_t)c->numCUs + 64;
-    if ((rc = dev_alloc(c, &c->tagged, c->taggedWords)))
-        return bail(rc);
     c->xcdWords = mlh_xcd_words(c);
     if ((rc = dev_alloc(c, &c->xcdBuf, c->xcdWords))) return bail(rc);
     if (hipMemset(c->xcdBuf, 0, c->xcdWords * 8) != hipSuccess || hipMemset(c->d_sync, 0, 64 * 24 * 4) != hipSuccess) {
@@ -211,10 +216,18 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         return bail(-2);
     }
     if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1) + 4 * 256))) return bail(rc);
-    c->copyBytes = (size_t)256 << 20;
-    char *cs, *cd;
-    if ((rc = dev_alloc(c, &cs, c->copyBytes)) || (rc = dev_alloc(c, &cd, c->copyBytes))) return bail(rc);
-    c->copySrc = cs; c->copyDst = cd;
+    c->copyBytes = (size_t)256 << 20; // calibration copy of MLH_K_COPY: the two buffers are allocated on its first use
+    {   // tuning knobs of the XCD-rank kernel: read once, here
+        auto knob = [](const char* name, int dflt, int lo, int hi) {
+            const char* e = getenv(name);
+            return e ? std::max(lo, std::min(hi, atoi(e))) : dflt;
+        };
+        c->xcdWide = knob("MLH_XCD_WIDE", 1, 0, 1);
+        c->xcdNapRound = knob("MLH_XCD_NAP_ROUND", 3, 0, 400);
+        static const char* names[5] = {"MLH_XCD_NAP_CROSS", "MLH_XCD_NAP_GATHER", "MLH_XCD_NAP_QKV", "MLH_XCD_NAP_U", "MLH_XCD_NAP_PART"};
+        static const int dflt[5] = {44, 0, 0, 0, 0};
+        for (int k = 0; k < 5; k++) c->xcdNap[k] = knob(names[k], dflt[k], 0, 400);
+    }
 
     std::vector<int> pt((size_t)S * c->pagesPerSeq);
     for (size_t i = 0; i < pt.size(); i++) pt[i] = (int)i;
@@ -376,6 +389,10 @@ extern "C" int mlh_finalize(mlh_ctx* c) {
     if (rc == 0) rc = mlh_build_gemm_operands(c);
     if (rc) return rc;
     MLH_CHECK(c, hipMemcpy(c->d_layers, c->layers.data(), c->layers.size() * sizeof(LayerDev), hipMemcpyHostToDevice));
+    // function attributes and occupancy of the single-launch decode kernels, here and not on every launch
+    c->xcdPrepared = c->persistentPrepared = false;
+    if (mlh_xcd_supported(c) && (rc = mlh_launch_xcd(c, 0))) return rc;
+    if (mlh_persistent_supported(c) && mlh_launch_persistent(c, 0)) c->err.clear(); // a model too wide for it simply does not use it
     MLH_CHECK(c, hipDeviceSynchronize());
     c->finalized = true;
     return 0;
@@ -583,84 +600,21 @@ static bool use_persistent(const mlh_ctx* c, int nseq) {
     return nseq == 1 && c->usePersistent && c->temperature <= 0.f && mlh_persistent_supported(c);
 }
 
-// After the stream has drained: a persistent launch that gave up a bounded wait leaves its flag set.
-static void dump_persistent_timing(mlh_ctx* c) {
-    if (!c->d_timing) return;
-    const int n = 16 * c->hp.transformers;
-    std::vector<unsigned long long> t(n);
-    if (hipMemcpy(t.data(), c->d_timing, (size_t)n * 8, hipMemcpyDeviceToHost) != hipSuccess) return;
-    const char* names[15] = {"A.norm", "A.rows", "A->B sync", "B.mix", "B->C sync", "C.prologue", "C.rows", "C->D sync",
-                                    "D.norm", "D.rows", "D->E sync", "E.load", "E.rows", "E->A sync", "x.load"};
-    double tot[15] = {0};
-    const bool xcd = c->usePersistent == 3 && mlh_xcd_supported(c);
-    for (int l = 0; l < c->hp.transformers; l++)
-        for (int k = 0; k < (xcd ? 5 : 15); k++) tot[k] += (double)(t[l * 16 + k + 1] - t[l * 16 + k]) / 100.0; // 100 MHz clock
-    static const char* tnames[15] = {"x.wait", "A.norm", "A.rows", "B.mix", "C.wait", "C.rows", "h1.wait", "D.norm", "D.rows",
-                                     "u.wait", "E.rows", "-", "-", "-", "-"};
-    static const char* xnames[15] = {"x.exchange", "A+hop", "B+hop", "C+2hops", "D+hop", "-", "-", "-", "-", "-", "-", "-", "-", "-", "-"};
-    if (c->usePersistent == 2) for (int k = 0; k < 15; k++) names[k] = tnames[k];
-    if (xcd) for (int k = 0; k < 15; k++) names[k] = xnames[k];
-    if (xcd) { // skew between workgroups at four points of the last layer pass
-        std::vector<unsigned long long> sk(4 * 256);
-        if (hipMemcpy(sk.data(), c->d_timing + 16 * (c->hp.transformers + 1), sk.size() * 8, hipMemcpyDeviceToHost) == hipSuccess) {
-            {   // per workgroup with a unit on wave 0: wait for the tile, unit, combine
-                std::vector<double> a1, a2, a3;
-                for (int w = 0; w < 256; w++)
-                    if (sk[4 * w] && sk[4 * w + 1]) {
-                        a1.push_back(((double)sk[4 * w + 3] - (double)sk[4 * w + 1]) / 100.0);
-                        a2.push_back(((double)sk[4 * w] - (double)sk[4 * w + 3]) / 100.0);
-                        a3.push_back(((double)sk[4 * w + 2] - (double)sk[4 * w]) / 100.0);
-                    }
-                auto pr = [&](const char* nm, std::vector<double>& v) { std::sort(v.begin(), v.end()); if (!v.empty()) fprintf(stderr, "[xcd unit] %-28s n %zu min %.2f median %.2f max %.2f us\n", nm, v.size(), v[0], v[v.size() / 2], v.back()); };
-                pr("barrier 2 -> tile waited for", a1); pr("tile ready -> unit end", a2); pr("unit end -> combine done", a3);
-            }
-            const char* what[4] = {"attention wave 0 end", "wave 0 unit start", "wave 0 combine done", "wave 0 tile ready"};
-            unsigned long long t0 = ~0ull;
-            for (int w = 0; w < 256; w++) if (sk[4 * w]) t0 = std::min(t0, sk[4 * w]);
-            for (int k = 0; k < 4; k++) {
-                std::vector<double> v;
-                for (int w = 0; w < 256; w++) v.push_back(sk[4 * w + k] ? ((double)sk[4 * w + k] - (double)t0) / 100.0 : -1.0);
-                double perX[8] = {0};
-                std::vector<double> sorted = v;
-                std::sort(sorted.begin(), sorted.end());
-                const size_t first = std::lower_bound(sorted.begin(), sorted.end(), 0.0) - sorted.begin(), cnt = 256 - first;
-                if (!cnt) continue;
-                fprintf(stderr, "[xcd skew] %-20s n %zu min %.2f median %.2f max %.2f us (first 8 workgroups:", what[k], cnt, sorted[first], sorted[first + cnt / 2], sorted[255]);
-                for (int w = 0; w < 8; w++) fprintf(stderr, " %.2f", v[w]);
-                fprintf(stderr, ")\n");
-                (void)perX;
-            }
-        }
-    }
-    if (xcd) { // raw stamps relative to the start of the layer pass: communicator 0-9, worker wave 0 10-14
-        double rel[16] = {0};
-        for (int l = 0; l < c->hp.transformers; l++)
-            for (int k = 0; k < 16; k++) rel[k] += ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 / c->hp.transformers;
-        for (int l = 0; l < c->hp.transformers; l++) {
-            fprintf(stderr, "[xcd layer %2d]", l);
-            for (int k = 0; k < 16; k++) fprintf(stderr, " %d:%.2f", k, t[l * 16 + k] ? ((double)t[l * 16 + k] - (double)t[l * 16]) / 100.0 : -1.0);
-            fprintf(stderr, "\n");
-        }
-        fprintf(stderr, "[xcd stamps, us from layer start] x: partials seen %.2f gathered %.2f | worker A %.2f..%.2f | q,k,v in LDS %.2f | "
-                        "wave 0: units done %.2f combine done %.2f | worker C %.2f..%.2f | h1: partials seen %.2f gathered %.2f | worker D end %.2f | "
-                        "u in LDS %.2f | worker E end %.2f\n",
-                rel[6], rel[1], rel[10], rel[11], rel[2], rel[12], rel[15], rel[13], rel[14], rel[8], rel[4], rel[7], rel[5], rel[9]);
-
-    }
-    fprintf(stderr, "[persistent decode, workgroup 0, last step] mean us per layer:");
-    double sum = 0;
-    for (int k = 0; k < 15; k++) { fprintf(stderr, " %s=%.2f", names[k], tot[k] / c->hp.transformers); sum += tot[k] / c->hp.transformers; }
-    fprintf(stderr, " | layer total %.2f\n", sum);
-}
-
+// After the stream has drained: a single-launch decode that gave up a bounded wait leaves its flag set.  Nothing of
+// the sequence has advanced then (position, token, GDN states and the tag counter are written at the kernel's normal
+// end only), so the caller can run the same steps again another way.
 static int check_persistent_abort(mlh_ctx* c) {
-    dump_persistent_timing(c);
+    if (c->d_timing) mlh_dump_persistent_timing(c);
     unsigned flag = 0;
     MLH_CHECK(c, hipMemcpy(&flag, c->d_sync + 64 * 20, 4, hipMemcpyDeviceToHost));
     if (flag) {
         c->err = flag == 2 ? "XCD-rank decode kernel: the workgroups did not spread evenly over the XCDs"
                            : "persistent decode kernel abandoned a wait (were all workgroups resident?)";
-        if (c->usePersistent == 3 && mlh_xcd_reset(c) == 0) (void)hipStreamSynchronize(c->stream); // tags of the abandoned launch must not be met again
+        if (c->usePersistent == 3 && mlh_xcd_supported(c)) { // tags of the abandoned launch must not be met again
+            int rc = mlh_xcd_reset(c);
+            if (rc) return rc;
+            MLH_CHECK(c, hipStreamSynchronize(c->stream));
+        }
         return -3;
     }
     return 0;
@@ -702,16 +656,30 @@ static int check_decode(mlh_ctx* c, const int32_t* ids, int nseq, int steps) {
     return set_identity_slots(c, nseq);
 }
 
+// The single-launch kernels need every compute unit for themselves.  When one gives up (another process or stream
+// holds units), the call is redone as the kernel sequence and the context stays in that mode: the steps cost more,
+// the results are the same.  mlh_get_persistent shows the mode in effect, mlh_persistent_fallbacks how often it happened.
+static int fall_back_to_kernel_sequence(mlh_ctx* c) {
+    c->persistentFallbacks++;
+    c->usePersistent = 0;
+    return 0;
+}
+
 extern "C" int mlh_decode_loop(mlh_ctx* c, const int32_t* first, int nseq, int steps, int32_t* out) {
     int rc = check_decode(c, first, nseq, steps);
     if (rc) return rc;
     if (!out) { c->err = "null output"; return -1; }
-    MLH_CHECK(c, hipMemcpyAsync(c->d_tok, first, (size_t)nseq * 4, hipMemcpyHostToDevice, c->stream));
-    MLH_CHECK(c, hipMemsetAsync(c->d_stepCounter, 0, 4, c->stream));
-    if ((rc = run_steps(c, nseq, steps))) return rc;
-    MLH_CHECK(c, hipMemcpyAsync(out, c->d_outIds, (size_t)steps * nseq * 4, hipMemcpyDeviceToHost, c->stream));
-    MLH_CHECK(c, hipStreamSynchronize(c->stream));
-    if (use_persistent(c, nseq) && (rc = check_persistent_abort(c))) return rc;
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const bool single = use_persistent(c, nseq);
+        MLH_CHECK(c, hipMemcpyAsync(c->d_tok, first, (size_t)nseq * 4, hipMemcpyHostToDevice, c->stream));
+        MLH_CHECK(c, hipMemsetAsync(c->d_stepCounter, 0, 4, c->stream));
+        if ((rc = run_steps(c, nseq, steps))) return rc;
+        MLH_CHECK(c, hipMemcpyAsync(out, c->d_outIds, (size_t)steps * nseq * 4, hipMemcpyDeviceToHost, c->stream));
+        MLH_CHECK(c, hipStreamSynchronize(c->stream));
+        if (!single || (rc = check_persistent_abort(c)) == 0) break;
+        if (rc != -3) return rc;
+        fall_back_to_kernel_sequence(c); // and once more, as a sequence of kernels
+    }
     for (int s = 0; s < nseq; s++) c->h_len[s] += steps;
     return 0;
 }
@@ -727,19 +695,25 @@ extern "C" int mlh_time_decode(mlh_ctx* c, const int32_t* first, int nseq, int s
     hipEvent_t e0, e1;
     MLH_CHECK(c, hipEventCreate(&e0));
     MLH_CHECK(c, hipEventCreate(&e1));
-    MLH_CHECK(c, hipMemcpyAsync(c->d_tok, first, (size_t)nseq * 4, hipMemcpyHostToDevice, c->stream));
-    MLH_CHECK(c, hipMemsetAsync(c->d_stepCounter, 0, 4, c->stream));
-    MLH_CHECK(c, hipStreamSynchronize(c->stream));
-    MLH_CHECK(c, hipEventRecord(e0, c->stream));
-    rc = run_steps(c, nseq, steps);
-    MLH_CHECK(c, hipEventRecord(e1, c->stream));
-    MLH_CHECK(c, hipEventSynchronize(e1));
     float ms = 0.f;
-    MLH_CHECK(c, hipEventElapsedTime(&ms, e0, e1));
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const bool single = use_persistent(c, nseq);
+        MLH_CHECK(c, hipMemcpyAsync(c->d_tok, first, (size_t)nseq * 4, hipMemcpyHostToDevice, c->stream));
+        MLH_CHECK(c, hipMemsetAsync(c->d_stepCounter, 0, 4, c->stream));
+        MLH_CHECK(c, hipStreamSynchronize(c->stream));
+        MLH_CHECK(c, hipEventRecord(e0, c->stream));
+        rc = run_steps(c, nseq, steps);
+        MLH_CHECK(c, hipEventRecord(e1, c->stream));
+        MLH_CHECK(c, hipEventSynchronize(e1));
+        MLH_CHECK(c, hipEventElapsedTime(&ms, e0, e1));
+        if (rc) break;
+        if (!single || (rc = check_persistent_abort(c)) == 0) break;
+        if (rc != -3) break;
+        fall_back_to_kernel_sequence(c);
+    }
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
     if (rc) return rc;
-    if (use_persistent(c, nseq) && (rc = check_persistent_abort(c))) return rc;
     *totalMs = ms;
     for (int s = 0; s < nseq; s++) c->h_len[s] += steps;
     return 0;
@@ -833,8 +807,26 @@ extern "C" int mlh_set_graph(mlh_ctx* c, int stepsPerGraph) {
 
 extern "C" int mlh_set_persistent(mlh_ctx* c, int enabled) {
     if (!c) return -1;
-    if (enabled < 0 || enabled > 3) { c->err = "persistent mode must be 0..3"; return -1; }
+    if (enabled != 0 && enabled != 1 && enabled != 3) { c->err = "persistent mode must be 0, 1 or 3"; return -1; }
     c->usePersistent = enabled;
+    return 0;
+}
+
+extern "C" int mlh_get_persistent(mlh_ctx* c) { return c ? c->usePersistent : -1; }
+extern "C" int mlh_persistent_fallbacks(mlh_ctx* c) { return c ? c->persistentFallbacks : -1; }
+
+extern "C" int mlh_debug_inject_abort(mlh_ctx* c, int launches) {
+    if (!c || launches < 0) return -1;
+    c->injectAbort = launches;
+    return 0;
+}
+
+extern "C" int mlh_debug_set_xcd_tag(mlh_ctx* c, unsigned tagsUsed) {
+    int rc = check_ready(c);
+    if (rc) return rc;
+    MLH_CHECK(c, hipStreamSynchronize(c->stream));
+    MLH_CHECK(c, hipMemcpy(c->d_sync + 64 * 21, &tagsUsed, 4, hipMemcpyHostToDevice));
+    c->xcdTagNext = tagsUsed;
     return 0;
 }
 

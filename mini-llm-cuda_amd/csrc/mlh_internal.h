@@ -132,12 +132,16 @@ struct mlh_ctx {
     bool coopLaunch = false;
     float temperature = 0.f;       // 0: greedy; > 0: temperature sampling (kernel-sequence and batched paths)
     unsigned long long sampleSeed = 0;
-    int usePersistent = 3;         // 0: kernel sequence; 1: persistent kernel with grid barriers; 2: tagged exchange;
+    int usePersistent = 3;         // 0: kernel sequence; 1: persistent kernel with grid barriers;
                                    // 3: XCD ranks where the model and device allow it, else as 1
+    int persistentFallbacks = 0;   // single-launch decode calls that gave up a wait and were redone as the kernel sequence
+    int injectAbort = 0;           // test hook: the next n single-launch decode launches give up at their start
+    unsigned long long xcdTagNext = 0; // host mirror of the XCD-rank kernel's tag counter (tags used so far)
+    bool xcdPrepared = false;      // function attribute and occupancy of the XCD-rank kernel checked
+    bool persistentPrepared = false;
+    int xcdWide = 1, xcdNapRound = 3, xcdNap[5] = {44, 0, 0, 0, 0}; // tuning knobs, read from the environment once at creation
     unsigned long long* xcdBuf = nullptr; // (value, tag) exchange words of mode 3
     size_t xcdWords = 0;
-    unsigned long long* tagged = nullptr; // (value, tag) exchange words of mode 2
-    size_t taggedWords = 0;
     LayerDev* d_layers = nullptr;  // device copy of `layers`
     unsigned* d_sync = nullptr;    // barrier words + abort flag
     float* pamaxVal = nullptr;     // [numCUs]
@@ -182,6 +186,7 @@ int mlh_launch_one(mlh_ctx* c, int kernel, int layer, int nseq);
 double mlh_kernel_bytes(mlh_ctx* c, int kernel, int layer, int nseq);
 void mlh_fill_args(mlh_ctx* c, StepArgs& a, int nseq, const int* tokPtr);
 int mlh_launch_copy(mlh_ctx* c);
+int mlh_dev_alloc_bytes(mlh_ctx* c, void** p, size_t bytes); // mlh_api.hip: an allocation owned by the context
 int mlh_launch_probs(mlh_ctx* c, int seq);
 int mlh_init_kernels(mlh_ctx* c);
 
@@ -218,6 +223,10 @@ int mlh_launch_softmax_rows(mlh_ctx* c, const float* logits, float* probs, const
 // kernels_persistent.hip
 bool mlh_persistent_supported(const mlh_ctx* c);
 int mlh_launch_persistent(mlh_ctx* c, int steps);
+
+// measure_timing.hip: decodes and prints the phase clock stamps of the single-launch decode kernels
+// (collected only when MLH_PERSIST_TIMING is set at context creation)
+void mlh_dump_persistent_timing(mlh_ctx* c);
 
 // kernels_xcd.hip
 size_t mlh_xcd_words(const mlh_ctx* c);

@@ -49,7 +49,7 @@ def make(pkg, orc, hp, seed, bf16=False):
     return model, dev, w
 
 
-@pytest.mark.parametrize("persistent", [3, 2, 1, 0], ids=["xcd", "tagged", "persistent", "kernels"])
+@pytest.mark.parametrize("persistent", [3, 1, 0], ids=["xcd", "persistent", "kernels"])
 @pytest.mark.parametrize("kind,plen,steps", [("attn", 16, 40), ("attn_flags", 16, 40), ("hybrid", 16, 40),
                                              ("hybrid_flags", 16, 40), ("hd128", 16, 40), ("attn_long", 300, 12)])
 def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
@@ -74,7 +74,7 @@ def test_stepwise_logits_and_ids(pkg, orc, kind, plen, steps, persistent):
     dev.close()
 
 
-@pytest.mark.parametrize("persistent", [3, 2, 1, 0], ids=["xcd", "tagged", "persistent", "kernels"])
+@pytest.mark.parametrize("persistent", [3, 1, 0], ids=["xcd", "persistent", "kernels"])
 def test_config1_golden_horizon(pkg, orc, persistent):
     """Configuration 1 at full size: 16-token prompt, 128 greedy steps on the device loop, checked
     against the oracle and against the committed golden ids."""
@@ -150,6 +150,82 @@ def test_xcd_rank_kernel_shapes(pkg, orc, case):
             assert worst < 1e-4
         tok = int(out[-1])
         assert tok == nxt or abs(float(lg[tok]) - float(lg[nxt])) < (2e-2 if bf16 else GAP_TOL)
+    dev.close()
+
+
+def _hybrid12(pkg):
+    hp = pkg.config(3, dim=768, attnHeads=12, gdnHeads=12, headDim=64, ffnDim=512, transformers=4, vocabSize=1024, maxL=200)
+    pkg.set_layer_pattern(hp, 3)
+    return hp
+
+
+@pytest.mark.parametrize("mode", [3, 1], ids=["xcd", "persistent"])
+def test_single_launch_gives_up_and_falls_back(pkg, orc, mode):
+    """A single-launch decode that finds its wait given up (forced from the host, so every kernel still exits
+    normally) advances nothing; the call redoes its steps as the kernel sequence, the context stays at mode 0,
+    and everything decoded before, during and after agrees with the oracle -- also after switching back."""
+    hp = _hybrid12(pkg) if mode == 3 else small_cfg(pkg, "hybrid")
+    model, dev, w = make(pkg, orc, hp, seed=31)
+    dev.set_persistent(mode)
+    assert dev.xcd_decode_supported() == (mode == 3)
+    prompt = pkg.random_tokens(31, 0, hp.vocabSize, 40)
+    dev.prefill(0, prompt)
+    dec = orc.Decoder(w, "f64")
+    for t in prompt:
+        nxt, lg = dec.step(int(t))
+    tok = dev.greedy_token(0)
+
+    def run(n):
+        nonlocal tok, nxt, lg
+        out = dev.decode_loop([tok], n)[:, 0]
+        for t in [tok] + [int(v) for v in out[:-1]]:
+            nxt, lg = dec.step(t)
+        assert_logits_close(dev.logits(0), lg, FP32_RTOL, f"mode {mode}")
+        tok = int(out[-1])
+        assert tok == nxt or abs(float(lg[tok]) - float(lg[nxt])) < GAP_TOL
+
+    run(3)
+    assert dev.get_persistent() == mode and dev.persistent_fallbacks() == 0
+    dev.debug_inject_abort(1)
+    run(5)                                  # gives up, is redone as the kernel sequence
+    assert dev.get_persistent() == 0 and dev.persistent_fallbacks() == 1
+    assert dev.seq_len(0) == 40 + 8
+    run(2)                                  # stays on the kernel sequence
+    assert dev.persistent_fallbacks() == 1
+    dev.set_persistent(mode)                # and the single launch works again afterwards (exchange words were cleared)
+    run(4)
+    assert dev.get_persistent() == mode and dev.persistent_fallbacks() == 1
+    # the timed entry point takes the same way out
+    dev.debug_inject_abort(1)
+    ms = dev.time_decode([tok], 2)
+    assert ms > 0 and dev.get_persistent() == 0 and dev.persistent_fallbacks() == 2 and dev.seq_len(0) == 40 + 16
+    dev.close()
+
+
+def test_xcd_tags_are_cleared_before_they_wrap(pkg, orc):
+    """The XCD-rank kernel tags every exchanged word with a 32-bit running count of layer passes.  With the count
+    set just below 2^32 the next launch must start from cleared words and count 0 instead of wrapping into tags
+    that are still in the buffers; the decode stays on the single launch and agrees with the oracle."""
+    hp = _hybrid12(pkg)
+    model, dev, w = make(pkg, orc, hp, seed=32)
+    dev.set_persistent(3)
+    assert dev.xcd_decode_supported()
+    prompt = pkg.random_tokens(32, 0, hp.vocabSize, 30)
+    dev.prefill(0, prompt)
+    dec = orc.Decoder(w, "f64")
+    for t in prompt:
+        nxt, lg = dec.step(int(t))
+    tok = dev.greedy_token(0)
+    for n, seed_tag in ((4, None), (6, 0xFFFFFFFF - 9), (3, None), (5, 0xFFFFFFFF - 4 * 5 - 2), (2, None)):
+        if seed_tag is not None:
+            dev.debug_set_xcd_tag(seed_tag)   # 6 steps x 4 layers + 1 tags do not fit below 2^32 any more
+        out = dev.decode_loop([tok], n)[:, 0]
+        for t in [tok] + [int(v) for v in out[:-1]]:
+            nxt, lg = dec.step(t)
+        assert_logits_close(dev.logits(0), lg, FP32_RTOL, f"launch of {n}")
+        tok = int(out[-1])
+        assert tok == nxt or abs(float(lg[tok]) - float(lg[nxt])) < GAP_TOL
+    assert dev.get_persistent() == 3 and dev.persistent_fallbacks() == 0
     dev.close()
 
 
