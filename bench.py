@@ -261,9 +261,48 @@ def gemm_leg(m, iters=3, reps=1):
     b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
     runs = [m.selftest_gemm(a, b, None, f16=True, iters=iters)[1] for _ in range(reps)]
     us = stats(runs)["median"]
-    tf = 2.0 * M * 2 * hp.ffnDim * hp.dim / us / 1e6
-    return {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "avg_us": us, "avg_us_stats": stats(runs), "TFLOPs": tf,
-            "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
+    flop = 2.0 * M * 2 * hp.ffnDim * hp.dim
+    tf = flop / us / 1e6
+    out = {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "avg_us": us, "avg_us_stats": stats(runs), "TFLOPs": tf,
+           "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
+    if reps > 1:
+        # Two yardsticks on the same box in the same run, neither on the product path: the same kernel on all-zero
+        # operands (no switching activity: what the code alone allows, without the part's power management), and the
+        # vendor library's GEMM (torch.matmul -> hipBLASLt) on the same shape, type and data distribution.
+        z = np.zeros_like(a), np.zeros_like(b)
+        uz = stats([m.selftest_gemm(z[0], z[1], None, f16=True, iters=iters)[1] for _ in range(3)])["median"]
+        out["same_kernel_zero_operands"] = {"avg_us": uz, "TFLOPs": flop / uz / 1e6}
+        try:
+            out["vendor_library_yardstick"] = vendor_gemm(a, b, iters, reps, flop)
+            out["ratio_to_vendor_library"] = out["vendor_library_yardstick"]["avg_us"] / us
+        except Exception as e:  # a yardstick, never required
+            out["vendor_library_yardstick"] = {"failed": repr(e)}
+    return out
+
+
+def vendor_gemm(a, b, iters, reps, flop):
+    """torch.matmul (the vendor BLAS library) on the GEMM leg's operands: a yardstick beside the hand-written kernel."""
+    import torch
+    ta = torch.from_numpy(a).to("cuda:0", dtype=torch.float16)
+    tb = torch.from_numpy(b).to("cuda:0", dtype=torch.float16)
+    res = {}
+    for label, (x, y) in (("normal_data", (ta, tb)), ("zero_operands", (torch.zeros_like(ta), torch.zeros_like(tb)))):
+        for _ in range(3):
+            x @ y.t()
+        torch.cuda.synchronize()
+        runs = []
+        for _ in range(reps if label == "normal_data" else 3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                x @ y.t()
+            e1.record()
+            torch.cuda.synchronize()
+            runs.append(e0.elapsed_time(e1) * 1e3 / iters)
+        res[label] = {"avg_us": stats(runs)["median"], "TFLOPs": flop / stats(runs)["median"] / 1e6}
+    return {"what": "torch.matmul, fp16, same shape and N(0,1) data, back-to-back launches", "avg_us": res["normal_data"]["avg_us"],
+            "TFLOPs": res["normal_data"]["TFLOPs"], "frac_of_bf16_peak": res["normal_data"]["TFLOPs"] * 1e12 / MFMA_BF16_PEAK,
+            "zero_operands": res["zero_operands"]}
 
 
 def timed_decode(dev, prompt, K, W, persistent, maxL):

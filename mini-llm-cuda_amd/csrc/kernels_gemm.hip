@@ -41,25 +41,28 @@ template <> struct GemmTraits<float> {
         c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
     }
     static __device__ __forceinline__ void put(float* p, float v) { *p = v; }
+    static __device__ __forceinline__ uint32_t bits(float v) { return __float_as_uint(v); }
 };
 template <> struct GemmTraits<bf16_t> {
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x16& c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
-    static __device__ __forceinline__ void put(bf16_t* p, float v) {
-        uint32_t u = __float_as_uint(v);
-        *p = (bf16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+    static __device__ __forceinline__ uint32_t bits(float v) {
+        const uint32_t u = __float_as_uint(v);
+        return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
     }
+    static __device__ __forceinline__ void put(bf16_t* p, float v) { *p = (bf16_t)bits(v); }
 };
 
 template <> struct GemmTraits<f16_t> {
     static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x16& c) {
         c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
     }
-    static __device__ __forceinline__ void put(f16_t* p, float v) { // saturating: an overflow must not become inf
+    static __device__ __forceinline__ uint32_t bits(float v) { // saturating: an overflow must not become inf
         const _Float16 h = (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f);
-        p->bits = __builtin_bit_cast(uint16_t, h);
+        return __builtin_bit_cast(uint16_t, h);
     }
+    static __device__ __forceinline__ void put(f16_t* p, float v) { p->bits = (uint16_t)bits(v); }
 };
 
 // Workgroups that run at the same time on one XCD (ids congruent mod 8 go to the same XCD and share its
@@ -282,38 +285,115 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
 #pragma unroll
             for (int bm = 0; bm < 2; bm++)
 #pragma unroll
-                for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
+                for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fb[jj & 1][bn], fa[jj & 1][bm], acc[bm][bn]);
             __builtin_amdgcn_sched_barrier(0);
             if (jj < 3) frags(jj + 1, (jj + 1) & 1);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int bm = 2; bm < 4; bm++)
 #pragma unroll
-                for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fa[jj & 1][bm], fb[jj & 1][bn], acc[bm][bn]);
+                for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fb[jj & 1][bn], fa[jj & 1][bm], acc[bm][bn]);
         }
         __builtin_amdgcn_sched_barrier(0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // slice s+1 has landed
         __syncthreads();                                  // ... for every wave, and everyone is done with slice s
     }
 
+    // Epilogue.  The product was formed transposed (weights as the first MFMA operand), so lane (lrow, half) holds, for
+    // every 32 x 32 block, row lrow of C and the columns 8 g + 4 half + 0..3 in acc[..][4 g + 0..3]: the gate and up value
+    // of a SwiGLU pair sit in one lane.  A block then goes through a patch of LDS of the wave's own (the stages are free:
+    // the loop ended with a barrier) and is read back with several lanes per row, so that a store instruction writes whole
+    // rows of 64 or 128 bytes instead of 64 scattered pieces; the residual is read the same way.
+    {
+        constexpr int EP = 144;                                  // patch row pitch in bytes (16-byte aligned, rows 4 banks apart)
+        typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+        typedef __attribute__((address_space(3))) uint32_t lds_u32;
+        typedef __attribute__((address_space(3))) float lds_f32;
+        const unsigned patch = (unsigned)(unsigned long long)gsm + wave * (2 * 32 * EP);
+        const int mW = m0 + wm * 128, nW = n0 + wn * 32 * GB_BN;
+        if (EPI == GEMM_EPI_PLAIN) {
+            const bool vec = ((ldc & 3) == 0) && (!R || (ldr & 3) == 0) && (((unsigned long long)Cv & 15) == 0) && (((unsigned long long)R & 15) == 0);
+            const unsigned wr = patch + lrow * EP + half * 16, rd = patch + (lane >> 3) * EP + (lane & 7) * 16;
+            int blk = 0;
 #pragma unroll
-    for (int bm = 0; bm < 4; bm++)
+            for (int bm = 0; bm < 4; bm++)
 #pragma unroll
-        for (int bn = 0; bn < GB_BN; bn++) {
-            const int col = n0 + wn * 32 * GB_BN + bn * 32 + lrow;
+                for (int bn = 0; bn < GB_BN; bn++, blk++) {
+                    const unsigned pb = (blk & 1) * (32 * EP); // two patches in turn: the next block's writes do not wait for this one's reads
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int row = m0 + wm * 128 + bm * 32 + 8 * (i >> 2) + 4 * half + (i & 3);
-                float v = acc[bm][bn][i] * alpha;
-                if (EPI == GEMM_EPI_SWIGLU) {
-                    const float o = __shfl_xor(v, 1, 64);
-                    if (!(lane & 1) && row < M && col < N) GemmTraits<T>::put((T*)Cv + (size_t)row * ldc + (col >> 1), (v / (1.0f + expf(-v))) * o);
-                } else if (row < M && col < N) {
-                    if (R) v += R[(size_t)row * ldr + col];
-                    ((float*)Cv)[(size_t)row * ldc + col] = v;
+                    for (int g = 0; g < 4; g++) {
+                        f32x4 v;
+                        v.x = acc[bm][bn][4 * g] * alpha; v.y = acc[bm][bn][4 * g + 1] * alpha; v.z = acc[bm][bn][4 * g + 2] * alpha; v.w = acc[bm][bn][4 * g + 3] * alpha;
+                        *(lds_f32x4*)(wr + pb + g * 32) = v;
+                    }
+                    const int rowb = mW + bm * 32 + (lane >> 3), col = nW + bn * 32 + (lane & 7) * 4;
+                    f32x4 v[4];
+#pragma unroll
+                    for (int k = 0; k < 4; k++) v[k] = *(const lds_f32x4*)(rd + pb + k * 8 * EP);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const int row = rowb + 8 * k;
+                        if (row >= M || col >= N) continue;
+                        float* cp = (float*)Cv + (size_t)row * ldc + col;
+                        if (vec && col + 3 < N) {
+                            if (R) v[k] += *reinterpret_cast<const f32x4*>(R + (size_t)row * ldr + col);
+                            *reinterpret_cast<f32x4*>(cp) = v[k];
+                        } else {
+                            const float* rp = R ? R + (size_t)row * ldr + col : nullptr;
+                            cp[0] = v[k].x + (rp ? rp[0] : 0.f);
+                            if (col + 1 < N) cp[1] = v[k].y + (rp ? rp[1] : 0.f);
+                            if (col + 2 < N) cp[2] = v[k].z + (rp ? rp[2] : 0.f);
+                            if (col + 3 < N) cp[3] = v[k].w + (rp ? rp[3] : 0.f);
+                        }
+                    }
+                }
+        } else { // SwiGLU: columns 2 j, 2 j + 1 of the product are gate and up of unit j; U[m, j] = silu(gate) * up in the operand type
+            constexpr int ES = (int)sizeof(T);                   // 2 or 4
+            constexpr int OUTW = 16 * GB_BN;                     // units per row of the wave's tile
+            constexpr int LPR = OUTW * ES / 16;                  // lanes per row when reading back 16 bytes each
+            constexpr int RPP = 64 / LPR;                        // rows per pass
+            const bool vec = (((size_t)ldc * ES) & 15) == 0 && (((unsigned long long)Cv & 15) == 0);
+            const int jW = nW >> 1, NU = N >> 1;
+#pragma unroll
+            for (int bm = 0; bm < 4; bm++) {
+                const unsigned pb = (bm & 1) * (32 * EP);
+#pragma unroll
+                for (int bn = 0; bn < GB_BN; bn++)
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float g0 = acc[bm][bn][4 * g] * alpha, u0 = acc[bm][bn][4 * g + 1] * alpha;
+                        const float g1 = acc[bm][bn][4 * g + 2] * alpha, u1 = acc[bm][bn][4 * g + 3] * alpha;
+                        const float o0 = (g0 / (1.0f + expf(-g0))) * u0, o1 = (g1 / (1.0f + expf(-g1))) * u1;
+                        const unsigned at = patch + pb + lrow * EP + (bn * 16 + 4 * g + 2 * half) * ES;
+                        if (ES == 2) {
+                            *(lds_u32*)at = GemmTraits<T>::bits(o0) | (GemmTraits<T>::bits(o1) << 16);
+                        } else {
+                            *(lds_f32*)at = o0;
+                            *(lds_f32*)(at + 4) = o1;
+                        }
+                    }
+#pragma unroll
+                for (int k = 0; k < 32 / RPP; k++) {
+                    const int rl = (lane / LPR) + RPP * k, piece = lane % LPR;
+                    const f32x4 v = *(const lds_f32x4*)(patch + pb + rl * EP + piece * 16);
+                    const int row = mW + bm * 32 + rl, j = jW + piece * (16 / ES);
+                    if (row >= M || j >= NU) continue;
+                    T* up = (T*)Cv + (size_t)row * ldc + j;
+                    if (vec && j + 16 / ES - 1 < NU) {
+                        *reinterpret_cast<f32x4*>(up) = v;
+                    } else {
+                        const uint32_t w[4] = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+#pragma unroll
+                        for (int e = 0; e < 16 / ES; e++)
+                            if (j + e < NU) {
+                                if (ES == 2) reinterpret_cast<uint16_t*>(up)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+                                else reinterpret_cast<uint32_t*>(up)[e] = w[e];
+                            }
+                    }
                 }
             }
         }
+    }
 }
 
 template <typename T>
