@@ -73,7 +73,7 @@ __device__ __forceinline__ void gemm_tile_of(int id, int tilesM, int tilesN, int
     const int total = tilesM * tilesN;
     const int per = (total + 7) / 8;
     int t = (id & 7) * per + (id >> 3);
-    if (t >= total) { tm = -1; tn = -1; return; }
+    if ((id >> 3) >= per || t >= total) { tm = -1; tn = -1; return; } // (ids past an XCD's share would walk into the next XCD's)
     const int panel = t / (4 * tilesM);
     const int pw = min(4, tilesN - 4 * panel);
     const int r = t - panel * 4 * tilesM;
@@ -200,36 +200,42 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
     extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 2, wn = wave & 3;
-    int tm, tn;
-    gemm_tile_of(blockIdx.x, tilesM, tilesN, tm, tn);
+    // A workgroup walks the tiles id, id + gridDim.x, ... (one workgroup per compute unit): the first slice of the next
+    // tile is fetched during the last slice of the current one and the epilogue's stores drain under the next tile's
+    // first slices, so a tile boundary costs the epilogue's issue time, not a kernel launch, a cold start and a drain.
+    int id = blockIdx.x, tm, tn;
+    gemm_tile_of(id, tilesM, tilesN, tm, tn);
     if (tm < 0) return;
-    const int m0 = tm * GB_T, n0 = tn * GB_T;
     const int nslices = (int)(((size_t)K * sizeof(T)) / GKB);
     const size_t ldaB = (size_t)lda * sizeof(T), ldbB = (size_t)ldb * sizeof(T);
 
     // A loading wave fills 64 rows of A and of B, eight rows per load instruction.  A load's address is
     // a scalar base (the tile's first row, advanced by one slice per trip on the scalar unit) plus a 32-bit lane offset
-    // that never changes, and its LDS target is scalar too: issuing a slice's loads takes no vector-ALU instruction,
-    // so it does not queue behind the MFMAs of the other wave on the SIMD.
+    // that changes only from tile to tile, and its LDS target is scalar too: issuing a slice's loads takes no vector-ALU
+    // instruction, so it does not queue behind the MFMAs of the other wave on the SIMD.
     // Only the first wave of every SIMD (waves 0..3) loads, for its own rows and for those of the SIMD's second wave:
     // the load path takes an instruction every ~50 ns per SIMD and a wave starts its MFMAs only when its loads are
     // out, so the second wave multiplies while the first one feeds the load path.  (Spreading the loads between the
     // MFMAs instead, by quarters or one per MFMA pair, measured 5-9 % slower.)
     unsigned goffA[8], goffB[8];
-#pragma unroll
-    for (int q = 0; q < 8; q++) {
-        const int r = (wave & 3) * 64 + q * 8 + (lane >> 3);
-        const int pc = (lane & 7) ^ ((r >> 1) & 7);
-        goffA[q] = (unsigned)((size_t)(min(m0 + r, M - 1) - m0) * ldaB) + pc * 16; // rows past the end: the last row again
-        goffB[q] = (unsigned)((size_t)(min(n0 + r, N - 1) - n0) * ldbB) + pc * 16;
-    }
     auto uniform_base = [](const void* p) { // wave-uniform pointer into global memory, kept in scalar registers
         unsigned long long v = (unsigned long long)p;
         asm("" : "+s"(v));
         return (const unsigned char*)(__attribute__((address_space(1))) const unsigned char*)v;
     };
-    const unsigned char* baseA = uniform_base(reinterpret_cast<const unsigned char*>(A) + (size_t)m0 * ldaB);
-    const unsigned char* baseB = uniform_base(reinterpret_cast<const unsigned char*>(B) + (size_t)n0 * ldbB);
+    const unsigned char *baseA, *baseB;
+    auto aim = [&](int tm_, int tn_) { // lane offsets and scalar bases of tile (tm_, tn_)
+        const int m0_ = tm_ * GB_T, n0_ = tn_ * GB_T;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int r = (wave & 3) * 64 + q * 8 + (lane >> 3);
+            const int pc = (lane & 7) ^ ((r >> 1) & 7);
+            goffA[q] = (unsigned)((size_t)(min(m0_ + r, M - 1) - m0_) * ldaB) + pc * 16; // rows past the end: the last row again
+            goffB[q] = (unsigned)((size_t)(min(n0_ + r, N - 1) - n0_) * ldbB) + pc * 16;
+        }
+        baseA = uniform_base(reinterpret_cast<const unsigned char*>(A) + (size_t)m0_ * ldaB);
+        baseB = uniform_base(reinterpret_cast<const unsigned char*>(B) + (size_t)n0_ * ldbB);
+    };
     // (written as the instruction itself: through the builtin the compiler either re-forms 64-bit lane addresses or
     // copies the offsets, one vector-ALU instruction per load either way)
     auto dma16 = [](unsigned long long sbase, unsigned laneOff, unsigned ldsAddr) {
@@ -247,22 +253,28 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
         }
     };
 
-    f32x16 acc[4][GB_BN];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
-#pragma unroll
-        for (int j = 0; j < GB_BN; j++) acc[i][j] = (f32x16)(0.f);
-
     const int half = lane >> 5, lrow = lane & 31;
     // row offsets and swizzle keys of this lane's operand rows ((row >> 1) & 7 does not depend on the 32-row block)
     const int keyA = ((wm * 128 + lrow) >> 1) & 7, keyB = ((wn * 32 * GB_BN + lrow) >> 1) & 7;
     const int offA = (wm * 128 + lrow) * GKB, offB = GB_T * GKB + (wn * 32 * GB_BN + lrow) * GKB;
 
+    aim(tm, tn);
     issue(0, 0);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    for (int s = 0; s < nslices; s++) {
-        const int stage = s & 1;
+    int gs = 0; // slices consumed so far, over all tiles: slice gs sits in stage gs & 1
+  for (;;) {
+    const int m0 = tm * GB_T, n0 = tn * GB_T;
+    int tmN, tnN;
+    gemm_tile_of(id + (int)gridDim.x, tilesM, tilesN, tmN, tnN);
+    const bool more = tmN >= 0;
+    f32x16 acc[4][GB_BN];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < GB_BN; j++) acc[i][j] = (f32x16)(0.f);
+    for (int s = 0; s < nslices; s++, gs++) {
+        const int stage = gs & 1;
         const unsigned char* base = gsm + stage * GB_STAGE;
         // operand fragments one 16-wide step ahead of the MFMAs that use them
         u32x4 fa[2][4], fb[2][GB_BN];
@@ -276,6 +288,7 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
         frags(0, 0); // before the loads: the first operands cross the LDS latency while the loads go out
         __builtin_amdgcn_sched_barrier(0);
         if (s + 1 < nslices) issue(s + 1, stage ^ 1);
+        else if (more) { aim(tmN, tnN); issue(0, stage ^ 1); } // the tile's own slices are all out: the next tile's first one
 #pragma unroll
         for (int jj = 0; jj < 4; jj++) {
             // the reads of step jj+1 go out in the middle of step jj's MFMAs: early enough to have landed when
@@ -295,9 +308,10 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
                 for (int bn = 0; bn < GB_BN; bn++) GemmTraits<T>::mma(fb[jj & 1][bn], fa[jj & 1][bm], acc[bm][bn]);
         }
         __builtin_amdgcn_sched_barrier(0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // slice s+1 has landed
-        __syncthreads();                                  // ... for every wave, and everyone is done with slice s
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the slice after this one has landed
+        __syncthreads();                                  // ... for every wave, and everyone is done with this one
     }
+    unsigned char* const freeStage = gsm + ((gs - 1) & 1) * GB_STAGE; // the stage consumed last: the epilogue's patches live there
 
     // Epilogue.  The product was formed transposed (weights as the first MFMA operand), so lane (lrow, half) holds, for
     // every 32 x 32 block, row lrow of C and the columns 8 g + 4 half + 0..3 in acc[..][4 g + 0..3]: the gate and up value
@@ -309,17 +323,16 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
         typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
         typedef __attribute__((address_space(3))) uint32_t lds_u32;
         typedef __attribute__((address_space(3))) float lds_f32;
-        const unsigned patch = (unsigned)(unsigned long long)gsm + wave * (2 * 32 * EP);
+        const unsigned patch = (unsigned)(unsigned long long)freeStage + wave * (32 * EP); // 8 x 4.5 KB inside the 64 KB stage
         const int mW = m0 + wm * 128, nW = n0 + wn * 32 * GB_BN;
         if (EPI == GEMM_EPI_PLAIN) {
             const bool vec = ((ldc & 3) == 0) && (!R || (ldr & 3) == 0) && (((unsigned long long)Cv & 15) == 0) && (((unsigned long long)R & 15) == 0);
             const unsigned wr = patch + lrow * EP + half * 16, rd = patch + (lane >> 3) * EP + (lane & 7) * 16;
-            int blk = 0;
 #pragma unroll
             for (int bm = 0; bm < 4; bm++)
 #pragma unroll
-                for (int bn = 0; bn < GB_BN; bn++, blk++) {
-                    const unsigned pb = (blk & 1) * (32 * EP); // two patches in turn: the next block's writes do not wait for this one's reads
+                for (int bn = 0; bn < GB_BN; bn++) {
+                    const unsigned pb = 0;
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         f32x4 v;
@@ -356,7 +369,7 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
             const int jW = nW >> 1, NU = N >> 1;
 #pragma unroll
             for (int bm = 0; bm < 4; bm++) {
-                const unsigned pb = (bm & 1) * (32 * EP);
+                const unsigned pb = 0;
 #pragma unroll
                 for (int bn = 0; bn < GB_BN; bn++)
 #pragma unroll
@@ -394,13 +407,24 @@ __global__ void __launch_bounds__(GB_THREADS) k_gemm_tn_big(const T* __restrict_
             }
         }
     }
+    if (!more) break;
+    __syncthreads(); // every wave is done with its patch: the stage may be fetched into again
+    id += (int)gridDim.x; tm = tmN; tn = tnN;
+  }
 }
 
 template <typename T>
 static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                                   const float* R, int ldr, int M, int N, int K, float alpha) {
     const int tilesM = (M + GB_T - 1) / GB_T, tilesN = (N + GB_T - 1) / GB_T;
-    const unsigned grid = (unsigned)(((tilesM * tilesN + 7) / 8) * 8);
+    static int numCUs = 0;
+    if (!numCUs) {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipErrorInvalidDevice;
+        numCUs = std::max(8, (prop.multiProcessorCount / 8) * 8);
+    }
+    const unsigned grid = (unsigned)std::min(numCUs, ((tilesM * tilesN + 7) / 8) * 8); // one workgroup per compute unit walks its tiles
     const size_t lds = 2 * GB_STAGE;
     static bool attr = false;
     if (!attr) {
