@@ -82,23 +82,55 @@ __global__ void k_pf_embed(PfArgs P) {
     P.X[(size_t)row * P.a.dim + i] = getw<WT>((const WT*)P.a.E + (size_t)P.ids[row] * P.a.dim + i);
 }
 
-// inference.cu:24-50 + 83-95, one wave per row (d is a multiple of 8 on this path: 16-byte loads)
+// inference.cu:24-50 + 83-95, one wave per row (d is a multiple of 8 on this path: 16-byte loads).  Rows of up to
+// 4096 elements stay in registers between the sum of squares and the scaling (one pass over memory), and a lane's
+// four results leave as one store.
+template <typename AT> __device__ __forceinline__ void put4(AT* o, float a, float b, float c, float d);
+template <> __device__ __forceinline__ void put4<float>(float* o, float a, float b, float c, float d) {
+    f32x4 v; v.x = a; v.y = b; v.z = c; v.w = d;
+    *reinterpret_cast<f32x4*>(o) = v;
+}
+template <> __device__ __forceinline__ void put4<bf16_t>(bf16_t* o, float a, float b, float c, float d) {
+    put<bf16_t>(o, a); put<bf16_t>(o + 1, b); put<bf16_t>(o + 2, c); put<bf16_t>(o + 3, d);
+}
+template <> __device__ __forceinline__ void put4<f16_t>(f16_t* o, float a, float b, float c, float d) { // saturating like put<f16_t>
+    auto h = [](float v) { return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f)); };
+    uint2 w;
+    w.x = h(a) | (h(b) << 16); w.y = h(c) | (h(d) << 16);
+    *reinterpret_cast<uint2*>(o) = w;
+}
+
 template <typename AT>
 __global__ void __launch_bounds__(PWG) k_pf_rmsnorm(const float* __restrict__ X, const float* __restrict__ gamma, AT* out, int n, int d) {
     const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (row >= n) return;
     const float* x = X + (size_t)row * d;
+    constexpr int KEEP = 16; // 16-byte pieces a lane keeps: rows of up to 64 * 4 * 16 = 4096 elements
+    f32x4 keep[KEEP];
     float s = 0.f;
-    for (int i = lane * 4; i < d; i += 256) {
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) {
+        const int i = lane * 4 + k * 256;
+        keep[k] = i < d ? *reinterpret_cast<const f32x4*>(x + i) : (f32x4)(0.f);
+        s = fmaf(keep[k].x, keep[k].x, s); s = fmaf(keep[k].y, keep[k].y, s); s = fmaf(keep[k].z, keep[k].z, s); s = fmaf(keep[k].w, keep[k].w, s);
+    }
+    for (int i = lane * 4 + KEEP * 256; i < d; i += 256) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(x + i);
         s = fmaf(v.x, v.x, s); s = fmaf(v.y, v.y, s); s = fmaf(v.z, v.z, s); s = fmaf(v.w, v.w, s);
     }
     s = pf_wave_sum(s);
     const float r = sqrtf(s / (float)d + 1e-8f);
-    for (int i = lane * 4; i < d; i += 256) {
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) {
+        const int i = lane * 4 + k * 256;
+        if (i < d) {
+            const f32x4 v = keep[k], g = *reinterpret_cast<const f32x4*>(gamma + i);
+            put4<AT>(out + (size_t)row * d + i, g.x * (v.x / r), g.y * (v.y / r), g.z * (v.z / r), g.w * (v.w / r));
+        }
+    }
+    for (int i = lane * 4 + KEEP * 256; i < d; i += 256) {
         const f32x4 v = *reinterpret_cast<const f32x4*>(x + i), g = *reinterpret_cast<const f32x4*>(gamma + i);
-        AT* o = out + (size_t)row * d + i;
-        put<AT>(o, g.x * (v.x / r)); put<AT>(o + 1, g.y * (v.y / r)); put<AT>(o + 2, g.z * (v.z / r)); put<AT>(o + 3, g.w * (v.w / r));
+        put4<AT>(out + (size_t)row * d + i, g.x * (v.x / r), g.y * (v.y / r), g.z * (v.z / r), g.w * (v.w / r));
     }
 }
 
