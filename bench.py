@@ -263,8 +263,22 @@ def gemm_leg(m, iters=3, reps=1):
     us = stats(runs)["median"]
     flop = 2.0 * M * 2 * hp.ffnDim * hp.dim
     tf = flop / us / 1e6
-    out = {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "avg_us": us, "avg_us_stats": stats(runs), "TFLOPs": tf,
-           "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
+    out = {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "epilogue": "plain, fp32 output", "avg_us": us, "avg_us_stats": stats(runs),
+           "TFLOPs": tf, "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
+    if reps > 1:  # the same product as the prefill pass itself runs it: SiLU(gate) * up in the epilogue, half output
+        sruns = [m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)[1] for _ in range(reps)]
+        su = stats(sruns)["median"]
+        out["as_in_the_pass_swiglu_epilogue"] = {"avg_us": su, "avg_us_stats": stats(sruns), "TFLOPs": flop / su / 1e6,
+                                                 "frac_of_bf16_peak": flop / su / 1e6 * 1e12 / MFMA_BF16_PEAK}
+        # One launch at a time with the device idle in between: in the prefill pass a GEMM is followed by lighter kernels,
+        # not by nine more GEMMs, and the part's clock under real operand data depends on how long the load has lasted.
+        singles = []
+        for _ in range(7):
+            time.sleep(0.05)
+            singles.append(m.selftest_gemm(a, b, None, f16=True, iters=1, swiglu=True)[1])
+        s1 = stats(singles)["median"]
+        out["single_launch_swiglu_epilogue"] = {"avg_us": s1, "avg_us_stats": stats(singles), "TFLOPs": flop / s1 / 1e6,
+                                                "frac_of_bf16_peak": flop / s1 / 1e6 * 1e12 / MFMA_BF16_PEAK}
     if reps > 1:
         # Two yardsticks on the same box in the same run, neither on the product path: the same kernel on all-zero
         # operands (no switching activity: what the code alone allows, without the part's power management), and the

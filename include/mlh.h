@@ -258,8 +258,11 @@ int mlh_probe_hops(mlh_ctx* ctx, int iters, double* us);
 int mlh_time_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, double* total_ms);
 
 /* Stand-alone run of the MFMA GEMM used by prefill and batched decode (no context needed):
- * C[M,N] = A[M,K] . B[N,K]^T (+ R[M,N]), host fp32 arrays in and out; with MLH_DTYPE_BF16 both
- * operands are rounded to bf16 first.  K*4 (fp32) or K*2 (bf16) must be a multiple of 128.
+ * C[M,N] = A[M,K] . B[N,K]^T (+ R[M,N]), host fp32 arrays in and out; with MLH_DTYPE_BF16 (or 2 = IEEE half) both
+ * operands are rounded to that type first.  K*4 (fp32) or K*2 (bf16, half) must be a multiple of 128.
+ * dtype | 0x100 selects the SwiGLU epilogue of the gate/up projection instead (R must be null, N even): columns 2j and
+ * 2j+1 of the product are gate and up of unit j and C is [M, N/2] with C[m, j] = silu(gate) * up, rounded to the
+ * operand type as the prefill pass stores it (inference.cu:262-281).
  * iters > 0 additionally times that many launches with HIP events (mean microseconds in avg_us).
  * Replaces nothing in the reference by itself: it exposes the kernel that stands in for the
  * cublasGemmEx calls of inference.cu:401-743 so that it can be checked and measured alone. */

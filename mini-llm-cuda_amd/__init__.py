@@ -468,17 +468,19 @@ class Vocab:
             pass
 
 
-def selftest_gemm(a, b, r=None, bf16=False, iters=0, f16=False):
-    """C = a . b^T (+ r) through the device GEMM kernel; returns (C, mean microseconds or None)."""
+def selftest_gemm(a, b, r=None, bf16=False, iters=0, f16=False, swiglu=False):
+    """C = a . b^T (+ r) through the device GEMM kernel; returns (C, mean microseconds or None).  swiglu: the
+    gate/up epilogue instead, C[m, j] = silu(P[m, 2j]) * P[m, 2j+1] in the operand type, shape [M, N/2]."""
     a = np.ascontiguousarray(a, dtype=np.float32)
     b = np.ascontiguousarray(b, dtype=np.float32)
     m, k = a.shape
     n = b.shape[0]
     if r is not None:
         r = np.ascontiguousarray(r, dtype=np.float32)
-    c = np.empty((m, n), dtype=np.float32)
+    c = np.empty((m, n // 2 if swiglu else n), dtype=np.float32)
     us = c_double()
-    rc = dev.mlh_selftest_gemm(2 if f16 else (DTYPE_BF16 if bf16 else DTYPE_F32), m, n, k, a.ctypes.data, b.ctypes.data,
+    code = (2 if f16 else (DTYPE_BF16 if bf16 else DTYPE_F32)) | (0x100 if swiglu else 0)
+    rc = dev.mlh_selftest_gemm(code, m, n, k, a.ctypes.data, b.ctypes.data,
                                r.ctypes.data if r is not None else None, c.ctypes.data, iters, byref(us))
     if rc != 0:
         raise MlhError(f"GEMM self-test failed ({rc}): unsupported shape or no device")

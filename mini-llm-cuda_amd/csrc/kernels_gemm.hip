@@ -1141,15 +1141,20 @@ static void host_to_f16(const float* src, f16_t* dst, size_t n) {
 
 // Stand-alone check and timing of the GEMM kernel: host fp32 inputs (rounded to bf16 first when
 // dtype says so), result back on the host, mean launch time over `iters` launches from HIP events.
-extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A, const float* B, const float* R, float* C,
+extern "C" int mlh_selftest_gemm(int dtypeAndEpilogue, int M, int N, int K, const float* A, const float* B, const float* R, float* C,
                                  int iters, double* avgUs) {
-    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return -1;
+    const int dtype = dtypeAndEpilogue & 0xff;
+    const bool swiglu = (dtypeAndEpilogue & MLH_SELFTEST_SWIGLU) != 0; // C is then [M, N / 2]: silu(gate) * up of the column pairs
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0 || (swiglu && (R || (N & 1)))) return -1;
     if (mlh_device_count() <= 0) return -1;
     const size_t esz = dtype == MLH_DTYPE_F32 ? 4 : 2;
-    void *dA = nullptr, *dB = nullptr, *dW = nullptr;
-    float *dC = nullptr, *dR = nullptr;
+    const int NC = swiglu ? N / 2 : N;
+    const size_t csz = swiglu ? esz : 4; // the SwiGLU epilogue writes the operand type
+    void *dA = nullptr, *dB = nullptr, *dW = nullptr, *dC = nullptr;
+    float* dR = nullptr;
     int rc = 0;
     std::vector<bf16_t> ha, hb;
+    std::vector<uint16_t> hc;
     const void *srcA = A, *srcB = B;
     if (dtype == MLH_DTYPE_BF16) {
         ha.resize((size_t)M * K); hb.resize((size_t)N * K);
@@ -1160,28 +1165,38 @@ extern "C" int mlh_selftest_gemm(int dtype, int M, int N, int K, const float* A,
         host_to_f16(A, (f16_t*)ha.data(), ha.size()); host_to_f16(B, (f16_t*)hb.data(), hb.size());
         srcA = ha.data(); srcB = hb.data();
     }
+    const int epi = swiglu ? GEMM_EPI_SWIGLU : GEMM_EPI_PLAIN;
     hipEvent_t e0 = nullptr, e1 = nullptr;
 #define ST(x) do { if ((x) != hipSuccess) { rc = -2; goto done; } } while (0)
     ST(hipMalloc(&dA, (size_t)M * K * esz)); ST(hipMalloc(&dB, (size_t)N * K * esz));
-    ST(hipMalloc((void**)&dC, (size_t)M * N * 4));
+    ST(hipMalloc(&dC, (size_t)M * NC * csz));
     if (R) { ST(hipMalloc((void**)&dR, (size_t)M * N * 4)); ST(hipMemcpy(dR, R, (size_t)M * N * 4, hipMemcpyHostToDevice)); }
     ST(hipMemcpy(dA, srcA, (size_t)M * K * esz, hipMemcpyHostToDevice));
     ST(hipMemcpy(dB, srcB, (size_t)N * K * esz, hipMemcpyHostToDevice));
     ST(hipMalloc(&dW, mlh_gemm_workspace_bytes()));
     ST(hipMemset(dW, 0, mlh_gemm_workspace_bytes()));
-    ST(mlh_gemm_tn_epi(nullptr, dtype, GEMM_EPI_PLAIN, dA, K, dB, K, dC, N, dR, N, M, N, K, dW));
+    ST(mlh_gemm_tn_epi(nullptr, dtype, epi, dA, K, dB, K, dC, NC, dR, N, M, N, K, dW));
     ST(hipDeviceSynchronize());
     if (iters > 0 && avgUs) {
         ST(hipEventCreate(&e0)); ST(hipEventCreate(&e1));
         ST(hipEventRecord(e0, nullptr));
-        for (int i = 0; i < iters; i++) ST(mlh_gemm_tn_epi(nullptr, dtype, GEMM_EPI_PLAIN, dA, K, dB, K, dC, N, dR, N, M, N, K, dW));
+        for (int i = 0; i < iters; i++) ST(mlh_gemm_tn_epi(nullptr, dtype, epi, dA, K, dB, K, dC, NC, dR, N, M, N, K, dW));
         ST(hipEventRecord(e1, nullptr));
         ST(hipEventSynchronize(e1));
         float ms = 0.f;
         ST(hipEventElapsedTime(&ms, e0, e1));
         *avgUs = (double)ms * 1000.0 / iters;
     }
-    ST(hipMemcpy(C, dC, (size_t)M * N * 4, hipMemcpyDeviceToHost));
+    if (csz == 4) {
+        ST(hipMemcpy(C, dC, (size_t)M * NC * 4, hipMemcpyDeviceToHost));
+    } else { // half or bf16 results back as floats
+        hc.resize((size_t)M * NC);
+        ST(hipMemcpy(hc.data(), dC, hc.size() * 2, hipMemcpyDeviceToHost));
+        for (size_t i = 0; i < hc.size(); i++) {
+            if (dtype == MLH_DTYPE_BF16) { const uint32_t u = (uint32_t)hc[i] << 16; memcpy(&C[i], &u, 4); }
+            else { _Float16 h; memcpy(&h, &hc[i], 2); C[i] = (float)h; }
+        }
+    }
 #undef ST
 done:
     if (e0) (void)hipEventDestroy(e0);

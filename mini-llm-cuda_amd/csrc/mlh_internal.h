@@ -17,6 +17,7 @@ typedef uint16_t bf16_t;
 // IEEE half, as the MFMA path stores weights and activations of bf16 models (see MLH_GEMM_F16)
 struct f16_t { uint16_t bits; };
 #define MLH_GEMM_F16 2 // GEMM operand type code beside MLH_DTYPE_F32 / MLH_DTYPE_BF16
+#define MLH_SELFTEST_SWIGLU 0x100 // mlh_selftest_gemm: flag beside the operand type, selects the SwiGLU epilogue
 
 // Device-side description of one transformer block.
 struct LayerDev {

@@ -57,6 +57,27 @@ def test_gemm_f16(pkg, m, n, k):
     assert np.max(np.abs(c - want)) <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5
 
 
+@pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("m,n,k", [(300, 512, 256), (257, 1000, 704), (130, 36, 128), (100, 256, 512), (64, 320, 256), (9, 128, 2048)])
+def test_gemm_swiglu_epilogue(pkg, orc, kind, m, n, k):
+    """The gate/up epilogue (inference.cu:262-281) of all three tile families: columns 2j, 2j+1 of the product are
+    gate and up of unit j, the result silu(gate) * up is stored in the operand type; ragged M, N/2 not a multiple
+    of the store width."""
+    rng = np.random.default_rng(m + 7 * n + k)
+    a = (0.5 * rng.standard_normal((m, k))).astype(np.float32)
+    b = (0.5 * rng.standard_normal((n, k)) / np.sqrt(k) * 8).astype(np.float32)
+    if kind == "bf16":
+        a, b = orc.round_bf16(a), orc.round_bf16(b)
+    elif kind == "f16":
+        a, b = a.astype(np.float16).astype(np.float32), b.astype(np.float16).astype(np.float32)
+    c, _ = pkg.selftest_gemm(a, b, None, bf16=(kind == "bf16"), f16=(kind == "f16"), swiglu=True)
+    assert c.shape == (m, n // 2)
+    p = a.astype(np.float64) @ b.astype(np.float64).T
+    want = p[:, 0::2] / (1 + np.exp(-p[:, 0::2])) * p[:, 1::2]
+    tol = {"f32": 2e-5, "bf16": 2.0 ** -8, "f16": 2.0 ** -11}[kind]  # the result is rounded to the operand type
+    assert np.max(np.abs(c - want)) <= tol * np.max(np.abs(want)) + 2e-5 * np.sqrt(k), (kind, m, n, k)
+
+
 def test_gemm_rejects_bad_k(pkg):
     a = np.zeros((4, 40), dtype=np.float32)
     with pytest.raises(RuntimeError):
