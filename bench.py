@@ -259,6 +259,8 @@ def gemm_leg(m, iters=3, reps=1):
     rng = np.random.default_rng(5)
     a = rng.standard_normal((M, hp.dim), dtype=np.float32)
     b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
+    if reps == 1:  # profiler runs: the product once more with the epilogue the pass uses
+        m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)
     runs = [m.selftest_gemm(a, b, None, f16=True, iters=iters)[1] for _ in range(reps)]
     us = stats(runs)["median"]
     flop = 2.0 * M * 2 * hp.ffnDim * hp.dim
