@@ -440,6 +440,321 @@ static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, in
     return hipGetLastError();
 }
 
+// ----------------------------------------------------------------------------
+// Large-tile kernel for two-byte operands (the prefill path of a bf16 model): the same 256 x 256 tile, K slices and
+// LDS layout as k_gemm_tn_big, but FOUR waves per workgroup, one per SIMD, each owning 128 x 128 of the tile in 256
+// accumulator registers, multiplied with v_mfma_f32_16x16x32 (64 blocks of 16 x 16 per wave, two 32-wide steps per
+// slice).  On operand data that toggles the multipliers the part is limited by power, not by issue slots, and the
+// 16 x 16 x 32 form does a given product on less of it than 32 x 32 x 16 (an accumulator is read and written once per
+// 32 products instead of once per 16): a register-only loop of either form sustains 1.95 against 1.70 PFLOP/s on
+// N(0, s) data and the same 2.4-2.5 on zeros.
+// With one instruction stream per SIMD nothing takes turns: every wave issues its own 16 loads of a slice between its
+// own MFMAs (one load per GW_LR MFMAs), reads an operand fragment behind every other MFMA while there are any to read,
+// and the MFMA pipe only stands still at two points per slice:
+//   F  the wave has read the second (last) step's operands of the slice it is multiplying -- they are read during the
+//      first quarter of the slice -- so after a barrier the stage is free and the loads of the slice after next start
+//      flowing into it, more than a slice and a half before they are needed;
+//   R  the loads of the next slice have landed for every wave (vmcnt counts in issue order: the loads already out for
+//      the slice after next may stay in flight), so after a barrier its first step's operands are read under the last
+//      quarter of the current slice's MFMAs.
+// The load cursor runs ahead of the multiply position and crosses tile boundaries by itself: a workgroup walks its
+// tiles in one launch and the next tile's first two slices are in flight while the epilogue runs.  The epilogue uses a
+// patch of LDS per wave outside the two stages.  Per slice and wave: 128 MFMAs, 32 LDS reads, 16 loads -- a third fewer
+// LDS bytes per flop than the 8-wave kernel (128 x 128 per wave instead of 128 x 64).
+// ----------------------------------------------------------------------------
+#define GW_THREADS 256
+#define GW_FPOS 40     // MFMA index within a slice (0..127) in front of which F sits
+#define GW_RPOS 96     // ... and R
+#define GW_LR 6        // one load per this many MFMAs, starting at F
+#define GW_NOUT ((GW_RPOS - GW_FPOS + GW_LR - 1) / GW_LR) // loads of the slice after next that are out when R is reached
+#define GW_EP 144      // row pitch of a wave's epilogue patch in bytes (rows 4 banks apart)
+#define GW_LDS (2 * GB_STAGE + 4 * 16 * GW_EP)
+#define GW_LOADK(p_) (((p_) - GW_FPOS) / GW_LR)
+#define GW_ISLOAD(p_) ((p_) >= GW_FPOS && ((p_) - GW_FPOS) % GW_LR == 0 && GW_LOADK(p_) < 16)
+
+template <typename T> struct GemmMma16;
+// (written as the instruction: with 64 accumulator tuples the register allocator otherwise shuffles them between
+// MFMAs; the "a" constraint keeps every tuple in its accumulator registers from the first slice to the epilogue)
+template <> struct GemmMma16<f16_t> {
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+template <> struct GemmMma16<bf16_t> {
+    static __device__ __forceinline__ void mma(const u32x4& a, const u32x4& b, f32x4& c) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
+};
+
+template <typename T, int EPI>
+__global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__ A, int lda, const T* __restrict__ B, int ldb,
+                                                           void* Cv, int ldc, const float* R, int ldr, int M, int N, int K, int tilesM, int tilesN, float alpha) {
+    static_assert(sizeof(T) == 2, "two-byte operands only");
+    extern __shared__ __attribute__((aligned(16))) unsigned char gsm[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    int id = blockIdx.x, tm, tn;
+    gemm_tile_of(id, tilesM, tilesN, tm, tn);
+    if (tm < 0) return;
+    const int nslices = (int)(((size_t)K * sizeof(T)) / GKB);
+    const size_t ldaB = (size_t)lda * sizeof(T), ldbB = (size_t)ldb * sizeof(T);
+    const unsigned lds0 = (unsigned)(unsigned long long)gsm;
+    typedef __attribute__((address_space(3))) u32x4 lds_u32x4;
+    typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    auto lds_rd = [](unsigned addr, int imm) -> u32x4 { return *(const lds_u32x4*)(addr + (unsigned)imm); };
+
+    // ---- load side: wave w fetches rows 64 w .. 64 w + 63 of the A rows and of the B rows of the cursor's tile, eight rows
+    // per instruction; address = scalar base (advanced slice by slice) + a lane offset that only changes from tile to tile,
+    // LDS target scalar: no vector-ALU instruction per load.  Rows past the end of a matrix fetch its last row again.
+    unsigned goffA[8], goffB[8];
+    unsigned long long baseA, baseB;
+    auto uniform64 = [](unsigned long long v) { asm("" : "+s"(v)); return v; };
+    auto aim = [&](int tm_, int tn_) {
+        const int m0_ = tm_ * GB_T, n0_ = tn_ * GB_T;
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const int r = wave * 64 + q * 8 + (lane >> 3);
+            const int pc = (lane & 7) ^ ((r >> 1) & 7);
+            goffA[q] = (unsigned)((size_t)(min(m0_ + r, M - 1) - m0_) * ldaB) + pc * 16;
+            goffB[q] = (unsigned)((size_t)(min(n0_ + r, N - 1) - n0_) * ldbB) + pc * 16;
+        }
+        baseA = uniform64((unsigned long long)A + (size_t)m0_ * ldaB);
+        baseB = uniform64((unsigned long long)B + (size_t)n0_ * ldbB);
+    };
+    auto dma16 = [](unsigned long long sbase, unsigned laneOff, unsigned ldsAddr) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsAddr), "v"(laneOff), "s"(sbase) : "memory", "m0");
+    };
+    const unsigned ldsLoad = lds0 + (unsigned)(wave * 64 * GKB);
+    // load i (0..15) of the cursor's slice into the stage at byte offset SOFF: even i -> A rows, odd i -> B rows
+#define GW_LOAD1(i, SOFF)                                                                                                \
+    do {                                                                                                                 \
+        if (((i) & 1) == 0) dma16(baseA, goffA[(i) >> 1], ldsLoad + (SOFF) + ((i) >> 1) * 8 * GKB);                       \
+        else dma16(baseB, goffB[(i) >> 1], ldsLoad + (SOFF) + GB_T * GKB + ((i) >> 1) * 8 * GKB);                         \
+    } while (0)
+    int curId = id, curS = 0;
+    aim(tm, tn);
+    auto advance = [&]() { // the cursor's slice is out: on to the next one, of the next tile when this one is through
+        curS++;
+        baseA += GKB; baseB += GKB;
+        if (curS == nslices) {
+            curS = 0;
+            curId += (int)gridDim.x;
+            int a, b;
+            gemm_tile_of(curId, tilesM, tilesN, a, b);
+            if (a >= 0) aim(a, b);
+            else { baseA -= (unsigned long long)nslices * GKB; baseB -= (unsigned long long)nslices * GKB; } // past the last tile: the same rows again, never multiplied
+        }
+    };
+
+    // ---- operand side: lane (r16 = lane & 15, kq = lane >> 4) supplies row r16 of a 16-row block and the eight K elements
+    // 8 kq .. 8 kq + 7 of a 32-wide step kk: piece 4 kk + kq of the row's 128-byte slice, read from the slot the fetching
+    // lane put it in.  Block b of the wave's A rows at + b * 16 rows (an immediate), the B rows behind the stage's A rows.
+    // The stage of the slice being multiplied alternates: its offset is kept in the addresses themselves and flipped
+    // after every slice, so there is one copy of the slice's code.
+    const int r16 = lane & 15, kq = lane >> 4;
+    const int key = (r16 >> 1) & 7;
+    unsigned rdA[2], rdB[2], rdNextA, rdNextB; // this stage, steps 0 and 1; the other stage, step 0
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+        rdA[kk] = lds0 + wm * 128 * GKB + r16 * GKB + ((4 * kk + kq) ^ key) * 16;
+        rdB[kk] = rdA[kk] - wm * 128 * GKB + GB_T * GKB + wn * 128 * GKB;
+    }
+    rdNextA = rdA[0] + GB_STAGE;
+    rdNextB = rdB[0] + GB_STAGE;
+    unsigned stageOff = 0; // scalar: byte offset of the stage being multiplied
+
+    f32x4 acc[8][8];
+    u32x4 fa[2][8], fb[2][8];
+    // prologue: slice 0 whole, then the loads of slice 1 that a slice in front of it would have issued after its F
+#pragma unroll
+    for (int i = 0; i < 16; i++) GW_LOAD1(i, 0u);
+    advance();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < 8; b++) {
+        fb[0][b] = lds_rd(rdB[0], b * 16 * GKB);
+        fa[0][b] = lds_rd(rdA[0], b * 16 * GKB);
+    }
+#pragma unroll
+    for (int p = GW_FPOS; p < 128; p++)
+        if (GW_ISLOAD(p)) { GW_LOAD1(GW_LOADK(p), (unsigned)GB_STAGE); if (GW_LOADK(p) == 15) advance(); }
+
+    // One slice; p = 64 kk + 8 bn + bm is the MFMA's index within it.  On entry fa[0] / fb[0] hold the first step's operands.
+    // Reads (behind MFMAs with an odd index, the loads go behind even ones): the second step's during p = 1..31, the next
+    // slice's first step (other stage) from R on, in the order the MFMAs need them (B block 0, the eight A blocks, B 1..7).
+    // Loads: the slice after next from F on (into this stage), its tail during the first MFMAs of the next slice.
+    // The product is formed transposed (weights as the first operand): see the epilogue.  firstOfTile: R also has the
+    // epilogue's stores of the previous tile in front of it and waits for everything.
+#define GW_SLICE(firstOfTile)                                                                                                \
+    {                                                                                                                        \
+        const unsigned otherOff = stageOff ^ (unsigned)GB_STAGE;                                                             \
+        _Pragma("unroll") for (int kk = 0; kk < 2; kk++) {                                                                   \
+            _Pragma("unroll") for (int bn = 0; bn < 8; bn++)                                                                 \
+            _Pragma("unroll") for (int bm = 0; bm < 8; bm++) {                                                               \
+                const int i = 8 * bn + bm, p = 64 * kk + i;                                                                  \
+                if (p == GW_FPOS) {                                                                                          \
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                                       \
+                    __builtin_amdgcn_s_barrier();                                                                            \
+                    __builtin_amdgcn_sched_barrier(0);                                                                       \
+                }                                                                                                            \
+                if (p == GW_RPOS) {                                                                                          \
+                    if (firstOfTile) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                        \
+                    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(GW_NOUT) : "memory");                                      \
+                    __builtin_amdgcn_s_barrier();                                                                            \
+                    __builtin_amdgcn_sched_barrier(0);                                                                       \
+                }                                                                                                            \
+                GemmMma16<T>::mma(fb[kk][bn], fa[kk][bm], acc[bm][bn]);                                                      \
+                {                                                                                                            \
+                    int q = -1;                                                                                              \
+                    if (kk == 0 && i < 32 && (i & 1)) q = i >> 1;                                                            \
+                    if (kk == 1 && p > GW_RPOS && ((p - GW_RPOS) & 1) && (p - GW_RPOS) / 2 < 16) q = (p - GW_RPOS) / 2;       \
+                    if (q >= 0) {                                                                                            \
+                        const int nb = kk ^ 1;                                                                               \
+                        const unsigned raA = kk == 0 ? rdA[1] : rdNextA, raB = kk == 0 ? rdB[1] : rdNextB;                    \
+                        if (q == 0) fb[nb][0] = lds_rd(raB, 0);                                                              \
+                        else if (q < 9) fa[nb][q - 1] = lds_rd(raA, (q - 1) * 16 * GKB);                                     \
+                        else fb[nb][q - 8] = lds_rd(raB, (q - 8) * 16 * GKB);                                                \
+                    }                                                                                                        \
+                }                                                                                                            \
+                if (GW_ISLOAD(p)) { GW_LOAD1(GW_LOADK(p), stageOff); if (GW_LOADK(p) == 15) advance(); }                     \
+                if (GW_ISLOAD(p + 128)) { GW_LOAD1(GW_LOADK(p + 128), otherOff); if (GW_LOADK(p + 128) == 15) advance(); }   \
+                __builtin_amdgcn_sched_barrier(0);                                                                           \
+            }                                                                                                                \
+        }                                                                                                                    \
+        stageOff = otherOff;                                                                                                 \
+        rdA[0] ^= (unsigned)GB_STAGE; rdA[1] ^= (unsigned)GB_STAGE; rdB[0] ^= (unsigned)GB_STAGE; rdB[1] ^= (unsigned)GB_STAGE; \
+        rdNextA ^= (unsigned)GB_STAGE; rdNextB ^= (unsigned)GB_STAGE;                                                        \
+    }
+
+    for (bool firstTile = true;; firstTile = false) {
+        const int m0 = tm * GB_T, n0 = tn * GB_T;
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[i][j] = (f32x4)(0.f);
+        for (int s = 0; s < nslices; s++) GW_SLICE(s == 0 && !firstTile)
+
+        // Epilogue.  Lane (r16, kq) holds, for every 16 x 16 block, row r16 of C and the columns 4 kq .. 4 kq + 3: a SwiGLU
+        // lane has two (gate, up) pairs.  Blocks go through the wave's patch of LDS (16 rows of 128 bytes) and are read back
+        // with eight lanes per row, so that a store instruction writes whole 128-byte lines; the residual is read the same
+        // way.  LDS instructions of a wave execute in order: the next writes need not wait for this read-back.
+        {
+            const unsigned patch = lds0 + 2 * GB_STAGE + wave * (16 * GW_EP);
+            const unsigned rdp = patch + (lane >> 3) * GW_EP + (lane & 7) * 16;
+            const int mW = m0 + wm * 128, nW = n0 + wn * 128;
+            if (EPI == GEMM_EPI_PLAIN) {
+                const bool vec = ((ldc & 3) == 0) && (!R || (ldr & 3) == 0) && (((unsigned long long)Cv & 15) == 0) && (((unsigned long long)R & 15) == 0);
+                const bool inside = vec && mW + 128 <= M && nW + 128 <= N; // the wave's whole 128 x 128 lies inside C: no per-element tests
+                const unsigned wr = patch + r16 * GW_EP + kq * 16;
+#pragma unroll
+                for (int bm = 0; bm < 8; bm++)
+#pragma unroll
+                    for (int bp = 0; bp < 4; bp++) { // two column blocks side by side: 32 columns = one 128-byte line per row
+                        *(lds_f32x4*)(wr) = acc[bm][2 * bp] * alpha;
+                        *(lds_f32x4*)(wr + 64) = acc[bm][2 * bp + 1] * alpha;
+                        const int rowb = mW + bm * 16 + (lane >> 3), col = nW + bp * 32 + (lane & 7) * 4;
+                        f32x4 v[2];
+#pragma unroll
+                        for (int k = 0; k < 2; k++) v[k] = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
+                        if (inside) {
+                            float* cp = (float*)Cv + (size_t)rowb * ldc + col;
+                            if (R) {
+                                const float* rp = R + (size_t)rowb * ldr + col;
+#pragma unroll
+                                for (int k = 0; k < 2; k++) v[k] += *reinterpret_cast<const f32x4*>(rp + (size_t)(8 * k) * ldr);
+                            }
+#pragma unroll
+                            for (int k = 0; k < 2; k++) *reinterpret_cast<f32x4*>(cp + (size_t)(8 * k) * ldc) = v[k];
+                            continue;
+                        }
+#pragma unroll
+                        for (int k = 0; k < 2; k++) {
+                            const int row = rowb + 8 * k;
+                            if (row >= M || col >= N) continue;
+                            float* cp = (float*)Cv + (size_t)row * ldc + col;
+                            if (vec && col + 3 < N) {
+                                if (R) v[k] += *reinterpret_cast<const f32x4*>(R + (size_t)row * ldr + col);
+                                *reinterpret_cast<f32x4*>(cp) = v[k];
+                            } else {
+                                const float* rp = R ? R + (size_t)row * ldr + col : nullptr;
+                                cp[0] = v[k].x + (rp ? rp[0] : 0.f);
+                                if (col + 1 < N) cp[1] = v[k].y + (rp ? rp[1] : 0.f);
+                                if (col + 2 < N) cp[2] = v[k].z + (rp ? rp[2] : 0.f);
+                                if (col + 3 < N) cp[3] = v[k].w + (rp ? rp[3] : 0.f);
+                            }
+                        }
+                    }
+            } else { // SwiGLU: columns 2 j, 2 j + 1 of the product are gate and up of unit j; U[m, j] = silu(gate) * up in the operand type
+                const bool vec = (((size_t)ldc * 2) & 15) == 0 && (((unsigned long long)Cv & 15) == 0);
+                const int jW = nW >> 1, NU = N >> 1; // the wave's 128 columns are 64 units: 128 bytes per row, eight lanes a row
+                const bool inside = vec && mW + 128 <= M && nW + 128 <= N;
+#pragma unroll
+                for (int bm = 0; bm < 8; bm++) {
+#pragma unroll
+                    for (int bn = 0; bn < 8; bn++) {
+                        const float g0 = acc[bm][bn].x * alpha, u0 = acc[bm][bn].y * alpha;
+                        const float g1 = acc[bm][bn].z * alpha, u1 = acc[bm][bn].w * alpha;
+                        const float o0 = (g0 / (1.0f + expf(-g0))) * u0, o1 = (g1 / (1.0f + expf(-g1))) * u1;
+                        *(lds_u32*)(patch + r16 * GW_EP + (bn * 8 + 2 * kq) * 2) = GemmTraits<T>::bits(o0) | (GemmTraits<T>::bits(o1) << 16);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 2; k++) {
+                        const int rl = (lane >> 3) + 8 * k, piece = lane & 7;
+                        const f32x4 v = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
+                        const int row = mW + bm * 16 + rl, j = jW + piece * 8;
+                        T* up = (T*)Cv + (size_t)row * ldc + j;
+                        if (inside) { *reinterpret_cast<f32x4*>(up) = v; continue; }
+                        if (row >= M || j >= NU) continue;
+                        if (vec && j + 7 < NU) {
+                            *reinterpret_cast<f32x4*>(up) = v;
+                        } else {
+                            const uint32_t w[4] = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+#pragma unroll
+                            for (int e = 0; e < 8; e++)
+                                if (j + e < NU) reinterpret_cast<uint16_t*>(up)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+                        }
+                    }
+                }
+            }
+        }
+        id += (int)gridDim.x;
+        gemm_tile_of(id, tilesM, tilesN, tm, tn);
+        if (tm < 0) break;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // the cursor's last loads target this workgroup's LDS: let them land before it is given up
+#undef GW_SLICE
+#undef GW_LOAD1
+}
+
+template <typename T>
+static hipError_t launch_gemm_w4(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
+                                 const float* R, int ldr, int M, int N, int K, float alpha) {
+    const int tilesM = (M + GB_T - 1) / GB_T, tilesN = (N + GB_T - 1) / GB_T;
+    static int numCUs = 0;
+    if (!numCUs) {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipErrorInvalidDevice;
+        numCUs = std::max(8, (prop.multiProcessorCount / 8) * 8);
+    }
+    const unsigned grid = (unsigned)std::min(numCUs, ((tilesM * tilesN + 7) / 8) * 8); // one workgroup per compute unit walks its tiles
+    const size_t lds = GW_LDS;
+    static bool attr = false;
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_w4<T, GEMM_EPI_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_w4<T, GEMM_EPI_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    if (epi == GEMM_EPI_SWIGLU)
+        hipLaunchKernelGGL((k_gemm_tn_w4<T, GEMM_EPI_SWIGLU>), dim3(grid), dim3(GW_THREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
+    else
+        hipLaunchKernelGGL((k_gemm_tn_w4<T, GEMM_EPI_PLAIN>), dim3(grid), dim3(GW_THREADS), lds, stream, (const T*)A, lda, (const T*)B, ldb, C, ldc, R, ldr, M, N, K, tilesM, tilesN, alpha);
+    return hipGetLastError();
+}
+
 template <typename T, int BM, int BN>
 static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                               const float* R, int ldr, int M, int N, int K, float alpha) {
@@ -1109,8 +1424,8 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
                      (launch_gemm_skinny<f16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)));
     if (M > 128)
         GEMM_BY_TYPE((launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
-                     (launch_gemm_big<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
-                     (launch_gemm_big<f16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)));
+                     (launch_gemm_w4<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
+                     (launch_gemm_w4<f16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)));
     GEMM_BY_TYPE((launch_gemm<float, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
                  (launch_gemm<bf16_t, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
                  (launch_gemm<f16_t, 2, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)));

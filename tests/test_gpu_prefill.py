@@ -32,7 +32,8 @@ def test_gemm_fp32(pkg, m, n, k):
         assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 1, 64), (17, 300, 128), (130, 257, 704), (300, 128, 2048), (8, 2048, 5632), (33, 96, 512)])
+@pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 1, 64), (17, 300, 128), (130, 257, 704), (300, 128, 2048), (8, 2048, 5632), (33, 96, 512),
+                                   (1100, 17000, 192), (300, 600, 64)])
 def test_gemm_bf16(pkg, orc, m, n, k):
     """bf16 operands (already representable, so the product is exact in fp32) with fp32 accumulation."""
     rng = np.random.default_rng(m * 1000 + n + k + 1)
@@ -46,9 +47,11 @@ def test_gemm_bf16(pkg, orc, m, n, k):
         assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 2048, 5632), (130, 257, 704), (300, 4096, 2048)])
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 5632), (130, 257, 704), (300, 4096, 2048), (1100, 17000, 192), (300, 600, 64), (2100, 9000, 448)])
 def test_gemm_f16(pkg, m, n, k):
-    """IEEE-half operands (what the MFMA path of bf16 models multiplies) with fp32 accumulation."""
+    """IEEE-half operands (what the MFMA path of bf16 models multiplies) with fp32 accumulation.  The larger shapes
+    give a workgroup of the 256 x 256-tile kernel several tiles (more than 256 tiles in all) with an odd and an even
+    number of K slices, ragged edges in M and N, and a single-slice K."""
     rng = np.random.default_rng(m + n + k)
     a = rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).astype(np.float32)
     b = rng.standard_normal((n, k), dtype=np.float32).astype(np.float16).astype(np.float32)
@@ -58,7 +61,8 @@ def test_gemm_f16(pkg, m, n, k):
 
 
 @pytest.mark.parametrize("kind", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("m,n,k", [(300, 512, 256), (257, 1000, 704), (130, 36, 128), (100, 256, 512), (64, 320, 256), (9, 128, 2048)])
+@pytest.mark.parametrize("m,n,k", [(300, 512, 256), (257, 1000, 704), (130, 36, 128), (100, 256, 512), (64, 320, 256), (9, 128, 2048),
+                                   (1100, 17000, 192)])
 def test_gemm_swiglu_epilogue(pkg, orc, kind, m, n, k):
     """The gate/up epilogue (inference.cu:262-281) of all three tile families: columns 2j, 2j+1 of the product are
     gate and up of unit j, the result silu(gate) * up is stored in the operand type; ragged M, N/2 not a multiple
