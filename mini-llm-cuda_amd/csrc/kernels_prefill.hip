@@ -42,6 +42,8 @@ struct PfArgs {
     int aLd;
     float* H1;         // [n, dim]
     void* U;           // [n, ffn]
+    uint16_t* Kh;      // [n, dim] IEEE-half copies of this call's K and V rows (after norm and RoPE), or null: what the MFMA
+    uint16_t* Vh;      //          attention reads when every segment starts at position 0 (all of its keys are rows of the call)
 };
 
 __device__ __forceinline__ float pf_wave_sum(float v) {
@@ -136,6 +138,10 @@ __global__ void __launch_bounds__(PWG) k_pf_rmsnorm(const float* __restrict__ X,
 
 // Per (head, row): per-head RMSNorm of q and k (inference.cu:52-81, 97-111), RoPE on adjacent pairs at the
 // row's position (inference.cu:113-134), q written back in place, k and v written to the KV pages.
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) { // two floats -> two IEEE halves (round to nearest even)
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
+}
+
 template <int HD>
 __global__ void __launch_bounds__(64) k_pf_qk_rope_kv(PfArgs P, LayerDev L) {
     constexpr int EPL = HD / 64;
@@ -181,6 +187,19 @@ __global__ void __launch_bounds__(64) k_pf_qk_rope_kv(PfArgs P, LayerDev L) {
         qkv[h * HD + i] = qv[e];
         L.K[o + i] = kv[e];
         L.V[o + i] = vv[e];
+    }
+    if (P.Kh) { // the half copies, rounded exactly as the attention kernel rounds the fp32 rows on its way into LDS
+        const size_t ho = (size_t)row * a.dim + h * HD + lane * EPL;
+        if (EPL == 2) {
+            *reinterpret_cast<uint32_t*>(P.Kh + ho) = pack_f16(kv[0], kv[1]);
+            *reinterpret_cast<uint32_t*>(P.Vh + ho) = pack_f16(vv[0], vv[1]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < EPL; e++) {
+                P.Kh[ho + e] = __builtin_bit_cast(uint16_t, (_Float16)kv[e]);
+                P.Vh[ho + e] = __builtin_bit_cast(uint16_t, (_Float16)vv[e]);
+            }
+        }
     }
 }
 
@@ -295,9 +314,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) { // two floats -> two IEEE halves (round to nearest even)
-    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (_Float16)hi) << 16);
-}
 
 // position of key k (0..63) of a page along the permuted contraction axis of O^T += V^T . P^T
 __device__ __forceinline__ int pv_slot(int k) {
@@ -306,8 +322,8 @@ __device__ __forceinline__ int pv_slot(int k) {
     return 16 * (2 * b + (i >> 3)) + 8 * hh + (i & 7);
 }
 
-template <int HD>
-__global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
+template <int HD, bool H16>
+__global__ void __launch_bounds__(PWG, H16 ? 2 : 1) k_pf_attn_mfma(PfArgs P, LayerDev L) {
     constexpr int KP = HD + 8;   // K tile row pitch (16-bit elements): 16-byte reads, rows 4 banks apart
     constexpr int VP = 64 + 8;   // V^T row pitch
     constexpr int KS = HD / 16;  // 16-wide contraction steps of K . Q^T
@@ -349,13 +365,34 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
     // A tile's K and V rows travel global -> registers -> LDS; the loads of tile t + 1 are issued before tile t is
     // multiplied, so their latency runs under the MFMAs.  Rows beyond the last position any query of the workgroup
     // may see are read from a clamped row and zeroed (every load unconditional: all of them in flight at once).
+    // H16: every segment of the call starts at position 0, so key j of the segment is row segStart + j of the call and
+    // its K and V rows exist as halves (written by the QK-norm / RoPE kernel): half the bytes, no conversion, and few
+    // enough registers for two workgroups per compute unit -- one multiplies while the other does its softmax.
     constexpr int NK = 64 * (HD / 4) / PWG, NV = 32 * (HD / 4) / PWG;
-    f32x4 kreg[NK], vreg[NV][2];
+    constexpr int NK16 = 64 * (HD / 8) / PWG, NV16 = 32 * (HD / 8) / PWG;
+    f32x4 kreg[H16 ? 1 : NK], vreg[H16 ? 1 : NV][2];
+    u32x4 kreg16[H16 ? NK16 : 1], vreg16[H16 ? NV16 : 1][2];
     auto fetch = [&](int t) {
         const int j0 = t << 6;
+        const int rmax = maxPos - j0; // >= 0
+        if (H16) {
+            const size_t base = ((size_t)P.segStart[seg] + j0) * a.dim + h * HD; // pos0 == 0: key position == row within the segment
+#pragma unroll
+            for (int n = 0; n < NK16; n++) {
+                const int i = tid + n * PWG, r = i / (HD / 8), c8 = (i % (HD / 8)) * 8;
+                kreg16[n] = *reinterpret_cast<const u32x4*>(P.Kh + base + (size_t)min(r, rmax) * a.dim + c8);
+            }
+#pragma unroll
+            for (int n = 0; n < NV16; n++) {
+                const int i = tid + n * PWG, kp = i & 7, g = (i >> 3) % (HD / 8), ko = (i >> 3) / (HD / 8);
+                const int k = 16 * ko + 2 * kp, c8 = 8 * g;
+                vreg16[n][0] = *reinterpret_cast<const u32x4*>(P.Vh + base + (size_t)min(k, rmax) * a.dim + c8);
+                vreg16[n][1] = *reinterpret_cast<const u32x4*>(P.Vh + base + (size_t)min(k + 1, rmax) * a.dim + c8);
+            }
+            return;
+        }
         const int page = a.pageTable[seq * a.pagesPerSeq + t];
         const size_t base = ((size_t)page * MLH_KV_PAGE) * a.dim + h * HD;
-        const int rmax = maxPos - j0; // >= 0
 #pragma unroll
         for (int n = 0; n < NK; n++) {
             const int i = tid + n * PWG, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
@@ -374,25 +411,48 @@ __global__ void __launch_bounds__(PWG) k_pf_attn_mfma(PfArgs P, LayerDev L) {
         const int j0 = t << 6;
         const int rmax = maxPos - j0;
         __syncthreads(); // the previous tile has been consumed
+        if (H16) {
+            // ---- K tile: natural layout, sixteen bytes per store ----
+#pragma unroll
+            for (int n = 0; n < NK16; n++) {
+                const int i = tid + n * PWG, r = i / (HD / 8), c8 = (i % (HD / 8)) * 8;
+                *reinterpret_cast<u32x4*>(Kt + r * KP + c8) = r <= rmax ? kreg16[n] : (u32x4)(0u);
+            }
+            // ---- V tile: transposed, keys in contraction-slot order; a lane carries two keys that are neighbours there:
+            // for every column the halves of both keys go into one 32-bit word (v_perm picks the two 16-bit pieces) ----
+#pragma unroll
+            for (int n = 0; n < NV16; n++) {
+                const int i = tid + n * PWG, kp = i & 7, g = (i >> 3) % (HD / 8), ko = (i >> 3) / (HD / 8);
+                const int k = 16 * ko + 2 * kp, c8 = 8 * g;
+                const u32x4 v0 = k <= rmax ? vreg16[n][0] : (u32x4)(0u), v1 = k + 1 <= rmax ? vreg16[n][1] : (u32x4)(0u);
+                const int slot = pv_slot(k); // even, and pv_slot(k + 1) == slot + 1
+#pragma unroll
+                for (int w = 0; w < 4; w++) { // word w holds columns c8 + 2 w (low half) and c8 + 2 w + 1 (high half)
+                    *reinterpret_cast<uint32_t*>(Vt + (c8 + 2 * w + 0) * VP + slot) = __builtin_amdgcn_perm(v1[w], v0[w], 0x05040100u);
+                    *reinterpret_cast<uint32_t*>(Vt + (c8 + 2 * w + 1) * VP + slot) = __builtin_amdgcn_perm(v1[w], v0[w], 0x07060302u);
+                }
+            }
+        } else {
         // ---- K tile: natural layout ----
 #pragma unroll
-        for (int n = 0; n < NK; n++) {
-            const int i = tid + n * PWG, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
-            const f32x4 kk = r <= rmax ? kreg[n] : (f32x4)(0.f);
-            u32x2 w; w.x = pack_f16(kk.x, kk.y); w.y = pack_f16(kk.z, kk.w);
-            *reinterpret_cast<u32x2*>(Kt + r * KP + c4) = w;
-        }
-        // ---- V tile: transposed, keys in contraction-slot order; a lane carries two keys that are neighbours there ----
+            for (int n = 0; n < NK; n++) {
+                const int i = tid + n * PWG, r = i / (HD / 4), c4 = (i % (HD / 4)) * 4;
+                const f32x4 kk = r <= rmax ? kreg[n] : (f32x4)(0.f);
+                u32x2 w; w.x = pack_f16(kk.x, kk.y); w.y = pack_f16(kk.z, kk.w);
+                *reinterpret_cast<u32x2*>(Kt + r * KP + c4) = w;
+            }
+            // ---- V tile: transposed, keys in contraction-slot order; a lane carries two keys that are neighbours there ----
 #pragma unroll
-        for (int n = 0; n < NV; n++) {
-            const int i = tid + n * PWG, kp = i & 7, g = (i >> 3) % (HD / 4), ko = (i >> 3) / (HD / 4); // key pair, column chunk, group of 8 pairs
-            const int k = 16 * ko + 2 * kp, c4 = 4 * g;
-            const f32x4 v0 = k <= rmax ? vreg[n][0] : (f32x4)(0.f), v1 = k + 1 <= rmax ? vreg[n][1] : (f32x4)(0.f);
-            const int slot = pv_slot(k); // even, and pv_slot(k + 1) == slot + 1
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 0) * VP + slot) = pack_f16(v0.x, v1.x);
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 1) * VP + slot) = pack_f16(v0.y, v1.y);
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 2) * VP + slot) = pack_f16(v0.z, v1.z);
-            *reinterpret_cast<uint32_t*>(Vt + (c4 + 3) * VP + slot) = pack_f16(v0.w, v1.w);
+            for (int n = 0; n < NV; n++) {
+                const int i = tid + n * PWG, kp = i & 7, g = (i >> 3) % (HD / 4), ko = (i >> 3) / (HD / 4); // key pair, column chunk, group of 8 pairs
+                const int k = 16 * ko + 2 * kp, c4 = 4 * g;
+                const f32x4 v0 = k <= rmax ? vreg[n][0] : (f32x4)(0.f), v1 = k + 1 <= rmax ? vreg[n][1] : (f32x4)(0.f);
+                const int slot = pv_slot(k); // even, and pv_slot(k + 1) == slot + 1
+                *reinterpret_cast<uint32_t*>(Vt + (c4 + 0) * VP + slot) = pack_f16(v0.x, v1.x);
+                *reinterpret_cast<uint32_t*>(Vt + (c4 + 1) * VP + slot) = pack_f16(v0.y, v1.y);
+                *reinterpret_cast<uint32_t*>(Vt + (c4 + 2) * VP + slot) = pack_f16(v0.z, v1.z);
+                *reinterpret_cast<uint32_t*>(Vt + (c4 + 3) * VP + slot) = pack_f16(v0.w, v1.w);
+            }
         }
         __syncthreads();
         if (t + 1 < ntiles) fetch(t + 1);
@@ -1206,6 +1266,7 @@ static int ensure_prefill_buffers(mlh_ctx* c, int rows) {
         (rc = alloc((void**)&c->pfQKV, n * c->maxRowsA * 4)) || (rc = alloc(&c->pfA, n * (c->maxAd + hp.pleDim) * wb)) ||
         (rc = alloc((void**)&c->pfH1, n * hp.dim * 4)) ||
         (rc = alloc(&c->pfU, n * hp.ffnDim * wb)) ||
+        (hp.weightDtype == MLH_DTYPE_BF16 && ((rc = alloc((void**)&c->pfKh, n * hp.dim * 2)) || (rc = alloc((void**)&c->pfVh, n * hp.dim * 2)))) ||
         (rc = alloc((void**)&c->pfMeta, (3 * n + 4 * (size_t)hp.maxSeqs + 2 * (size_t)nblk + 2 * (size_t)nchunk + hp.maxSeqs) * 4)))
         return rc;
     c->pfRows = rows;
@@ -1285,6 +1346,10 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
     P.blkSeg = d_blk; P.blkQ0 = d_blk + c->pfBlkCap;
     P.X = c->pfX; P.Xn = c->pfXn; P.QKV = c->pfQKV; P.qkvLd = c->maxRowsA; P.Amix = c->pfA; P.aLd = c->maxAd + hp.pleDim;
     P.H1 = c->pfH1; P.U = c->pfU;
+    bool fresh = true; // every segment starts its sequence: all keys of the call are rows of the call
+    for (int s = 0; s < nseg; s++) fresh = fresh && segPos0[s] == 0;
+    P.Kh = mfmaAttn && fresh ? c->pfKh : nullptr;
+    P.Vh = mfmaAttn && fresh ? c->pfVh : nullptr;
     const int d_ = hp.dim, F = hp.ffnDim, dt = c->gemmDtype;
 #define GEMM(A, lda, B, alpha, ldb, C, ldc, R, ldr, M, N, K)                                                \
     do {                                                                                                    \
@@ -1302,11 +1367,13 @@ int mlh_run_prefill_gemm(mlh_ctx* c, int nseg, const int32_t* seqs, const int32_
         if (L.kind == MLH_KIND_ATTENTION) {
             if (hp.headDim == 64) {
                 hipLaunchKernelGGL((k_pf_qk_rope_kv<64>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
-                if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<64>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
+                if (mfmaAttn && P.Kh) hipLaunchKernelGGL((k_pf_attn_mfma<64, true>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
+                else if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<64, false>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
                 else hipLaunchKernelGGL((k_pf_attn<64, float>), dim3(hp.attnHeads, nblk), dim3(PWG), (size_t)(2 * 64 * 68 + PF_QB * 64) * 4, st, P, L);
             } else {
                 hipLaunchKernelGGL((k_pf_qk_rope_kv<128>), dim3(hp.attnHeads, n), dim3(64), 0, st, P, L);
-                if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<128>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
+                if (mfmaAttn && P.Kh) hipLaunchKernelGGL((k_pf_attn_mfma<128, true>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
+                else if (mfmaAttn) hipLaunchKernelGGL((k_pf_attn_mfma<128, false>), dim3(hp.attnHeads, nblk), dim3(PWG), 0, st, P, L);
                 else hipLaunchKernelGGL((k_pf_attn<128, float>), dim3(hp.attnHeads, nblk), dim3(PWG), (size_t)(2 * 64 * 132 + PF_QB * 128) * 4, st, P, L);
             }
         } else {

@@ -159,6 +159,7 @@ struct mlh_ctx {
     std::vector<void*> pfAllocs;
     float *pfX = nullptr, *pfQKV = nullptr, *pfH1 = nullptr;
     void *pfXn = nullptr, *pfA = nullptr, *pfU = nullptr;
+    uint16_t *pfKh = nullptr, *pfVh = nullptr; // half copies of a call's K and V rows for the MFMA attention of a fresh prefill
     int* pfMeta = nullptr;
     int pfChunkCap = 0;
     void* pfGdnWs = nullptr;   // chunk operands of the chunk-parallel GDN prefill
