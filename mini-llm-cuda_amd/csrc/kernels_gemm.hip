@@ -648,10 +648,27 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
                 const bool vec = ((ldc & 3) == 0) && (!R || (ldr & 3) == 0) && (((unsigned long long)Cv & 15) == 0) && (((unsigned long long)R & 15) == 0);
                 const bool inside = vec && mW + 128 <= M && nW + 128 <= N; // the wave's whole 128 x 128 lies inside C: no per-element tests
                 const unsigned wr = patch + r16 * GW_EP + kq * 16;
+                // The residual of the interior path is fetched GW_RPF iterations ahead: an iteration is two stores' worth of
+                // time and a load's latency is several of those, so waited for on the spot (32 times per tile) it would cost
+                // more than the stores themselves.
+                constexpr int GW_RPF = 6;
+                f32x4 rpre[GW_RPF][2];
+                const bool resid = inside && R != nullptr;
+                auto rfetch = [&](int it, int slot) { // iteration it = 4 bm + bp
+                    const int bm = it >> 2, bp = it & 3;
+                    const float* rp = R + (size_t)(mW + bm * 16 + (lane >> 3)) * ldr + nW + bp * 32 + (lane & 7) * 4;
+#pragma unroll
+                    for (int k2 = 0; k2 < 2; k2++) rpre[slot][k2] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(rp + (size_t)(8 * k2) * ldr));
+                };
+                if (resid) {
+#pragma unroll
+                    for (int it = 0; it < GW_RPF; it++) rfetch(it, it);
+                }
 #pragma unroll
                 for (int bm = 0; bm < 8; bm++)
 #pragma unroll
                     for (int bp = 0; bp < 4; bp++) { // two column blocks side by side: 32 columns = one 128-byte line per row
+                        const int it = 4 * bm + bp;
                         *(lds_f32x4*)(wr) = acc[bm][2 * bp] * alpha;
                         *(lds_f32x4*)(wr + 64) = acc[bm][2 * bp + 1] * alpha;
                         const int rowb = mW + bm * 16 + (lane >> 3), col = nW + bp * 32 + (lane & 7) * 4;
@@ -660,10 +677,10 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
                         for (int k = 0; k < 2; k++) v[k] = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
                         if (inside) {
                             float* cp = (float*)Cv + (size_t)rowb * ldc + col;
-                            if (R) {
-                                const float* rp = R + (size_t)rowb * ldr + col;
+                            if (resid) {
 #pragma unroll
-                                for (int k = 0; k < 2; k++) v[k] += __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(rp + (size_t)(8 * k) * ldr));
+                                for (int k = 0; k < 2; k++) v[k] += rpre[it % GW_RPF][k];
+                                if (it + GW_RPF < 32) rfetch(it + GW_RPF, it % GW_RPF);
                             }
                             // (streaming stores: the output is far larger than the caches and is read by a later kernel,
                             // keeping it out of the L2 leaves the operand panels there and drains 5-8 % faster)
