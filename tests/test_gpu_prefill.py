@@ -220,6 +220,42 @@ def test_prefill_bf16(pkg, orc, kind, plen):
     dev.close()
 
 
+@pytest.mark.parametrize("kind", ["attn_flags", "hd128"])
+def test_prefill_bf16_ragged_batch_both_attention_variants(pkg, orc, kind):
+    """bf16 weights, several sequences of different lengths in one pass.  A call whose segments all start at position 0
+    runs the attention on the half copies of K and V that the RoPE kernel writes (keys = rows of the call); a prompt
+    appended in two calls reads the fp32 pages instead.  Both against the float64 oracle, the batch also against each
+    sequence prefilled alone (other row offsets, and for the short ones other GEMM tile families)."""
+    extra = {"maxL": 200} if kind == "attn_flags" else {}
+    hp = small_cfg(pkg, kind, weightDtype=pkg.DTYPE_BF16, maxSeqs=5, **extra)
+    model, dev, w = make(pkg, orc, hp, seed=41, bf16=True)
+    lens = [37, 128, 1, 199, 65]
+    seqs = [3, 0, 4, 1, 2]
+    prompts = [pkg.random_tokens(300 + i, 0, hp.vocabSize, n) for i, n in enumerate(lens)]
+    wants = [orc.forward_full(w, p, "f64", last_only=True)["logits"][-1] for p in prompts]
+    dev.prefill_batch(seqs, prompts)
+    batch = {s: dev.logits(s).copy() for s in seqs}
+    for s, p, want in zip(seqs, prompts, wants):
+        err = float(np.max(np.abs(batch[s] - want)) / np.max(np.abs(want)))
+        assert err <= 4e-3 <= BF16_RTOL, ("batch", s, len(p), err)
+    dev.reset()
+    for s, p, want in zip(seqs, prompts, wants):  # alone
+        dev.prefill(s, p)
+        assert float(np.max(np.abs(dev.logits(s) - want)) / np.max(np.abs(want))) <= 4e-3, ("alone", s, len(p))
+        assert float(np.max(np.abs(dev.logits(s) - batch[s])) / np.max(np.abs(want))) <= 4e-3, ("alone vs batch", s, len(p))
+    dev.reset()
+    for s, p, want in zip(seqs, prompts, wants):  # in two calls: the second one's keys start in the pages
+        if len(p) < 40:
+            continue
+        cut = len(p) // 2 + 3
+        dev.prefill(s, p[:cut])
+        dev.prefill(s, p[cut:])
+        err = float(np.max(np.abs(dev.logits(s) - want)) / np.max(np.abs(want)))
+        assert err <= 4e-3, ("pieces", s, len(p), err)
+        assert float(np.max(np.abs(dev.logits(s) - batch[s])) / np.max(np.abs(want))) <= 4e-3
+    dev.close()
+
+
 # ---- batched decode through the skinny GEMM ------------------------------------------------------
 @pytest.mark.parametrize("kind,nseq,graph", [("hybrid", 8, 0), ("hybrid_flags", 13, 1), ("attn_long", 33, 0), ("hd128", 64, 2)])
 def test_batched_decode_gemm_path(pkg, orc, kind, nseq, graph):
