@@ -251,48 +251,50 @@ def prefill_leg(m, reps=REPS):
 
 def gemm_leg(m, iters=3, reps=1):
     """The gate/up product of one config-5 prefill pass alone (16384 x 11264 x 2048, half operands -- what the bf16
-    model's MFMA path multiplies --, plain epilogue, N(0,1) data): mean launch time over `iters` back-to-back
-    launches from HIP events, median of `reps` such runs.  Also the launch the operand-path counters of the big GEMM
-    kernel are collected on."""
+    model's MFMA path multiplies --, N(0,1) data), timed with HIP events.  The headline figure is the product as the pass
+    runs it: SiLU(gate) * up in the epilogue, half output, one launch at a time with the device idle in between (in the
+    pass a GEMM is followed by lighter kernels, not by nine more GEMMs, and under real operand data the part's clock
+    depends on how long the load has lasted).  Beside it: the same launch ten times back to back, the plain fp32 epilogue
+    back to back, the kernel on all-zero operands and the vendor library on the same operands.  With reps == 1 (profiler
+    and counter runs) both epilogues are launched `iters` times and only the plain timing is reported."""
     hp = m.config(5)
     M = 8 * 2048
     rng = np.random.default_rng(5)
     a = rng.standard_normal((M, hp.dim), dtype=np.float32)
     b = rng.standard_normal((2 * hp.ffnDim, hp.dim), dtype=np.float32)
-    if reps == 1:  # profiler runs: the product once more with the epilogue the pass uses
-        m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)
-    runs = [m.selftest_gemm(a, b, None, f16=True, iters=iters)[1] for _ in range(reps)]
-    us = stats(runs)["median"]
     flop = 2.0 * M * 2 * hp.ffnDim * hp.dim
-    tf = flop / us / 1e6
-    out = {"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "epilogue": "plain, fp32 output", "avg_us": us, "avg_us_stats": stats(runs),
-           "TFLOPs": tf, "frac_of_bf16_peak": tf * 1e12 / MFMA_BF16_PEAK}
-    if reps > 1:  # the same product as the prefill pass itself runs it: SiLU(gate) * up in the epilogue, half output
-        sruns = [m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)[1] for _ in range(reps)]
-        su = stats(sruns)["median"]
-        out["as_in_the_pass_swiglu_epilogue"] = {"avg_us": su, "avg_us_stats": stats(sruns), "TFLOPs": flop / su / 1e6,
-                                                 "frac_of_bf16_peak": flop / su / 1e6 * 1e12 / MFMA_BF16_PEAK}
-        # One launch at a time with the device idle in between: in the prefill pass a GEMM is followed by lighter kernels,
-        # not by nine more GEMMs, and the part's clock under real operand data depends on how long the load has lasted.
-        singles = []
-        for _ in range(7):
-            time.sleep(0.05)
-            singles.append(m.selftest_gemm(a, b, None, f16=True, iters=1, swiglu=True)[1])
-        s1 = stats(singles)["median"]
-        out["single_launch_swiglu_epilogue"] = {"avg_us": s1, "avg_us_stats": stats(singles), "TFLOPs": flop / s1 / 1e6,
-                                                "frac_of_bf16_peak": flop / s1 / 1e6 * 1e12 / MFMA_BF16_PEAK}
-    if reps > 1:
-        # Two yardsticks on the same box in the same run, neither on the product path: the same kernel on all-zero
-        # operands (no switching activity: what the code alone allows, without the part's power management), and the
-        # vendor library's GEMM (torch.matmul -> hipBLASLt) on the same shape, type and data distribution.
-        z = np.zeros_like(a), np.zeros_like(b)
-        uz = stats([m.selftest_gemm(z[0], z[1], None, f16=True, iters=iters)[1] for _ in range(3)])["median"]
-        out["same_kernel_zero_operands"] = {"avg_us": uz, "TFLOPs": flop / uz / 1e6}
-        try:
-            out["vendor_library_yardstick"] = vendor_gemm(a, b, iters, reps, flop)
-            out["ratio_to_vendor_library"] = out["vendor_library_yardstick"]["avg_us"] / us
-        except Exception as e:  # a yardstick, never required
-            out["vendor_library_yardstick"] = {"failed": repr(e)}
+
+    def fig(us_list):
+        us = stats(us_list)["median"]
+        return {"avg_us": us, "avg_us_stats": stats(us_list), "TFLOPs": flop / us / 1e6, "frac_of_bf16_peak": flop / us / 1e6 * 1e12 / MFMA_BF16_PEAK}
+
+    if reps == 1:
+        m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)
+        out = fig([m.selftest_gemm(a, b, None, f16=True, iters=iters)[1]])
+        out.update({"shape": [M, 2 * hp.ffnDim, hp.dim], "iters": iters, "epilogue": "plain, fp32 output"})
+        return out
+    m.selftest_gemm(a, b, None, f16=True, iters=2, swiglu=True)  # warm
+    singles = []
+    for _ in range(9):
+        time.sleep(0.05)
+        singles.append(m.selftest_gemm(a, b, None, f16=True, iters=1, swiglu=True)[1])
+    out = fig(singles)
+    out.update({"shape": [M, 2 * hp.ffnDim, hp.dim], "epilogue": "SiLU(gate) * up, half output (as the prefill pass runs this product)",
+                "protocol": "median of 9 single launches, 50 ms idle before each, HIP events around the launch"})
+    out["back_to_back_%d_launches_swiglu_epilogue" % iters] = fig([m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)[1] for _ in range(reps)])
+    plain = fig([m.selftest_gemm(a, b, None, f16=True, iters=iters)[1] for _ in range(reps)])
+    out["back_to_back_%d_launches_plain_fp32_epilogue" % iters] = plain
+    # Two yardsticks on the same box in the same run, neither on the product path: the same kernel on all-zero
+    # operands (no switching activity: what the code alone allows, without the part's power management), and the
+    # vendor library's GEMM (torch.matmul -> hipBLASLt) on the same shape, type and data distribution.
+    z = np.zeros_like(a), np.zeros_like(b)
+    uz = stats([m.selftest_gemm(z[0], z[1], None, f16=True, iters=iters)[1] for _ in range(3)])["median"]
+    out["same_kernel_zero_operands_plain_epilogue"] = {"avg_us": uz, "TFLOPs": flop / uz / 1e6}
+    try:
+        out["vendor_library_yardstick"] = vendor_gemm(a, b, iters, reps, flop)
+        out["back_to_back_ratio_to_vendor_library"] = out["vendor_library_yardstick"]["avg_us"] / out["back_to_back_%d_launches_swiglu_epilogue" % iters]["avg_us"]
+    except Exception as e:  # a yardstick, never required
+        out["vendor_library_yardstick"] = {"failed": repr(e)}
     return out
 
 
