@@ -710,7 +710,7 @@ template <int DK> struct GdLayout { // one chunk's operand image (bytes), rows p
 __device__ __forceinline__ uint16_t f16_bits(float v) { return __builtin_bit_cast(uint16_t, (_Float16)v); }
 
 template <int DK>
-__global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const int* __restrict__ chunkSeg, const int* __restrict__ chunkT0,
+__global__ void __launch_bounds__(2 * DK, 2) k_gdn_prep(PfArgs P, LayerDev L, const int* __restrict__ chunkSeg, const int* __restrict__ chunkT0,
                                                       unsigned char* __restrict__ ws, float* __restrict__ gCexp) {
     constexpr int DV = DK, NT = 2 * DK;
     typedef GdLayout<DK> Lay;
@@ -830,18 +830,92 @@ __global__ void __launch_bounds__(2 * DK) k_gdn_prep(PfArgs P, LayerDev L, const
 #pragma unroll
         for (int t = 0; t < GD_C; t++) X[t] = beta[t] * eg[t] * colv[t];
     }
-#pragma unroll
-    for (int t = 1; t < GD_C; t++) {
-        float acc0 = X[t], acc1 = 0.f, acc2 = 0.f, acc3 = 0.f; // four chains: the row's dot product is on the serial path
-#pragma unroll
-        for (int i4 = 0; i4 < t; i4 += 4) {
-            const f32x4 a4 = *reinterpret_cast<const f32x4*>(Am + t * GD_C + i4); // zero at and beyond the diagonal
-            acc0 = fmaf(-a4.x, X[i4], acc0);
-            if (i4 + 1 < t) acc1 = fmaf(-a4.y, X[i4 + 1], acc1);
-            if (i4 + 2 < t) acc2 = fmaf(-a4.z, X[i4 + 2], acc2);
-            if (i4 + 3 < t) acc3 = fmaf(-a4.w, X[i4 + 3], acc3);
+    // Blocked forward substitution.  The 64 rows go in four blocks of 16: inside a block a thread solves its column in
+    // fp32 as before (the block's own triangle, 120 multiply-adds); what the solved block contributes to all later rows,
+    // A[later rows, block] X[block], is a matrix product and runs on the MFMA units with half operands -- a wave takes
+    // its own 64 columns (two column tiles), so nothing here needs a workgroup barrier: LDS instructions of a wave
+    // execute in order.  Per wave 8 MFMAs replace three quarters of the 2016 multiply-adds a thread had on its chain.
+    {
+        constexpr int AHP = GD_C + 8;                       // pitch of the half copy of A (elements): 16-byte reads, rows 4 banks apart
+        uint16_t* Ah = k16;                                 // [64][AHP]; k16 / q16 are free: their MFMAs are done (barrier above)
+        unsigned char* wsc = reinterpret_cast<unsigned char*>(Ah + GD_C * AHP) + wave * (64 * 80); // this wave's exchange area
+        // X of the solved block as halves, [column][16] with pitch 48 bytes (B operand); the update of the next block's
+        // rows, [column][16] floats with pitch 80 bytes -- both conflict-free for 16-byte accesses, and they may share
+        // the area: the MFMAs have read the one before the other is written (same wave, in order)
+        for (int i = tid; i < GD_C * GD_C / 2; i += NT) { // half copy of A, two elements per thread and trip
+            const int t = i / (GD_C / 2), i2 = (i % (GD_C / 2)) * 2;
+            *reinterpret_cast<uint32_t*>(Ah + t * AHP + i2) = pack_f16(Am[t * GD_C + i2], Am[t * GD_C + i2 + 1]);
         }
-        X[t] = (acc0 + acc1) + (acc2 + acc3);
+        __syncthreads();
+        const int n32 = lane & 31, half = lane >> 5;
+        f32x16 upd[2]; // [column tile of the wave]: what the solved blocks contribute to rows 32 .. 63
+#pragma unroll
+        for (int ct = 0; ct < 2; ct++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) upd[ct][e] = 0.f;
+        auto hand_over = [&](const f32x16& u, int ct, int e0) { // elements e0 .. e0 + 7 = 16 rows of a tile, to the owners of the columns
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                f32x4 v;
+                v.x = u[e0 + 4 * j]; v.y = u[e0 + 4 * j + 1]; v.z = u[e0 + 4 * j + 2]; v.w = u[e0 + 4 * j + 3];
+                *reinterpret_cast<f32x4*>(wsc + (32 * ct + n32) * 80 + (8 * j + 4 * half) * 4) = v; // rows 8 j + 4 half + 0..3 of the block
+            }
+        };
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            if (b > 1) { // rows 16 b .. 16 b + 15: elements 8 (b & 1) .. + 7 of the tile of rows 32 .. 63 (block 1's were handed over by block 0)
+                hand_over(upd[0], 0, 8 * (b & 1));
+                hand_over(upd[1], 1, 8 * (b & 1));
+            }
+            if (b > 0) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const f32x4 u = *reinterpret_cast<const f32x4*>(wsc + lane * 80 + q * 16);
+                    X[16 * b + 4 * q] -= u.x; X[16 * b + 4 * q + 1] -= u.y; X[16 * b + 4 * q + 2] -= u.z; X[16 * b + 4 * q + 3] -= u.w;
+                }
+            }
+#pragma unroll
+            for (int tt = 1; tt < 16; tt++) { // the block's own triangle
+                const int t = 16 * b + tt;
+                float acc0 = X[t], acc1 = 0.f, acc2 = 0.f, acc3 = 0.f; // four chains: the row's dot product is on the serial path
+#pragma unroll
+                for (int i4 = 0; i4 < tt; i4 += 4) {
+                    const f32x4 a4 = *reinterpret_cast<const f32x4*>(Am + t * GD_C + 16 * b + i4); // zero at and beyond the diagonal
+                    acc0 = fmaf(-a4.x, X[16 * b + i4], acc0);
+                    if (i4 + 1 < tt) acc1 = fmaf(-a4.y, X[16 * b + i4 + 1], acc1);
+                    if (i4 + 2 < tt) acc2 = fmaf(-a4.z, X[16 * b + i4 + 2], acc2);
+                    if (i4 + 3 < tt) acc3 = fmaf(-a4.w, X[16 * b + i4 + 3], acc3);
+                }
+                X[t] = (acc0 + acc1) + (acc2 + acc3);
+            }
+            if (b < 3) { // publish the block as halves and add its contribution to the later rows
+                u32x4 w0, w1;
+                w0.x = pack_f16(X[16 * b + 0], X[16 * b + 1]); w0.y = pack_f16(X[16 * b + 2], X[16 * b + 3]);
+                w0.z = pack_f16(X[16 * b + 4], X[16 * b + 5]); w0.w = pack_f16(X[16 * b + 6], X[16 * b + 7]);
+                w1.x = pack_f16(X[16 * b + 8], X[16 * b + 9]); w1.y = pack_f16(X[16 * b + 10], X[16 * b + 11]);
+                w1.z = pack_f16(X[16 * b + 12], X[16 * b + 13]); w1.w = pack_f16(X[16 * b + 14], X[16 * b + 15]);
+                *reinterpret_cast<u32x4*>(wsc + lane * 48) = w0;
+                *reinterpret_cast<u32x4*>(wsc + lane * 48 + 16) = w1;
+                u32x4 xop[2];
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++) xop[ct] = *reinterpret_cast<const u32x4*>(wsc + (32 * ct + n32) * 48 + 16 * half);
+                const u32x4 aop1 = *reinterpret_cast<const u32x4*>(Ah + (32 + n32) * AHP + 16 * b + 8 * half);
+#pragma unroll
+                for (int ct = 0; ct < 2; ct++)
+                    upd[ct] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, aop1), __builtin_bit_cast(f16x8, xop[ct]), upd[ct], 0, 0, 0);
+                if (b == 0) { // rows 16 .. 31 are fed by block 0 alone: their tile lives only until it is handed over
+                    const u32x4 aop0 = *reinterpret_cast<const u32x4*>(Ah + n32 * AHP + 8 * half);
+#pragma unroll
+                    for (int ct = 0; ct < 2; ct++) {
+                        f32x16 u0;
+#pragma unroll
+                        for (int e = 0; e < 16; e++) u0[e] = 0.f;
+                        u0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, aop0), __builtin_bit_cast(f16x8, xop[ct]), u0, 0, 0, 0);
+                        hand_over(u0, ct, 8); // (the exchange area is free: both column tiles' operands are in registers)
+                    }
+                }
+            }
+        }
     }
     const float gC = g[GD_C - 1];
     const int sl = slot_of(col);
