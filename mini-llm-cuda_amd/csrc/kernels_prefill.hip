@@ -342,13 +342,15 @@ __global__ void __launch_bounds__(PWG, H16 ? 2 : 1) k_pf_attn_mfma(PfArgs P, Lay
     const int maxPos = pos0 + min(q0 + PF_MQB, len) - 1;
     const bool waveActive = q0 + wave * 32 < len;
 
-    // Q^T operand (fp16): for step s the lane holds q[16 s + 8 half .. +7] of its query
+    // Q^T operand (fp16): for step s the lane holds q[16 s + 8 half .. +7] of its query, times log2(e) / sqrt(HD): the
+    // scores come out of the MFMA ready for exp2
     u32x4 qop[KS];
     {
         const float* q = P.QKV + (size_t)qrow * P.qkvLd + h * HD + 8 * half;
+        const float qs = 1.44269504088896341f / sqrtf((float)HD);
 #pragma unroll
         for (int s = 0; s < KS; s++) {
-            const f32x4 lo = *reinterpret_cast<const f32x4*>(q + 16 * s), hi = *reinterpret_cast<const f32x4*>(q + 16 * s + 4);
+            const f32x4 lo = *reinterpret_cast<const f32x4*>(q + 16 * s) * qs, hi = *reinterpret_cast<const f32x4*>(q + 16 * s + 4) * qs;
             qop[s].x = pack_f16(lo.x, lo.y); qop[s].y = pack_f16(lo.z, lo.w);
             qop[s].z = pack_f16(hi.x, hi.y); qop[s].w = pack_f16(hi.z, hi.w);
         }
@@ -359,7 +361,7 @@ __global__ void __launch_bounds__(PWG, H16 ? 2 : 1) k_pf_attn_mfma(PfArgs P, Lay
 #pragma unroll
         for (int i = 0; i < 16; i++) oacc[b][i] = 0.f;
     float m_run = -1.0e30f, l_run = 0.f;
-    const float inv_scale = 1.0f / sqrtf((float)HD);
+    const int waveMinPos = pos0 + q0 + wave * 32; // the lowest query position of the wave
     const int ntiles = (maxPos >> 6) + 1;
 
     // A tile's K and V rows travel global -> registers -> LDS; the loads of tile t + 1 are issued before tile t is
@@ -469,36 +471,60 @@ __global__ void __launch_bounds__(PWG, H16 ? 2 : 1) k_pf_attn_mfma(PfArgs P, Lay
                 sacc[b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, kop), __builtin_bit_cast(f16x8, qop[s]), sacc[b], 0, 0, 0);
             }
         }
-        // ---- scale, causal mask, online softmax down the key axis ----
+        // ---- causal mask, online softmax down the key axis (base 2: the scores carry log2(e) / sqrt(HD)) ----
+        // A tile that lies entirely at or below the wave's lowest query position needs no mask (all but the last one or
+        // two tiles of a wave), and the output is only rescaled when some query's running maximum moved.
         float mx = -1.0e30f;
+        const bool fullTile = j0 + 63 <= waveMinPos; // wave-uniform
+        if (fullTile) {
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+            for (int b = 0; b < 2; b++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int key = j0 + 32 * b + 8 * (i >> 2) + 4 * half + (i & 3);
-                const float sv = key <= qpos ? sacc[b][i] * inv_scale : -1.0e30f;
-                sacc[b][i] = sv;
-                mx = fmaxf(mx, sv);
-            }
+                for (int i = 0; i < 16; i += 2) mx = fmaxf(mx, fmaxf(sacc[b][i], sacc[b][i + 1]));
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int key = j0 + 32 * b + 8 * (i >> 2) + 4 * half + (i & 3);
+                    const float sv = key <= qpos ? sacc[b][i] : -1.0e30f;
+                    sacc[b][i] = sv;
+                    mx = fmaxf(mx, sv);
+                }
+        }
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float mn = fmaxf(m_run, mx);
-        const float corr = __expf(m_run - mn);
         float ls = 0.f;
+        if (fullTile) {
 #pragma unroll
-        for (int b = 0; b < 2; b++)
+            for (int b = 0; b < 2; b++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float pv = sacc[b][i] > -1.0e29f ? __expf(sacc[b][i] - mn) : 0.f;
-                sacc[b][i] = pv;
-                ls += pv;
-            }
+                for (int i = 0; i < 16; i++) {
+                    const float pv = __builtin_amdgcn_exp2f(sacc[b][i] - mn);
+                    sacc[b][i] = pv;
+                    ls += pv;
+                }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const float pv = sacc[b][i] > -1.0e29f ? __builtin_amdgcn_exp2f(sacc[b][i] - mn) : 0.f;
+                    sacc[b][i] = pv;
+                    ls += pv;
+                }
+        }
         ls += __shfl_xor(ls, 32, 64);
-        l_run = l_run * corr + ls;
+        if (__any(mn > m_run)) { // wave-uniform
+            const float corr = __builtin_amdgcn_exp2f(m_run - mn);
+            l_run *= corr;
+#pragma unroll
+            for (int b = 0; b < MB; b++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) oacc[b][i] *= corr;
+        }
+        l_run += ls;
         m_run = mn;
-#pragma unroll
-        for (int b = 0; b < MB; b++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) oacc[b][i] *= corr;
         // ---- O^T += V^T . P^T ----
 #pragma unroll
         for (int st = 0; st < 4; st++) {
