@@ -461,40 +461,23 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
 }
 
 // ----------------------------------------------------------------------------
-// gated-delta-net state update, one head's state per workgroup:
+// gated-delta-net state update, one head's state per RS workgroups (rows of the state are independent):
 //   q,k L2-normalised; alpha = exp(-softplus(za + ba)); beta = sigmoid(zb + bb)
 //   u = S k ; S <- alpha (S - beta u k^T) + beta v k^T ; o = S q
-// S is [DV, DK] row-major, held in registers for the step.
+// S is [DV, DK] row-major, held in registers for the step; workgroup z of a head takes rows [z DV/RS, (z+1) DV/RS).
+// The normalised q and k are formed once per workgroup in LDS.
 // ----------------------------------------------------------------------------
-template <int DK, int DV>
+template <int DK, int DV, int RS>
 __global__ void __launch_bounds__(WG) k_gdn(StepArgs a, LayerDev L) {
-    constexpr int TPR = WG / DV;  // threads per state row
-    constexpr int CPT = DK / TPR; // columns per thread
-    static_assert(TPR >= 1 && (TPR & (TPR - 1)) == 0 && CPT % 4 == 0, "unsupported GDN shape");
-    __shared__ float qs[DK], ks[DK];
+    constexpr int TPR = WG * RS / DV; // threads per state row
+    constexpr int CPT = DK / TPR;     // columns per thread
+    static_assert(TPR >= 1 && TPR <= 64 && (TPR & (TPR - 1)) == 0 && CPT % 4 == 0 && DK % 64 == 0, "unsupported GDN shape");
+    __shared__ float qn[DK], kn[DK];
     const int h = blockIdx.x, slot = blockIdx.y, tid = threadIdx.x;
     const int seq = a.sidx[slot];
     const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
-    for (int i = tid; i < DK; i += WG) {
-        qs[i] = qkv[h * DK + i];
-        ks[i] = qkv[L.offK + h * DK + i];
-    }
-    __syncthreads();
-    float sq = 0.f, sk = 0.f;
-#pragma unroll 8
-    for (int i = 0; i < DK; i++) {
-        sq = fmaf(qs[i], qs[i], sq);
-        sk = fmaf(ks[i], ks[i], sk);
-    }
-    const float rq = sqrtf(sq + 1e-6f), rk = sqrtf(sk + 1e-6f);
-    const float za = qkv[L.offGa + h] + L.gdnBa[h];
-    const float zb = qkv[L.offGb + h] + L.gdnBb[h];
-    const float sp = fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)));
-    const float alpha = expf(-sp);
-    const float beta = sigmoidf_ref(zb);
-
-    const int r = tid / TPR, cg = tid % TPR, c0 = cg * CPT;
-    const float vr = qkv[L.offV + h * DV + r];
+    const int r = (int)blockIdx.z * (DV / RS) + tid / TPR, cg = tid % TPR, c0 = cg * CPT;
+    // the state row's loads go out first: nothing below depends on them until the products
     float* Srow = L.S + (((size_t)seq * a.gdnHeads + h) * DV + r) * DK + c0;
     float S[CPT];
 #pragma unroll
@@ -502,17 +485,44 @@ __global__ void __launch_bounds__(WG) k_gdn(StepArgs a, LayerDev L) {
         float4 t = *reinterpret_cast<const float4*>(Srow + c);
         S[c] = t.x; S[c + 1] = t.y; S[c + 2] = t.z; S[c + 3] = t.w;
     }
+    const float vr = qkv[L.offV + h * DV + r];
+    float qv[DK / 64], kv[DK / 64];
+    if (tid < 64) { // wave 0: the two norms
+        float sq = 0.f, sk = 0.f;
+#pragma unroll
+        for (int i = 0; i < DK / 64; i++) {
+            qv[i] = qkv[h * DK + tid + 64 * i];
+            kv[i] = qkv[L.offK + h * DK + tid + 64 * i];
+            sq = fmaf(qv[i], qv[i], sq);
+            sk = fmaf(kv[i], kv[i], sk);
+        }
+        sq = wave_sum(sq);
+        sk = wave_sum(sk);
+        const float rq = sqrtf(sq + 1e-6f), rk = sqrtf(sk + 1e-6f);
+#pragma unroll
+        for (int i = 0; i < DK / 64; i++) {
+            qn[tid + 64 * i] = qv[i] / rq;
+            kn[tid + 64 * i] = kv[i] / rk;
+        }
+    }
+    const float za = qkv[L.offGa + h] + L.gdnBa[h];
+    const float zb = qkv[L.offGb + h] + L.gdnBb[h];
+    const float sp = fmaxf(za, 0.f) + log1pf(expf(-fabsf(za)));
+    const float alpha = expf(-sp);
+    const float beta = sigmoidf_ref(zb);
+    __syncthreads();
+
     float u = 0.f;
 #pragma unroll
-    for (int c = 0; c < CPT; c++) u = fmaf(S[c], ks[c0 + c] / rk, u);
+    for (int c = 0; c < CPT; c++) u = fmaf(S[c], kn[c0 + c], u);
 #pragma unroll
     for (int o = TPR / 2; o > 0; o >>= 1) u += __shfl_xor(u, o, MLH_WAVE);
     float oacc = 0.f;
 #pragma unroll
     for (int c = 0; c < CPT; c++) {
-        const float kn = ks[c0 + c] / rk;
-        S[c] = alpha * (S[c] - beta * u * kn) + beta * vr * kn;
-        oacc = fmaf(S[c], qs[c0 + c] / rq, oacc);
+        const float k1 = kn[c0 + c];
+        S[c] = alpha * (S[c] - beta * u * k1) + beta * vr * k1;
+        oacc = fmaf(S[c], qn[c0 + c], oacc);
     }
 #pragma unroll
     for (int o = TPR / 2; o > 0; o >>= 1) oacc += __shfl_xor(oacc, o, MLH_WAVE);
@@ -531,7 +541,7 @@ __global__ void __launch_bounds__(WG) k_gdn(StepArgs a, LayerDev L) {
         else ((float*)a.mixRows)[row + col] = v;
     };
     if (cg == 0) put_row((size_t)h * DV + r, oacc);
-    if (h == 0)
+    if (h == 0 && blockIdx.z == 0)
         for (int j = tid; j < a.ple; j += WG) {
             const size_t e = (size_t)a.tok[slot] * a.ple + j;
             const float p = a.wbytes == 2 ? __uint_as_float(((uint32_t)((const uint16_t*)L.pleTable)[e]) << 16) : ((const float*)L.pleTable)[e];
@@ -948,10 +958,15 @@ static int launch_mix(mlh_ctx* c, const StepArgs& a, const LayerDev& L) {
             return -1;
         }
     } else {
-        if (a.gdnDk == 64 && a.gdnDv == 64)
-            hipLaunchKernelGGL((k_gdn<64, 64>), dim3(a.gdnHeads, a.nseq), dim3(WG), 0, st, a, L);
-        else if (a.gdnDk == 128 && a.gdnDv == 128)
-            hipLaunchKernelGGL((k_gdn<128, 128>), dim3(a.gdnHeads, a.nseq), dim3(WG), 0, st, a, L);
+        // few (head, sequence) pairs: a head's rows are split over four workgroups so that every compute unit has work
+        const bool split = a.gdnHeads * a.nseq <= 256;
+        if (a.gdnDk == 64 && a.gdnDv == 64) {
+            if (split) hipLaunchKernelGGL((k_gdn<64, 64, 4>), dim3(a.gdnHeads, a.nseq, 4), dim3(WG), 0, st, a, L);
+            else hipLaunchKernelGGL((k_gdn<64, 64, 1>), dim3(a.gdnHeads, a.nseq), dim3(WG), 0, st, a, L);
+        } else if (a.gdnDk == 128 && a.gdnDv == 128) {
+            if (split) hipLaunchKernelGGL((k_gdn<128, 128, 4>), dim3(a.gdnHeads, a.nseq, 4), dim3(WG), 0, st, a, L);
+            else hipLaunchKernelGGL((k_gdn<128, 128, 1>), dim3(a.gdnHeads, a.nseq), dim3(WG), 0, st, a, L);
+        }
         else {
             c->err = "GDN kernel supports dk = dv = 64 or 128";
             return -1;
