@@ -445,6 +445,34 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
     float M = -1.0e30f;
 #pragma unroll
     for (int w = 0; w < NW; w++) M = fmaxf(M, comb[w * (HD + 2) + HD]);
+    if (a.mixRows && a.nsplit == 1) {
+        // batched step, one workgroup per (head, sequence): the finished mixing output (inference.cu:549-573), gated
+        // (inference.cu:241-250), goes straight into the output-projection GEMM's input row; the workgroup of head 0
+        // appends the PLE columns e = silu(gate) * P[tok]
+        float l = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; w++) l += expf(comb[w * (HD + 2) + HD] - M) * comb[w * (HD + 2) + HD + 1];
+        const size_t row = (size_t)slot * a.mixRowsLd;
+        auto put_row = [&](size_t col, float v) {
+            if (a.mixRowsHalf) ((_Float16*)a.mixRows)[row + col] = (_Float16)fminf(fmaxf(v, -65504.0f), 65504.0f); // saturating
+            else ((float*)a.mixRows)[row + col] = v;
+        };
+        for (int i = tid; i < HD; i += NW * 64) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; w++) s += expf(comb[w * (HD + 2) + HD] - M) * comb[w * (HD + 2) + i];
+            float v = s / l;
+            if (a.gating) v = v * sigmoidf_ref(qkv[L.offG + h * HD + i]);
+            put_row((size_t)h * HD + i, v);
+        }
+        if (h == 0)
+            for (int j = tid; j < a.ple; j += NW * 64) {
+                const size_t e = (size_t)a.tok[slot] * a.ple + j;
+                const float pv = a.wbytes == 2 ? __uint_as_float(((uint32_t)((const uint16_t*)L.pleTable)[e]) << 16) : ((const float*)L.pleTable)[e];
+                put_row((size_t)a.heads * HD + j, siluf_ref(qkv[L.offPle + j]) * pv);
+            }
+        return;
+    }
     for (int i = tid; i < HD; i += NW * 64) {
         float s = 0.f;
 #pragma unroll

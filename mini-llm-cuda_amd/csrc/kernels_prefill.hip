@@ -1603,10 +1603,33 @@ __global__ void __launch_bounds__(PWG) k_bd_finish(StepArgs a, const float* lg, 
     }
     float v = -3.0e38f;
     int idx = 0x7fffffff;
-    for (int i = tid; i < a.vocab; i += PWG) {
-        const float x = row[i];
-        dst[i] = x;
-        if (x > v) { v = x; idx = i; } // i ascends: ties keep the lower index
+    if ((a.vocab & 3) == 0) { // 16 bytes per lane, four loads in flight before the first store (row and dst do not overlap)
+        const f32x4* row4 = reinterpret_cast<const f32x4*>(row);
+        f32x4* dst4 = reinterpret_cast<f32x4*>(dst);
+        const int n4 = a.vocab >> 2;
+        for (int i0 = tid; i0 < n4; i0 += 4 * PWG) {
+            f32x4 x[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) x[k] = row4[min(i0 + k * PWG, n4 - 1)];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int i = i0 + k * PWG;
+                if (i < n4) {
+                    dst4[i] = x[k];
+                    // i ascends per thread and the four elements are taken in order: ties keep the lower index
+                    if (x[k].x > v) { v = x[k].x; idx = 4 * i; }
+                    if (x[k].y > v) { v = x[k].y; idx = 4 * i + 1; }
+                    if (x[k].z > v) { v = x[k].z; idx = 4 * i + 2; }
+                    if (x[k].w > v) { v = x[k].w; idx = 4 * i + 3; }
+                }
+            }
+        }
+    } else {
+        for (int i = tid; i < a.vocab; i += PWG) {
+            const float x = row[i];
+            dst[i] = x;
+            if (x > v) { v = x; idx = i; } // i ascends: ties keep the lower index
+        }
     }
     sv[tid] = v; si[tid] = idx;
     __syncthreads();
@@ -1675,7 +1698,8 @@ int mlh_launch_batch_step(mlh_ctx* c, int nseq, const int* tokPtr) {
         const bool gdn = L.kind != MLH_KIND_ATTENTION;
         // The GDN kernel writes its read-out and the PLE columns straight into the GEMM's input rows (mlh_launch_one
         // reads the step's tokens from the context's own buffer, hence the second condition).
-        const bool direct = gdn && tokPtr == c->d_tok;
+        // The attention kernel does the same when one workgroup holds all keys of a (head, sequence) pair.
+        const bool direct = (gdn || c->nsplit == 1) && tokPtr == c->d_tok;
         if (direct) { c->mixRows = c->pfA; c->mixRowsLd = c->maxAd + hp.pleDim; c->mixRowsHalf = bf ? 1 : 0; }
         int rc = mlh_launch_one(c, gdn ? MLH_K_GDN : MLH_K_ATTN, t, nseq);
         c->mixRows = nullptr;
