@@ -257,11 +257,13 @@ def test_prefill_bf16_ragged_batch_both_attention_variants(pkg, orc, kind):
 
 
 # ---- batched decode through the skinny GEMM ------------------------------------------------------
-@pytest.mark.parametrize("kind,nseq,graph", [("hybrid", 8, 0), ("hybrid_flags", 13, 1), ("attn_long", 33, 0), ("hd128", 64, 2)])
+@pytest.mark.parametrize("kind,nseq,graph", [("hybrid", 8, 0), ("hybrid_flags", 13, 1), ("hybrid_flags", 20, 0), ("attn_long", 33, 0), ("hd128", 64, 2)])
 def test_batched_decode_gemm_path(pkg, orc, kind, nseq, graph):
     """Eight or more sequences per step take the MFMA path (skinny GEMMs + decode attention/GDN kernels):
     ids and final logits against the float64 oracle, per sequence, with ragged prompt lengths; the same
-    run through the GEMV kernels (mode 1) must agree within the fp32 tolerance."""
+    run through the GEMV kernels (mode 1) must agree within the fp32 tolerance.  From 16 sequences on one attention
+    workgroup holds all keys of a (head, sequence) pair and writes the gated output rows itself; below that the
+    split-KV partials go through the combine kernel -- the flags case runs both ways."""
     hp = small_cfg(pkg, kind, maxSeqs=nseq)
     model, dev, w = make(pkg, orc, hp, seed=31)
     dev.set_graph(graph)
