@@ -304,3 +304,55 @@ def test_batched_equals_single(pkg, orc):
             _, lg = dec.step(int(t))
         assert_logits_close(batched_logits[s], lg, FP32_RTOL, f"seq {s}")
     dev.close()
+
+
+@pytest.mark.parametrize("persistent", [3, 0], ids=["xcd", "kernels"])
+def test_device_api_rejects_bad_arguments_and_fills_a_sequence_to_the_brim(pkg, orc, persistent):
+    """Argument checks of the C ABI (status -1 and a message, state untouched) and the maximum size: a sequence
+    filled to exactly maxL positions -- prompt plus decode steps -- still matches the oracle at its last step, one
+    position more is refused."""
+    hp = pkg.config(1, maxL=96, maxSeqs=2)
+    model, dev, w = make(pkg, orc, hp, seed=41)
+    dev.set_persistent(persistent)
+    V, maxL = hp.vocabSize, hp.maxL
+
+    def refused(fn, what):
+        with pytest.raises(pkg.MlhError) as e:
+            fn()
+        assert what in str(e.value), str(e.value)
+
+    refused(lambda: dev.prefill(0, []), "empty prompt")
+    refused(lambda: dev.prefill(2, [1, 2, 3]), "distinct and in range")
+    refused(lambda: dev.prefill(-1, [1, 2, 3]), "distinct and in range")
+    refused(lambda: dev.prefill_batch([0, 0], [[1, 2], [3]]), "distinct and in range")
+    refused(lambda: dev.prefill(0, [1, V, 3]), "token id out of range")
+    refused(lambda: dev.prefill(0, [1, -1, 3]), "token id out of range")
+    refused(lambda: dev.prefill(0, [1] * (maxL + 1)), "does not fit in maxL")
+    assert dev.seq_len(0) == 0 and dev.seq_len(1) == 0  # nothing of the refused calls was applied
+
+    prompt = pkg.random_tokens(41, 0, V, 40)
+    dev.prefill(0, prompt)
+    first = dev.greedy_token(0)
+    refused(lambda: dev.decode_loop([V], 1), "token id out of range")
+    refused(lambda: dev.decode_loop([first, first, first], 1), "nseq out of range")
+    refused(lambda: dev.decode_loop([first], maxL - 40 + 1), "exceed maxL")
+    assert dev.seq_len(0) == 40
+
+    steps = maxL - 40  # the last step reads positions 0 .. maxL - 1
+    out = dev.decode_loop([first], steps)
+    assert dev.seq_len(0) == maxL
+    ids = [first] + [int(t) for t in out[:, 0]]
+    dec = orc.Decoder(w, "f64")
+    exact, tol = check_greedy_against_oracle(dec, prompt, ids, GAP_TOL, what="sequence filled to maxL")
+    assert exact + tol == len(ids)
+    dec.reset()
+    for t in list(prompt) + ids[:-1]:
+        _, lg = dec.step(int(t))
+    assert_logits_close(dev.logits(0), lg, FP32_RTOL, "logits at position maxL - 1")
+    refused(lambda: dev.decode_loop([ids[-1]], 1), "exceed maxL")
+    refused(lambda: dev.prefill(0, [1]), "does not fit in maxL")
+    dev.reset(0)
+    assert dev.seq_len(0) == 0
+    dev.prefill(0, [5] * maxL)  # a prompt of exactly maxL tokens is taken
+    assert dev.seq_len(0) == maxL
+    dev.close()
