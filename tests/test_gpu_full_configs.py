@@ -224,3 +224,30 @@ def test_config5_width_prefill_2048_tokens(pkg, orc):
         print(f"config-5 width, prompt of {n}: max|diff|/max|logit| at the last position = {e:.3e}")
         assert e <= 1e-2 <= BF16_RTOL
     dev.close()
+
+
+def test_config5_full_size_prefill_against_committed_oracle_logits(pkg):
+    """Configuration 5 at its full size (24 layers, vocabulary 32000, bf16 weights) and one 2048-token prompt: the
+    MFMA prefill's last-position logits for prompts that end at chunk and page edges, at odd places and at 2048
+    tokens, against tests/golden/cfg5_prefill_golden.npz -- the float64 oracle's full recompute on the same
+    bf16-rounded weights, written by tests/golden/make_cfg5_golden.py (ten minutes of CPU, hence a fixture).
+    Bound: 2e-2 of the largest logit (bf16 path), asserted at 1e-2."""
+    import os
+    g = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "cfg5_prefill_golden.npz"))
+    hp = pkg.config(5, maxSeqs=1)
+    model = pkg.Model.generate(hp, seed=5)
+    assert np.array_equal(model.tensor(0, 0)[:4, :8], g["embedding_head"])  # same generator, same weights
+    toks = pkg.random_tokens(5, 0, hp.vocabSize, 2048)
+    assert np.array_equal(toks, g["tokens"])
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    worst = 0.0
+    for p, want in zip(g["positions"], g["logits"]):
+        dev.reset()
+        dev.prefill(0, toks[:int(p) + 1])
+        got = dev.logits(0)
+        e = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+        worst = max(worst, e)
+        print(f"config 5, full size, prompt of {int(p) + 1}: max|diff|/max|logit| = {e:.3e}, argmax {int(np.argmax(got))} / {int(np.argmax(want))}")
+        assert e <= 1e-2 <= BF16_RTOL
+    dev.close()
