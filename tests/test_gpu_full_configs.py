@@ -251,3 +251,118 @@ def test_config5_full_size_prefill_against_committed_oracle_logits(pkg):
         print(f"config 5, full size, prompt of {int(p) + 1}: max|diff|/max|logit| = {e:.3e}, argmax {int(np.argmax(got))} / {int(np.argmax(want))}")
         assert e <= 1e-2 <= BF16_RTOL
     dev.close()
+
+
+# ---- full decode horizons against committed oracle outcomes ------------------------------------------------------
+# tests/golden/horizon_cfg{3,4,5}_golden.npz hold what the float64 oracle produced for the benchmark workloads over
+# their whole horizons (tests/golden/make_horizon_golden.py; minutes to half an hour of CPU each, hence fixtures):
+# greedy ids, the four best logits of every step, complete logit rows at a few steps.
+def _golden(name):
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name)
+    if not os.path.exists(path):
+        pytest.skip(f"{name} has not been generated (tests/golden/make_horizon_golden.py)")
+    return np.load(path)
+
+
+def _compare_with_horizon(g, pre, ids_gpu, logits_gpu, gap_tol, logits_ok, what):
+    """ids: equal to the oracle's, or -- at the first difference -- within gap_tol of the oracle's best by the
+    oracle's own four best logits of that step (from there on the histories differ and the comparison ends).
+    logits_gpu {step: row}: compared with the fixture's rows at the steps both hold, up to that point."""
+    ids_o, top_idx, top_val = g[pre + "ids"], g[pre + "top_idx"], g[pre + "top_val"]
+    assert len(ids_gpu) == len(ids_o)
+    upto = len(ids_o)
+    for i, gid in enumerate(ids_gpu):
+        if int(gid) != int(ids_o[i]):
+            row = [int(t) for t in top_idx[i]]
+            assert int(gid) in row, f"{what} step {i}: GPU picked {int(gid)}, not among the oracle's best four {row}"
+            gap = float(top_val[i][0] - top_val[i][row.index(int(gid))])
+            assert gap <= gap_tol, f"{what} step {i}: GPU picked {int(gid)}, oracle {row[0]}, gap {gap:.3e} > {gap_tol}"
+            upto = i
+            break
+    checked = 0
+    for step, want in zip(g[pre + "full_steps"], g[pre + "full_logits"]):
+        if int(step) in logits_gpu and int(step) <= upto:
+            logits_ok(logits_gpu[int(step)], want, f"{what} step {int(step)}")
+            checked += 1
+    assert checked >= 1
+    return upto, checked
+
+
+def _fp32_ok(got, want, what):
+    assert_logits_close(got, want, FP32_RTOL, what)
+
+
+def _bf16_ok(got, want, what):
+    e = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+    assert e <= 1e-2 <= BF16_RTOL, (what, e)
+
+
+def test_config3_whole_horizon_against_committed_oracle(pkg):
+    """Hybrid 3 GDN : 1 attention + PLE, 128-token prompt, all 1024 greedy steps of the benchmark workload."""
+    g = _golden("horizon_cfg3_golden.npz")
+    hp = pkg.config(3)
+    hp.maxSeqs = 1
+    model = pkg.Model.generate(hp, 3)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    prompt = pkg.random_tokens(3, 0, hp.vocabSize, 128)
+    assert np.array_equal(prompt, g["prompt"])
+    dev.prefill(0, prompt)
+    ids = [dev.greedy_token(0)]
+    logits = {0: dev.logits(0)}
+    for n in (1, 254, 1, 255, 256, 257):  # lands on steps 1, 255, 256, 511, 767, 1024
+        ids += [int(t) for t in dev.decode_loop([ids[-1]], n)[:, 0]]
+        logits[len(ids) - 1] = dev.logits(0)
+    upto, checked = _compare_with_horizon(g, "", ids, logits, GAP_TOL, _fp32_ok, "config 3")
+    print(f"config 3: {upto} of {len(ids)} ids equal to the oracle's, logits compared at {checked} steps")
+    dev.close()
+
+
+def test_config4_whole_horizon_against_committed_oracle(pkg):
+    """64 sequences, prompts uniform in [32, 512], all 256 batched greedy steps; the shortest, a middle and the
+    longest sequence against the oracle's outcome for each."""
+    g = _golden("horizon_cfg4_golden.npz")
+    hp = pkg.config(4)
+    nseq = hp.maxSeqs
+    model = pkg.Model.generate(hp, 4)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    lens = np.random.default_rng(44).integers(32, 513, size=nseq)
+    assert np.array_equal(lens, g["lens"])
+    prompts = [pkg.random_tokens(44, s, hp.vocabSize, int(n)) for s, n in enumerate(lens)]
+    dev.prefill_batch(list(range(nseq)), prompts)
+    sel = [int(s) for s in g["seqs"]]
+    ids = np.array([[dev.greedy_token(s) for s in range(nseq)]], dtype=np.int32)
+    logits = {s: {0: dev.logits(s)} for s in sel}
+    for n in (128, 128):
+        ids = np.concatenate([ids, dev.decode_loop([int(t) for t in ids[-1]], n)])
+        for s in sel:
+            logits[s][ids.shape[0] - 1] = dev.logits(s)
+    for s in sel:
+        upto, checked = _compare_with_horizon(g, f"s{s}_", ids[:, s], logits[s], GAP_TOL, _fp32_ok, f"config 4 sequence {s}")
+        print(f"config 4 sequence {s} (prompt {lens[s]}): {upto} of {ids.shape[0]} ids equal to the oracle's, logits compared at {checked} steps")
+    dev.close()
+
+
+def test_config5_whole_horizon_against_committed_oracle(pkg):
+    """d2048 x 24 layers, bf16 weights: the 8 x 2048-token prefill in one pass and all 128 batched decode steps;
+    sequence 0 against the oracle's outcome (ids by the gap rule at 2e-2 of the largest logit, logits at 1e-2)."""
+    g = _golden("horizon_cfg5_golden.npz")
+    hp = pkg.config(5)
+    nseq, plen = 8, 2048
+    model = pkg.Model.generate(hp, 5)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    prompts = [pkg.random_tokens(55, s, hp.vocabSize, plen) for s in range(nseq)]
+    assert np.array_equal(prompts[0], g["prompt"])
+    dev.prefill_batch(list(range(nseq)), prompts)
+    ids = np.array([[dev.greedy_token(s) for s in range(nseq)]], dtype=np.int32)
+    logits = {0: dev.logits(0)}
+    for n in (64, 64):
+        ids = np.concatenate([ids, dev.decode_loop([int(t) for t in ids[-1]], n)])
+        logits[ids.shape[0] - 1] = dev.logits(0)
+    tied = BF16_RTOL * float(np.max(np.abs(g["full_logits"][0])))
+    upto, checked = _compare_with_horizon(g, "", ids[:, 0], logits, tied, _bf16_ok, "config 5 sequence 0")
+    print(f"config 5 sequence 0: {upto} of {ids.shape[0]} ids equal to the oracle's, logits compared at {checked} steps")
+    dev.close()
