@@ -346,23 +346,40 @@ def test_config4_whole_horizon_against_committed_oracle(pkg):
 
 
 def test_config5_whole_horizon_against_committed_oracle(pkg):
-    """d2048 x 24 layers, bf16 weights: the 8 x 2048-token prefill in one pass and all 128 batched decode steps;
-    sequence 0 against the oracle's outcome (ids by the gap rule at 2e-2 of the largest logit, logits at 1e-2)."""
+    """d2048 x 24 layers, bf16 weights: the 8 x 2048-token prefill in one pass and all 128 batched decode steps.
+    Sequence 0 is fed the oracle's own ids (the other seven decode greedily), so that the whole horizon is compared
+    although a bf16 pick may differ where two candidates are close: every pick of the device is the oracle's or within
+    2e-2 of the largest logit of it by the oracle's four best, and the logits at steps 0, 64, 128 are within 1e-2."""
     g = _golden("horizon_cfg5_golden.npz")
     hp = pkg.config(5)
-    nseq, plen = 8, 2048
+    nseq, plen, steps = 8, 2048, 128
     model = pkg.Model.generate(hp, 5)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     prompts = [pkg.random_tokens(55, s, hp.vocabSize, plen) for s in range(nseq)]
     assert np.array_equal(prompts[0], g["prompt"])
     dev.prefill_batch(list(range(nseq)), prompts)
-    ids = np.array([[dev.greedy_token(s) for s in range(nseq)]], dtype=np.int32)
-    logits = {0: dev.logits(0)}
-    for n in (64, 64):
-        ids = np.concatenate([ids, dev.decode_loop([int(t) for t in ids[-1]], n)])
-        logits[ids.shape[0] - 1] = dev.logits(0)
+    ids_o, top_idx, top_val = g["ids"], g["top_idx"], g["top_val"]
+    full = {int(st): row for st, row in zip(g["full_steps"], g["full_logits"])}
     tied = BF16_RTOL * float(np.max(np.abs(g["full_logits"][0])))
-    upto, checked = _compare_with_horizon(g, "", ids[:, 0], logits, tied, _bf16_ok, "config 5 sequence 0")
-    print(f"config 5 sequence 0: {upto} of {ids.shape[0]} ids equal to the oracle's, logits compared at {checked} steps")
+    picks = np.array([dev.greedy_token(s) for s in range(nseq)], dtype=np.int32)
+    exact = tolerated = checked = 0
+    for i in range(steps + 1):
+        row = [int(t) for t in top_idx[i]]
+        if int(picks[0]) == int(ids_o[i]):
+            exact += 1
+        else:
+            assert int(picks[0]) in row, f"step {i}: device picked {int(picks[0])}, not among the oracle's best four {row}"
+            gap = float(top_val[i][0] - top_val[i][row.index(int(picks[0]))])
+            assert gap <= tied, f"step {i}: device picked {int(picks[0])}, oracle {row[0]}, gap {gap:.3e} > {tied:.3e}"
+            tolerated += 1
+        if i in full:
+            _bf16_ok(dev.logits(0), full[i], f"config 5 sequence 0 step {i}")
+            checked += 1
+        if i < steps:
+            feed = picks.copy()
+            feed[0] = ids_o[i]  # sequence 0 follows the oracle's history
+            picks = dev.decode_step(feed)
+    print(f"config 5 sequence 0, history of the oracle: {exact} picks equal, {tolerated} within the tie tolerance, logits compared at {checked} steps")
+    assert checked == len(full) and exact >= (steps + 1) * 9 // 10
     dev.close()
