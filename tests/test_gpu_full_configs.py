@@ -383,3 +383,27 @@ def test_config5_whole_horizon_against_committed_oracle(pkg):
     print(f"config 5 sequence 0, history of the oracle: {exact} picks equal, {tolerated} within the tie tolerance, logits compared at {checked} steps")
     assert checked == len(full) and exact >= (steps + 1) * 9 // 10
     dev.close()
+
+
+def test_reference_default_shape_whole_context_against_committed_oracle(pkg):
+    """The shape the reference ships compiled in (network_meta.h:3-20: dim 768, 6 heads x 128, ffn 3072, 16 layers,
+    vocabulary 20160, QK-norm and query gating on, maxL 1280) with uniform +-0.02 weights: a 256-token prompt through
+    the prefill and 1024 greedy steps -- the KV cache filled to maxL -- against the oracle's outcome."""
+    g = _golden("horizon_refdefault_golden.npz")
+    hp = pkg.reference_defaults()
+    model = pkg.Model.new(hp)
+    model.init_uniform(9, 0.02)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    prompt = pkg.random_tokens(9, 0, hp.vocabSize, 256)
+    assert np.array_equal(prompt, g["prompt"])
+    dev.prefill(0, prompt)
+    ids = [dev.greedy_token(0)]
+    logits = {0: dev.logits(0)}
+    for n in (1, 254, 1, 444, 324):  # lands on steps 1, 255, 256, 700, 1024
+        ids += [int(t) for t in dev.decode_loop([ids[-1]], n)[:, 0]]
+        logits[len(ids) - 1] = dev.logits(0)
+    assert dev.seq_len(0) == hp.maxL
+    upto, checked = _compare_with_horizon(g, "", ids, logits, GAP_TOL, _fp32_ok, "reference-default shape")
+    print(f"reference-default shape: {upto} of {len(ids)} ids equal to the oracle's ({len(set(ids))} distinct), logits compared at {checked} steps")
+    dev.close()
