@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Writes horizon_cfg{3,4,5}_golden.npz and horizon_refdefault_golden.npz: the FULL decode horizons of configurations
+"""Writes horizon_cfg{3,4,5}_golden.npz, horizon_cfg2_flags_golden.npz and horizon_refdefault_golden.npz: the FULL decode horizons of configurations
 3, 4 and 5 (the benchmark workloads), and a long one at the shape the reference ships compiled in, through the float64 CPU oracle, one token at a time with its cache -- too slow to repeat inside a test
 (config 5: half an hour), so the outcome is kept: the oracle's greedy ids, its four best logits at every step, and
 complete logit rows (float32) at a few steps.
@@ -8,11 +8,13 @@ complete logit rows (float32) at a few steps.
   config 4  seed 4, 64 prompts uniform in [32, 512] (numpy default_rng(44)); the shortest, a middle and the longest
             sequence, 256 greedy steps each
   config 5  seed 5, bf16-rounded weights, sequence 0 of the 8 x 2048-token prompts (seed 55), 128 greedy steps
+  2         configuration 2 with BOTH architecture flags on (QK-norm, query gating: the reference's shipped setting,
+            network_meta.h:19-20), seed 1, 64-token prompt, 512 greedy steps
   0         the reference's compiled-in shape (network_meta.h:3-20: dim 768, 6 heads x 128, ffn 3072, 16 layers,
             vocabulary 20160, QK-norm and query gating on, maxL 1280), uniform +-0.02 weights from seed 9
             (random_weights.cu:15-25; own generator), a 256-token prompt and 1024 greedy steps: the cache filled to maxL
 
-Run from the repository root: python tests/golden/make_horizon_golden.py 3|4|5|0"""
+Run from the repository root: python tests/golden/make_horizon_golden.py 2|3|4|5|0"""
 import os
 import sys
 import time
@@ -79,6 +81,12 @@ def main(which):
         prompt = m.random_tokens(55, 0, hp.vocabSize, 2048)
         r = greedy(orc, orc.Weights.from_model(model, bf16=True), prompt, 128, (0, 64, 128))
         np.savez_compressed(os.path.join(HERE, "horizon_cfg5_golden.npz"), prompt=prompt.astype(np.int32), **r)
+    elif which == 2:
+        hp = m.config(2, qkRmsNorm=1, queryGating=1)
+        model = m.Model.generate(hp, 1)
+        prompt = m.random_tokens(1, 0, hp.vocabSize, 64)
+        r = greedy(orc, orc.Weights.from_model(model), prompt, 512, (0, 1, 64, 65, 200, 383, 512))
+        np.savez_compressed(os.path.join(HERE, "horizon_cfg2_flags_golden.npz"), prompt=prompt.astype(np.int32), **r)
     elif which == 0:
         hp = m.reference_defaults()
         model = m.Model.new(hp)

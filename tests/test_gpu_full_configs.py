@@ -407,3 +407,27 @@ def test_reference_default_shape_whole_context_against_committed_oracle(pkg):
     upto, checked = _compare_with_horizon(g, "", ids, logits, GAP_TOL, _fp32_ok, "reference-default shape")
     print(f"reference-default shape: {upto} of {len(ids)} ids equal to the oracle's ({len(set(ids))} distinct), logits compared at {checked} steps")
     dev.close()
+
+
+@pytest.mark.parametrize("path", [3, 0], ids=["xcd", "kernels"])
+def test_config2_with_both_flags_whole_horizon_against_committed_oracle(pkg, path):
+    """Configuration 2 with QK-norm and query gating on (the setting the reference ships, network_meta.h:19-20):
+    64-token prompt and all 512 greedy steps, on the single-launch path and on the kernel sequence."""
+    g = _golden("horizon_cfg2_flags_golden.npz")
+    hp = pkg.config(2, qkRmsNorm=1, queryGating=1)
+    hp.maxSeqs = 1
+    model = pkg.Model.generate(hp, 1)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    dev.set_persistent(path)
+    prompt = pkg.random_tokens(1, 0, hp.vocabSize, 64)
+    assert np.array_equal(prompt, g["prompt"])
+    dev.prefill(0, prompt)
+    ids = [dev.greedy_token(0)]
+    logits = {0: dev.logits(0)}
+    for n in (1, 63, 1, 135, 183, 129):  # lands on steps 1, 64, 65, 200, 383, 512
+        ids += [int(t) for t in dev.decode_loop([ids[-1]], n)[:, 0]]
+        logits[len(ids) - 1] = dev.logits(0)
+    upto, checked = _compare_with_horizon(g, "", ids, logits, GAP_TOL, _fp32_ok, "config 2 with both flags")
+    print(f"config 2 with both flags: {upto} of {len(ids)} ids equal to the oracle's ({len(set(ids))} distinct), logits compared at {checked} steps")
+    dev.close()
