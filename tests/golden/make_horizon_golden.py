@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Writes horizon_cfg{3,4,5}_golden.npz, horizon_cfg2_flags_golden.npz and horizon_refdefault_golden.npz: the FULL decode horizons of configurations
+"""Writes horizon_cfg{3,4,5}_golden.npz, horizon_cfg2_flags_golden.npz, horizon_refdefault_golden.npz and forward_refdefault_golden.npz: the FULL decode horizons of configurations
 3, 4 and 5 (the benchmark workloads), and a long one at the shape the reference ships compiled in, through the float64 CPU oracle, one token at a time with its cache -- too slow to repeat inside a test
 (config 5: half an hour), so the outcome is kept: the oracle's greedy ids, its four best logits at every step, and
 complete logit rows (float32) at a few steps.
@@ -10,11 +10,15 @@ complete logit rows (float32) at a few steps.
   config 5  seed 5, bf16-rounded weights, sequence 0 of the 8 x 2048-token prompts (seed 55), 128 greedy steps
   2         configuration 2 with BOTH architecture flags on (QK-norm, query gating: the reference's shipped setting,
             network_meta.h:19-20), seed 1, 64-token prompt, 512 greedy steps
+  1         the reference's compiled-in shape, teacher-forced: one random 1280-token sequence (maxL) through the full
+            recompute as the reference's runInference(L) does it -- per position the best two logits, the probability of
+            the token that follows (clamped at 1e-4 as training_orchestrator.cu:343-347 does) and complete rows at a few
+            positions (forward_refdefault_golden.npz)
   0         the reference's compiled-in shape (network_meta.h:3-20: dim 768, 6 heads x 128, ffn 3072, 16 layers,
             vocabulary 20160, QK-norm and query gating on, maxL 1280), uniform +-0.02 weights from seed 9
             (random_weights.cu:15-25; own generator), a 256-token prompt and 1024 greedy steps: the cache filled to maxL
 
-Run from the repository root: python tests/golden/make_horizon_golden.py 2|3|4|5|0"""
+Run from the repository root: python tests/golden/make_horizon_golden.py 0|1|2|3|4|5"""
 import os
 import sys
 import time
@@ -87,6 +91,22 @@ def main(which):
         prompt = m.random_tokens(1, 0, hp.vocabSize, 64)
         r = greedy(orc, orc.Weights.from_model(model), prompt, 512, (0, 1, 64, 65, 200, 383, 512))
         np.savez_compressed(os.path.join(HERE, "horizon_cfg2_flags_golden.npz"), prompt=prompt.astype(np.int32), **r)
+    elif which == 1:
+        hp = m.reference_defaults()
+        model = m.Model.new(hp)
+        model.init_uniform(9, 0.02)
+        toks = m.random_tokens(91, 0, hp.vocabSize, hp.maxL)
+        t0 = time.time()
+        ref = orc.forward_full(orc.Weights.from_model(model), toks, "f64", last_only=False, want_probs=True)
+        print(f"  full recompute of {hp.maxL} tokens: {time.time() - t0:.0f} s", flush=True)
+        lg, pr = ref["logits"], ref["probs"]
+        order = np.argsort(-lg, axis=1, kind="stable")[:, :2]
+        rows = (0, 63, 64, 639, hp.maxL - 1)
+        np.savez_compressed(os.path.join(HERE, "forward_refdefault_golden.npz"), tokens=toks.astype(np.int32),
+                            top_idx=order.astype(np.int32), top_val=np.take_along_axis(lg, order, axis=1),
+                            p_next=pr[np.arange(hp.maxL - 1), toks[1:]], p_max=pr.max(axis=1),
+                            rows=np.array(rows, dtype=np.int32), row_logits=lg[list(rows)].astype(np.float32),
+                            row_probs=pr[list(rows)].astype(np.float32))
     elif which == 0:
         hp = m.reference_defaults()
         model = m.Model.new(hp)

@@ -431,3 +431,42 @@ def test_config2_with_both_flags_whole_horizon_against_committed_oracle(pkg, pat
     upto, checked = _compare_with_horizon(g, "", ids, logits, GAP_TOL, _fp32_ok, "config 2 with both flags")
     print(f"config 2 with both flags: {upto} of {len(ids)} ids equal to the oracle's ({len(set(ids))} distinct), logits compared at {checked} steps")
     dev.close()
+
+
+def test_reference_default_shape_teacher_forced_full_context(pkg):
+    """What the reference's runInference(L) leaves behind for L = maxL = 1280 at its compiled-in shape (both flags):
+    logits and probabilities of EVERY position and the mean next-token loss of a random sequence, against the
+    oracle's full recompute kept in tests/golden/forward_refdefault_golden.npz (per position: best two logits,
+    probability of the following token, largest probability; complete rows at five positions)."""
+    g = _golden("forward_refdefault_golden.npz")
+    hp = pkg.reference_defaults()
+    model = pkg.Model.new(hp)
+    model.init_uniform(9, 0.02)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    toks = pkg.random_tokens(91, 0, hp.vocabSize, hp.maxL)
+    assert np.array_equal(toks, g["tokens"])
+    lg, pr, nll = dev.forward_full(0, toks)
+    n = hp.maxL
+    assert lg.shape == (n, hp.vocabSize) and dev.seq_len(0) == n
+    top_idx, top_val = g["top_idx"], g["top_val"]
+    scale = np.max(np.abs(top_val), axis=1)
+    # every position: the oracle's best two logits, the pick (or a tie within GAP_TOL), the probabilities the loss uses
+    pos = np.arange(n)
+    for k in range(2):
+        d = np.abs(lg[pos, top_idx[:, k]] - top_val[:, k])
+        assert float(np.max(d / scale)) <= FP32_RTOL, (k, float(np.max(d / scale)))
+    pick = np.argmax(lg, axis=1)
+    other = pick != top_idx[:, 0]
+    assert np.all(top_val[other, 0] - lg[pos[other], pick[other]] <= GAP_TOL + FP32_RTOL * scale[other])
+    assert float(np.max(np.abs(pr.max(axis=1) - g["p_max"]) / g["p_max"])) <= FP32_RTOL
+    p_next = pr[pos[:-1], toks[1:]]
+    assert float(np.max(np.abs(p_next - g["p_next"]) / np.maximum(g["p_next"], 1e-9))) <= 5 * FP32_RTOL
+    assert np.allclose(pr.sum(axis=1), 1.0, atol=1e-5)
+    want_nll = float(np.mean(-np.log(np.maximum(g["p_next"], 1e-4))))  # the reference's clamp
+    assert abs(nll - want_nll) <= 1e-4, (nll, want_nll)
+    for r, wl, wp in zip(g["rows"], g["row_logits"], g["row_probs"]):
+        assert_logits_close(lg[int(r)], wl, FP32_RTOL, f"reference-default shape, position {int(r)}")
+        assert np.max(np.abs(pr[int(r)] - wp)) <= 1e-6 + FP32_RTOL * np.max(wp)
+    print(f"reference-default shape, 1280 positions: mean loss {nll:.5f} (oracle {want_nll:.5f}), {int(other.sum())} picks differ within the tie rule")
+    dev.close()
