@@ -298,14 +298,17 @@ def _bf16_ok(got, want, what):
     assert e <= 1e-2 <= BF16_RTOL, (what, e)
 
 
-def test_config3_whole_horizon_against_committed_oracle(pkg):
-    """Hybrid 3 GDN : 1 attention + PLE, 128-token prompt, all 1024 greedy steps of the benchmark workload."""
+@pytest.mark.parametrize("path", [3, 1, 0], ids=["xcd", "barrier", "kernels"])
+def test_config3_whole_horizon_against_committed_oracle(pkg, path):
+    """Hybrid 3 GDN : 1 attention + PLE, 128-token prompt, all 1024 greedy steps of the benchmark workload, on each
+    of the three batch-1 decode paths (single launch with XCD ranks, single launch with grid barriers, kernel sequence)."""
     g = _golden("horizon_cfg3_golden.npz")
     hp = pkg.config(3)
     hp.maxSeqs = 1
     model = pkg.Model.generate(hp, 3)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
+    dev.set_persistent(path)
     prompt = pkg.random_tokens(3, 0, hp.vocabSize, 128)
     assert np.array_equal(prompt, g["prompt"])
     dev.prefill(0, prompt)
