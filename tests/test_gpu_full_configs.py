@@ -322,15 +322,18 @@ def test_config3_whole_horizon_against_committed_oracle(pkg, path):
     dev.close()
 
 
-def test_config4_whole_horizon_against_committed_oracle(pkg):
-    """64 sequences, prompts uniform in [32, 512], all 256 batched greedy steps; the shortest, a middle and the
-    longest sequence against the oracle's outcome for each."""
+@pytest.mark.parametrize("graph", [0, 4], ids=["launches", "graph-of-4-steps"])
+def test_config4_whole_horizon_against_committed_oracle(pkg, graph):
+    """64 sequences, prompts uniform in [32, 512], all 256 batched greedy steps (as plain launches, and replayed
+    as captured graphs of four steps); the shortest, a middle and the longest sequence against the oracle's outcome
+    for each."""
     g = _golden("horizon_cfg4_golden.npz")
     hp = pkg.config(4)
     nseq = hp.maxSeqs
     model = pkg.Model.generate(hp, 4)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
+    dev.set_graph(graph)
     lens = np.random.default_rng(44).integers(32, 513, size=nseq)
     assert np.array_equal(lens, g["lens"])
     prompts = [pkg.random_tokens(44, s, hp.vocabSize, int(n)) for s, n in enumerate(lens)]
