@@ -183,7 +183,9 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
  * per-layer embeddings of a width that is a multiple of 8) on a 256-unit device
  * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default.
  * Both need every compute unit for themselves and all their waits are bounded: when a launch gives up (units held
- * by other work), nothing of the sequence has advanced, and the call redoes its steps as the kernel sequence and
+ * by other work), the sequence is as it was before the launch (position, token and tags are written at a kernel's
+ * normal end only; the XCD-rank kernel keeps gated-delta-net states in LDS until then, the barrier kernel's are put
+ * back from a copy taken before its launch), and the call redoes its steps as the kernel sequence and
  * leaves the context at mode 0 (mlh_get_persistent, mlh_persistent_fallbacks).
  * Mode 0, unsupported shapes and nseq > 1: a sequence of kernels issued as mlh_set_graph says. */
 int mlh_set_persistent(mlh_ctx* ctx, int mode);
@@ -200,6 +202,10 @@ int mlh_persistent_fallbacks(mlh_ctx* ctx);
  * any wait having to expire.  mlh_debug_set_xcd_tag: sets the XCD-rank kernel's running tag count (device word and
  * host mirror), to exercise the reset that precedes a wrap of the 32-bit tags. */
 int mlh_debug_inject_abort(mlh_ctx* ctx, int launches);
+/* mlh_debug_inject_abort_at_step: the next single-launch decode launch gives up by itself when workgroup 0 reaches
+ * decode step `step` (> 0; counted from 0 inside the launch) -- after the earlier steps have run and written what
+ * they write -- so the test can see that the redo starts from the state before the launch.  0 switches it off. */
+int mlh_debug_inject_abort_at_step(mlh_ctx* ctx, int step);
 int mlh_debug_set_xcd_tag(mlh_ctx* ctx, unsigned tagsUsed);
 
 /* Next-token rule of the decode entry points.  temperature 0 (the default): greedy, the argmax fused into the

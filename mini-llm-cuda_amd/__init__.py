@@ -93,6 +93,7 @@ _sigs_dev = {
     "mlh_get_persistent": (c_int, [c_void_p]),
     "mlh_persistent_fallbacks": (c_int, [c_void_p]),
     "mlh_debug_inject_abort": (c_int, [c_void_p, c_int]),
+    "mlh_debug_inject_abort_at_step": (c_int, [c_void_p, c_int]),
     "mlh_debug_set_xcd_tag": (c_int, [c_void_p, ctypes.c_uint]),
     "mlh_xcd_decode_supported": (c_int, [c_void_p]),
     "mlh_synchronize": (c_int, [c_void_p]),
@@ -226,6 +227,22 @@ class Model:
     def init_uniform(self, seed, rng):
         host.mll_model_init_uniform(self._h, seed, rng)
 
+    GAIN_TENSORS = (T_FINAL_RMS_GAMMA, T_RMS_GAMMA, T_RMS_GAMMA2, T_QUERY_RMS_GAMMA, T_KEY_RMS_GAMMA)
+
+    def randomize_gains(self, seed, spread=0.3):
+        """Replaces every RMSNorm gain vector (finalRMSNormGamma, rmsGamma, rmsGamma2, queryRMSGamma, keyRMSGamma;
+        the generators set them to 1 as an untrained model has them) by 1 + spread * U(-1, 1), every element its
+        own draw -- what a trained model.bin carries (load_model.cu:378-390, 411-450).  Deterministic in seed."""
+        rng = np.random.default_rng([int(seed), 0x6761696E])
+        t = self.tensor(0, T_FINAL_RMS_GAMMA)
+        t[:] = 1 + spread * rng.uniform(-1, 1, size=t.shape)
+        for layer in range(self.hparams.transformers):
+            for tid in self.GAIN_TENSORS[1:]:
+                t = self.tensor(layer, tid)
+                if t is not None:
+                    t[:] = 1 + spread * rng.uniform(-1, 1, size=t.shape)
+        return self
+
     def close(self):
         if self._h:
             host.mll_model_free(self._h)
@@ -354,6 +371,9 @@ class Device:
 
     def debug_inject_abort(self, launches):
         self._check(dev.mlh_debug_inject_abort(self._h, int(launches)))
+
+    def debug_inject_abort_at_step(self, step):
+        self._check(dev.mlh_debug_inject_abort_at_step(self._h, int(step)))
 
     def debug_set_xcd_tag(self, tags_used):
         self._check(dev.mlh_debug_set_xcd_tag(self._h, int(tags_used)))

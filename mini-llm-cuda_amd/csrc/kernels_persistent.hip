@@ -160,6 +160,7 @@ struct PersistArgs {
     float* kvPart;       // attention partials [heads * maxTiles * (hd + 2)]
     int maxTiles;
     int stageFloats;     // LDS staging vector length
+    int abortAtStep;     // test hook: > 0 makes workgroup 0 raise the abort flag when it reaches this step of the launch
     unsigned long long* timing; // optional (may be null): phase timestamps of workgroup 0 during the last step
 };
 
@@ -268,6 +269,7 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
     RowPf<WT> pf;
 
     for (int step = 0; step < P.steps; step++) {
+        if (P.abortAtStep > 0 && step == P.abortAtStep && wg == 0 && tid == 0) astu(P.abortFlag, 1u); // test hook: given up in mid-launch
         // embedding gather (inference.cu:9-22): every workgroup keeps its own copy of the residual stream
         for (int i = tid; i < d; i += PWG) xres[i] = PVec<WT>::one((const WT*)a.E + (size_t)tok * d + i);
         pf_first<WT>(pf, (const WT*)Ls[P.NL - 1].Wa, d, Ls[P.NL - 1].rowsA, d, gw, TW);
@@ -660,6 +662,20 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
 
 __global__ void k_set_word(unsigned* p, unsigned v) { *p = v; }
 
+// The barrier kernel stores the updated gated-delta-net state of every GDN layer at every step, so a launch that
+// gives up in mid-run has advanced the states of the steps it finished.  Before the launch the states of the
+// sequence are copied aside (blockIdx.y = layer, n floats per layer), and put back before the steps are redone.
+__global__ void k_gdn_snapshot(const LayerDev* layers, int seq, int n, float* snap, int restore) {
+    const LayerDev& L = layers[blockIdx.y];
+    if (L.kind != MLH_KIND_GDN) return;
+    f32x4* state = reinterpret_cast<f32x4*>(L.S + (size_t)seq * n);
+    f32x4* keep = reinterpret_cast<f32x4*>(snap + (size_t)blockIdx.y * n);
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n / 4; i += gridDim.x * blockDim.x) {
+        if (restore) state[i] = keep[i];
+        else keep[i] = state[i];
+    }
+}
+
 __global__ void k_zero_words(unsigned* p, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0u;
@@ -676,6 +692,10 @@ static int launch_persistent(mlh_ctx* c, PersistArgs& P, size_t ldsBytes) {
         int perCu = 0;
         MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, fn, PWG, ldsBytes));
         if (perCu < 1) { c->err = "persistent decode kernel does not fit on a compute unit"; return -1; }
+        if (GDK > 0 && !c->gdnSnapshot) {
+            int rc = mlh_dev_alloc_bytes(c, (void**)&c->gdnSnapshot, (size_t)c->hp.transformers * c->hp.gdnHeads * c->hp.gdnDk * c->hp.gdnDv * 4);
+            if (rc) return rc;
+        }
         c->persistentPrepared = true;
     }
     if (P.steps <= 0) return 0; // preparation only
@@ -684,13 +704,27 @@ static int launch_persistent(mlh_ctx* c, PersistArgs& P, size_t ldsBytes) {
     // occupancy query above says each unit can hold one.  A plain launch then behaves like a
     // cooperative one (and, unlike it, is visible to rocprofv3 and capturable in a graph); if some
     // unit were busy with other work the bounded barrier wait gives up and the call reports it.
-    static const bool coop = getenv("MLH_PERSIST_COOPERATIVE") != nullptr;
-    if (coop) {
+    if (GDK > 0) { // sequence 0's states as they are before the launch (see k_gdn_snapshot)
+        const int n = c->hp.gdnHeads * c->hp.gdnDk * c->hp.gdnDv;
+        hipLaunchKernelGGL(k_gdn_snapshot, dim3(std::min(64, (n / 4 + 255) / 256), c->hp.transformers), dim3(256), 0, c->stream,
+                           (const LayerDev*)c->d_layers, P.seq, n, c->gdnSnapshot, 0);
+    }
+    if (c->persistCooperative) {
         MLH_CHECK(c, hipLaunchCooperativeKernel(fn, dim3(c->numCUs), dim3(PWG), args, (unsigned)ldsBytes, c->stream));
     } else {
         hipLaunchKernelGGL((k_decode_persistent<WT, HD, GDK>), dim3(c->numCUs), dim3(PWG), ldsBytes, c->stream, P);
         MLH_CHECK(c, hipGetLastError());
     }
+    return 0;
+}
+
+// After a barrier-kernel launch that gave up: sequence 0's gated-delta-net states go back to what they were before it.
+int mlh_persistent_restore_states(mlh_ctx* c) {
+    if (!c->gdnSnapshot) return 0; // no GDN layers
+    const int n = c->hp.gdnHeads * c->hp.gdnDk * c->hp.gdnDv;
+    hipLaunchKernelGGL(k_gdn_snapshot, dim3(std::min(64, (n / 4 + 255) / 256), c->hp.transformers), dim3(256), 0, c->stream,
+                       (const LayerDev*)c->d_layers, 0, n, c->gdnSnapshot, 1);
+    MLH_CHECK(c, hipGetLastError());
     return 0;
 }
 
@@ -721,6 +755,7 @@ int mlh_launch_persistent(mlh_ctx* c, int steps) {
     P.kvPart = c->kvPart;
     P.maxTiles = c->pagesPerSeq;
     P.timing = c->d_timing;
+    P.abortAtStep = 0;
     int stage = std::max(std::max(hp.dim, hp.ffnDim), c->maxAd + hp.pleDim);
     stage = (stage + 3) & ~3;
     P.stageFloats = stage;
@@ -735,6 +770,8 @@ int mlh_launch_persistent(mlh_ctx* c, int steps) {
         // abort flag; test hook: a flag that starts raised makes every workgroup leave at its first wait
         hipLaunchKernelGGL(k_set_word, dim3(1), dim3(1), 0, c->stream, P.abortFlag, c->injectAbort > 0 ? 1u : 0u);
         if (c->injectAbort > 0) c->injectAbort--;
+        P.abortAtStep = c->injectAbortStep;
+        c->injectAbortStep = 0;
     }
     const bool bf = hp.weightDtype == MLH_DTYPE_BF16;
     if (hd == 64) {

@@ -64,6 +64,7 @@ struct XcdArgs {
     StepArgs a;
     const LayerDev* layers;
     int NL, steps, seq;
+    int abortAtStep;        // test hook: > 0 makes workgroup 0 give up when it reaches this step of the launch
     unsigned* abortFlag;
     unsigned* tagCounter;   // tags already used by earlier launches (advanced by workgroup 0 at the end)
     unsigned* xcdCount;     // [XCDS] zero at launch: workgroups that have arrived on each XCD
@@ -451,6 +452,7 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
     for (int step = 0; step < P.steps; step++) {
         // embedding gather (inference.cu:9-22): every workgroup keeps its own copy of the residual stream
         for (int i = lane; i < d; i += 64) S.xs[i] = PVec<WT>::one((const WT*)a.E + (size_t)tok * d + i);
+        if (P.abortAtStep > 0 && step == P.abortAtStep && wg == 0) ok = false; // test hook: a wait given up in mid-launch
 
         for (int t = P.NL - 1; t >= 0; t--) { // file block 0 is the top of the stack (inference.cu:384-385)
             const LayerDev& L = S.Ls[t];
@@ -1190,6 +1192,7 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
     P.NL = hp.transformers;
     P.steps = steps;
     P.seq = 0;
+    P.abortAtStep = 0;
     P.abortFlag = c->d_sync + 64 * 20;
     P.tagCounter = c->d_sync + 64 * 21;
     P.xcdCount = c->d_sync + 64 * 22;
@@ -1222,6 +1225,8 @@ int mlh_launch_xcd(mlh_ctx* c, int steps) {
         // test hook: arrival counters that start full make every workgroup give up before it touches anything
         const unsigned startCount = c->injectAbort > 0 ? (unsigned)XPER : 0u;
         if (c->injectAbort > 0) c->injectAbort--;
+        P.abortAtStep = c->injectAbortStep;
+        c->injectAbortStep = 0;
         hipLaunchKernelGGL(k_xcd_prep, dim3(1), dim3(64), 0, c->stream, P.abortFlag, P.xcdCount, startCount);
     }
     if (hp.weightDtype == MLH_DTYPE_BF16) {

@@ -215,6 +215,7 @@ extern "C" int mlh_create(const mlh_hparams* hpIn, int device, mlh_ctx** out) {
         c->err = "clearing the exchange words failed";
         return bail(-2);
     }
+    c->persistCooperative = getenv("MLH_PERSIST_COOPERATIVE") != nullptr; // like the knobs below: the environment is read here only
     if (getenv("MLH_PERSIST_TIMING") && (rc = dev_alloc(c, &c->d_timing, (size_t)16 * (hp.transformers + 1) + 4 * 256))) return bail(rc);
     c->copyBytes = (size_t)256 << 20; // calibration copy of MLH_K_COPY: the two buffers are allocated on its first use
     {   // tuning knobs of the XCD-rank kernel: read once, here
@@ -600,9 +601,11 @@ static bool use_persistent(const mlh_ctx* c, int nseq) {
     return nseq == 1 && c->usePersistent && c->temperature <= 0.f && mlh_persistent_supported(c);
 }
 
-// After the stream has drained: a single-launch decode that gave up a bounded wait leaves its flag set.  Nothing of
-// the sequence has advanced then (position, token, GDN states and the tag counter are written at the kernel's normal
-// end only), so the caller can run the same steps again another way.
+// After the stream has drained: a single-launch decode that gave up a bounded wait leaves its flag set.  The sequence
+// is then put back to where it was before the launch, so the caller can run the same steps again another way:
+// position, token and the tag counter are written at a kernel's normal end only; K/V rows of the steps that did run
+// are written again with the same values; the XCD-rank kernel keeps gated-delta-net states in LDS until its normal
+// end; the barrier kernel stores them at every step, and gets them back from the copy taken before its launch.
 static int check_persistent_abort(mlh_ctx* c) {
     if (c->d_timing) mlh_dump_persistent_timing(c);
     unsigned flag = 0;
@@ -613,8 +616,11 @@ static int check_persistent_abort(mlh_ctx* c) {
         if (c->usePersistent == 3 && mlh_xcd_supported(c)) { // tags of the abandoned launch must not be met again
             int rc = mlh_xcd_reset(c);
             if (rc) return rc;
-            MLH_CHECK(c, hipStreamSynchronize(c->stream));
+        } else {
+            int rc = mlh_persistent_restore_states(c);
+            if (rc) return rc;
         }
+        MLH_CHECK(c, hipStreamSynchronize(c->stream));
         return -3;
     }
     return 0;
@@ -818,6 +824,12 @@ extern "C" int mlh_persistent_fallbacks(mlh_ctx* c) { return c ? c->persistentFa
 extern "C" int mlh_debug_inject_abort(mlh_ctx* c, int launches) {
     if (!c || launches < 0) return -1;
     c->injectAbort = launches;
+    return 0;
+}
+
+extern "C" int mlh_debug_inject_abort_at_step(mlh_ctx* c, int step) {
+    if (!c || step < 0) return -1;
+    c->injectAbortStep = step;
     return 0;
 }
 

@@ -137,6 +137,9 @@ struct mlh_ctx {
                                    // 3: XCD ranks where the model and device allow it, else as 1
     int persistentFallbacks = 0;   // single-launch decode calls that gave up a wait and were redone as the kernel sequence
     int injectAbort = 0;           // test hook: the next n single-launch decode launches give up at their start
+    int injectAbortStep = 0;       // test hook: the next single-launch decode launch gives up when it reaches this step (> 0)
+    bool persistCooperative = false; // MLH_PERSIST_COOPERATIVE, read once at creation: cooperative launch of the barrier kernel
+    float* gdnSnapshot = nullptr;  // barrier kernel: sequence 0's GDN states as they were before the launch
     unsigned long long xcdTagNext = 0; // host mirror of the XCD-rank kernel's tag counter (tags used so far)
     bool xcdPrepared = false;      // function attribute and occupancy of the XCD-rank kernel checked
     bool persistentPrepared = false;
@@ -225,6 +228,7 @@ int mlh_launch_softmax_rows(mlh_ctx* c, const float* logits, float* probs, const
 // kernels_persistent.hip
 bool mlh_persistent_supported(const mlh_ctx* c);
 int mlh_launch_persistent(mlh_ctx* c, int steps);
+int mlh_persistent_restore_states(mlh_ctx* c);
 
 // measure_timing.hip: decodes and prints the phase clock stamps of the single-launch decode kernels
 // (collected only when MLH_PERSIST_TIMING is set at context creation)

@@ -41,8 +41,13 @@ def small_cfg(pkg, kind, **kw):
     return hp
 
 
-def make(pkg, orc, hp, seed, bf16=False):
+def make(pkg, orc, hp, seed, bf16=False, gains=True):
+    """Model, device context with it uploaded, oracle weights.  All five kinds of RMSNorm gain vector are
+    randomised (a trained model.bin carries such gains; the generators leave them at 1, where a kernel that
+    ignores a gain, indexes the per-head gains by channel only, or norms after RoPE would go unseen)."""
     model = pkg.Model.generate(hp, seed)
+    if gains:
+        model.randomize_gains(seed)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     w = orc.Weights.from_model(model, bf16=bf16)
@@ -81,7 +86,7 @@ def test_config1_golden_horizon(pkg, orc, persistent):
     import os
     from conftest import GOLDEN
     hp = pkg.config(1)
-    model, dev, w = make(pkg, orc, hp, seed=0)
+    model, dev, w = make(pkg, orc, hp, seed=0, gains=False)  # the committed outcome is configuration 1 as stated: gains 1
     dev.set_persistent(persistent)
     prompt = pkg.random_tokens(0, 0, hp.vocabSize, 16)
     ids, _ = dev.generate(prompt, 128)
@@ -202,6 +207,39 @@ def test_single_launch_gives_up_and_falls_back(pkg, orc, mode):
     dev.close()
 
 
+@pytest.mark.parametrize("mode,kind", [(3, "hybrid12"), (1, "hybrid"), (1, "hd128")], ids=["xcd", "barrier", "barrier-hd128"])
+def test_single_launch_gives_up_in_mid_run(pkg, orc, mode, kind):
+    """A single-launch decode that gives up AFTER some of its steps have run (forced from the host: workgroup 0
+    raises the flag itself when it reaches step 3 of 7, every workgroup then leaves at its next wait): the steps
+    that did run have appended K/V rows and -- in the barrier kernel -- stored updated gated-delta-net states.  The
+    redo as the kernel sequence must start from the states before the launch (a second application of the delta
+    rule would show in every later logit), so the whole call and what follows agree with the oracle."""
+    hp = _hybrid12(pkg) if kind == "hybrid12" else small_cfg(pkg, kind)
+    model, dev, w = make(pkg, orc, hp, seed=33)
+    dev.set_persistent(mode)
+    assert dev.xcd_decode_supported() == (mode == 3)
+    prompt = pkg.random_tokens(33, 0, hp.vocabSize, 50)
+    dev.prefill(0, prompt)
+    dec = orc.Decoder(w, "f64")
+    for t in prompt:
+        nxt, lg = dec.step(int(t))
+    tok = dev.greedy_token(0)
+    for n, hook in ((2, 0), (7, 3), (3, 0)):
+        if hook:
+            dev.set_persistent(mode)
+            dev.debug_inject_abort_at_step(hook)
+        out = dev.decode_loop([tok], n)[:, 0]
+        for t in [tok] + [int(v) for v in out[:-1]]:
+            nxt, lg = dec.step(t)
+        assert_logits_close(dev.logits(0), lg, FP32_RTOL, f"mode {mode} {kind}, launch of {n}")
+        tok = int(out[-1])
+        assert tok == nxt or abs(float(lg[tok]) - float(lg[nxt])) < GAP_TOL
+        if hook:
+            assert dev.get_persistent() == 0 and dev.persistent_fallbacks() == 1
+    assert dev.seq_len(0) == 50 + 12
+    dev.close()
+
+
 def test_xcd_tags_are_cleared_before_they_wrap(pkg, orc):
     """The XCD-rank kernel tags every exchanged word with a 32-bit running count of layer passes.  With the count
     set just below 2^32 the next launch must start from cleared words and count 0 instead of wrapping into tags
@@ -279,7 +317,7 @@ def test_bf16_weights(pkg, orc):
 def test_batched_equals_single(pkg, orc):
     """Sequences decoded together give what each gives alone (ragged lengths, shuffled KV pages)."""
     hp1 = small_cfg(pkg, "hybrid", maxSeqs=5)
-    model = pkg.Model.generate(hp1, 21)
+    model = pkg.Model.generate(hp1, 21).randomize_gains(21)
     dev = pkg.Device(hp1, 0)
     dev.upload(model)
     pages_per_seq = (hp1.maxL + 63) // 64

@@ -23,7 +23,7 @@ def _run_single(pkg, orc, cfg, seed, plen, launches):
     left behind by every launch (and by the prefill) are compared with the oracle's at that step."""
     hp = pkg.config(cfg)
     hp.maxSeqs = 1
-    model = pkg.Model.generate(hp, seed)
+    model = pkg.Model.generate(hp, seed).randomize_gains(seed)  # live oracle below: gains as a trained file has them
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     w = orc.Weights.from_model(model)
@@ -63,7 +63,7 @@ def test_teacher_forced_random_history(pkg, orc, cfg, path):
     T = 64, 65, 128, 129, 300 and 575 tokens (page boundaries at multiples of 64)."""
     hp = pkg.config(cfg)
     hp.maxSeqs = 1
-    model = pkg.Model.generate(hp, 40 + cfg)
+    model = pkg.Model.generate(hp, 40 + cfg).randomize_gains(40 + cfg)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     dev.set_persistent(path)
@@ -97,7 +97,7 @@ def test_config4_batch64(pkg, orc):
     the gap rule, logits after the prefill and after the 32 steps."""
     hp = pkg.config(4)
     nseq = hp.maxSeqs
-    model = pkg.Model.generate(hp, 4)
+    model = pkg.Model.generate(hp, 4).randomize_gains(4)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     w = orc.Weights.from_model(model)
@@ -129,7 +129,7 @@ def test_config4_teacher_forced_batch(pkg, orc):
     oracle after steps 1, 12 and 24."""
     hp = pkg.config(4)
     nseq = hp.maxSeqs
-    model = pkg.Model.generate(hp, 44)
+    model = pkg.Model.generate(hp, 44).randomize_gains(44)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     w = orc.Weights.from_model(model)
@@ -165,7 +165,7 @@ def test_config5_bf16_prefill_and_decode(pkg, orc):
     hp = pkg.config(5)
     hp.maxSeqs = 8
     hp.maxL = 256
-    model = pkg.Model.generate(hp, 5)
+    model = pkg.Model.generate(hp, 5).randomize_gains(5)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     w = orc.Weights.from_model(model, bf16=True)
@@ -203,7 +203,7 @@ def test_config5_width_prefill_2048_tokens(pkg, orc):
     logit (bf16 path); the error must not grow along the sequence beyond it."""
     hp = pkg.config(5, transformers=4, vocabSize=4096, maxL=2048, maxSeqs=1)
     pkg.set_layer_pattern(hp, 3)
-    model = pkg.Model.generate(hp, 55)
+    model = pkg.Model.generate(hp, 55).randomize_gains(55)
     w = orc.Weights.from_model(model, bf16=True)
     toks = pkg.random_tokens(55, 0, hp.vocabSize, 2048)
     want = orc.forward_full(w, toks, "f64", last_only=False)["logits"]  # [2048, V]; about half a minute of CPU
@@ -475,4 +475,47 @@ def test_reference_default_shape_teacher_forced_full_context(pkg):
         assert_logits_close(lg[int(r)], wl, FP32_RTOL, f"reference-default shape, position {int(r)}")
         assert np.max(np.abs(pr[int(r)] - wp)) <= 1e-6 + FP32_RTOL * np.max(wp)
     print(f"reference-default shape, 1280 positions: mean loss {nll:.5f} (oracle {want_nll:.5f}), {int(other.sum())} picks differ within the tie rule")
+    dev.close()
+
+
+@pytest.mark.parametrize("path", [3, 0], ids=["default", "kernels"])
+@pytest.mark.parametrize("shape", ["config2_flags", "reference_default"])
+def test_full_size_both_flags_random_gains_live_oracle(pkg, orc, shape, path):
+    """Full-size models with QK-norm and query gating on AND every gain vector away from 1 (the committed horizons
+    above are configurations as stated, gains 1): configuration 2 with both flags, and the shape the reference ships
+    compiled in (network_meta.h:3-20), a 64-token prompt and 245 greedy steps on the default decode path and on the
+    kernel sequence, against the float64 oracle run live: ids by the gap rule, logits after the prefill and at the
+    end of every launch (steps 1, 64, 65, 165, 245).  A teacher-forced pass over a random 150-token history follows
+    through mlh_forward_full (every position's logits)."""
+    if shape == "config2_flags":
+        hp = pkg.config(2, qkRmsNorm=1, queryGating=1)
+        hp.maxSeqs = 1
+        model = pkg.Model.generate(hp, 71)
+    else:
+        hp = pkg.reference_defaults()
+        model = pkg.Model.new(hp)
+        model.init_uniform(72, 0.02)
+    model.randomize_gains(7, spread=0.4)
+    dev = pkg.Device(hp, 0)
+    dev.upload(model)
+    dev.set_persistent(path)
+    w = orc.Weights.from_model(model)
+    prompt = pkg.random_tokens(71, 0, hp.vocabSize, 64)
+    dev.prefill(0, prompt)
+    ids = [dev.greedy_token(0)]
+    logits = {0: dev.logits(0)}
+    for n in (1, 63, 1, 100, 80):
+        ids += [int(t) for t in dev.decode_loop([ids[-1]], n)[:, 0]]
+        logits[len(ids) - 1] = dev.logits(0)
+    dec = orc.Decoder(w, "f64")
+    exact, tol = check_greedy_against_oracle(dec, prompt, ids, GAP_TOL, logits, FP32_RTOL, what=f"{shape} path {path}")
+    assert exact + tol == len(ids)
+    print(f"{shape} path {path} with random gains: {exact} ids exact, {tol} within the tie rule, {len(set(ids))} distinct")
+    if path == 3:
+        dev.reset()
+        toks = pkg.random_tokens(73, 0, hp.vocabSize, 150)
+        lg, _, _ = dev.forward_full(0, toks, want_probs=False)
+        ref = orc.forward_full(w, toks, "f64", last_only=False)["logits"]
+        for i in range(len(toks)):
+            assert_logits_close(lg[i], ref[i], FP32_RTOL, f"{shape} forward position {i}")
     dev.close()

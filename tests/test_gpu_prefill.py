@@ -347,6 +347,7 @@ def test_reference_default_architecture(pkg, orc):
     hp.maxL = 128
     model = pkg.Model.new(hp)
     model.init_uniform(9, 0.02)
+    model.randomize_gains(9)
     dev = pkg.Device(hp, 0)
     dev.upload(model)
     w = orc.Weights.from_model(model)

@@ -437,6 +437,109 @@ def test_ple_branch_closed_form(pkg, orc):
     assert np.allclose(hid3[0], h1 + W2 @ ((a / (1 + np.exp(-a))) * (W1B @ hn)), rtol=1e-9, atol=1e-12)
 
 
+def test_attention_block_with_both_flags_closed_form(pkg, orc):
+    """One attention block with per-head QK RMSNorm and query gating on, random gains (rmsGamma,
+    queryRMSGamma, keyRMSGamma), random gate weights, Wo = I and the FFN off, so that hidden = x + gated attention
+    output.  Compared with an independent NumPy statement of inference.cu:467-483 (per-head norm with
+    gamma[h*hd + i], THEN RoPE) and inference.cu:486-508, 241-250 (gate = sigmoid(Wg xn) from the normed input,
+    applied before Wo).  Each plausible mistake is also formed in NumPy and must lie far outside the bound:
+    norm after RoPE, a head-shared gain gamma[i % hd], the gate taken from x instead of xn, the gate applied
+    after Wo (shown with a non-identity Wo), and a missing RMS1 gain."""
+    H, hd = 2, 64
+    d = H * hd
+    hp = pkg.config(1, dim=d, attnHeads=H, headDim=hd, ffnDim=64, transformers=1, vocabSize=32, maxL=8,
+                    qkRmsNorm=1, queryGating=1)
+    model = pkg.Model.generate(hp, 21)
+    rng = np.random.default_rng(21)
+    model.tensor(0, 2)[:] = 1 + 0.3 * rng.uniform(-1, 1, size=d)      # rmsGamma
+    model.tensor(0, 11)[:] = 1 + 0.5 * rng.uniform(-1, 1, size=d)     # queryRMSGamma: distinct per head and channel
+    model.tensor(0, 12)[:] = 1 + 0.5 * rng.uniform(-1, 1, size=d)     # keyRMSGamma
+    for tid in (3, 4, 5):
+        model.tensor(0, tid)[:] = rng.normal(size=(d, d)) * 0.3
+    model.tensor(0, 13)[:] = rng.normal(size=(d, d)) * 0.2            # gate pre-activations O(1)
+    model.tensor(0, 6)[:] = np.eye(d, dtype=np.float32)               # Wo = I
+    model.tensor(0, 8)[:] = 0                                         # FFN off
+    model.tensor(0, 0)[:] = rng.normal(size=(32, d))                  # embeddings of visible size
+    E = model.tensor(0, 0).astype(np.float64)
+    g1, gq, gk = (model.tensor(0, t).astype(np.float64) for t in (2, 11, 12))
+    Wq, Wk, Wv, Wg = (model.tensor(0, t).astype(np.float64) for t in (3, 4, 5, 13))
+    tab = pkg.rope_table(hp.maxL, hd).astype(np.float64)              # the table itself is pinned elsewhere
+    toks = np.array([3, 7, 11, 5], np.int32)
+
+    def head_norm(v, gamma, shared=False):
+        out = np.empty_like(v)
+        for h in range(H):
+            s = slice(h * hd, (h + 1) * hd)
+            r = np.sqrt(np.mean(v[s] ** 2) + 1e-8)
+            out[s] = (gamma[:hd] if shared else gamma[s]) * (v[s] / r)
+        return out
+
+    def rope(v, pos):
+        out = np.empty_like(v)
+        for h in range(H):
+            for i in range(hd // 2):
+                a, b = v[h * hd + 2 * i], v[h * hd + 2 * i + 1]
+                c, s = tab[pos, 2 * i], tab[pos, 2 * i + 1]
+                out[h * hd + 2 * i], out[h * hd + 2 * i + 1] = a * c - b * s, a * s + b * c
+        return out
+
+    def block(Wo=None, norm_after_rope=False, shared_gain=False, gate_from_x=False, gate_after_wo=False,
+              no_rms1_gain=False):
+        Ks, Vs, hid = [], [], []
+        for pos, t in enumerate(toks):
+            x = E[t]
+            xn = x / np.sqrt(np.mean(x * x) + 1e-8)
+            if not no_rms1_gain:
+                xn = g1 * xn
+            q, k, v = Wq @ xn, Wk @ xn, Wv @ xn
+            if norm_after_rope:
+                q, k = head_norm(rope(q, pos), gq, shared_gain), head_norm(rope(k, pos), gk, shared_gain)
+            else:
+                q, k = rope(head_norm(q, gq, shared_gain), pos), rope(head_norm(k, gk, shared_gain), pos)
+            Ks.append(k)
+            Vs.append(v)
+            a = np.empty(d)
+            for h in range(H):
+                s = slice(h * hd, (h + 1) * hd)
+                sc = np.array([kk[s] @ q[s] for kk in Ks]) / np.sqrt(hd)
+                p = np.exp(sc - sc.max())
+                p /= p.sum()
+                a[s] = sum(pj * vv[s] for pj, vv in zip(p, Vs))
+            gate = 1 / (1 + np.exp(-(Wg @ (x if gate_from_x else xn))))
+            if Wo is None:
+                hid.append(a * gate + x)
+            elif gate_after_wo:
+                hid.append((Wo @ a) * gate + x)
+            else:
+                hid.append(Wo @ (a * gate) + x)
+        return np.array(hid)
+
+    want = block()
+    w = orc.Weights.from_model(model)
+    hid = orc.forward_full(w, toks, "f64", want_hidden=True)["hidden"]
+    assert np.allclose(hid, want, rtol=1e-9, atol=1e-12)
+    # the same block through the cached decode path (logits are a fixed function of hidden)
+    dec = orc.Decoder(w, "f64")
+    for t in toks:
+        _, lg = dec.step(int(t))
+    assert np.allclose(lg, orc.forward_full(w, toks, "f64")["logits"][0], rtol=1e-11, atol=1e-13)
+    # float32 oracle agrees to float precision
+    hid32 = orc.forward_full(w, toks, "f32", want_hidden=True)["hidden"]
+    assert np.max(np.abs(hid32 - want)) < 2e-5 * np.max(np.abs(want))
+    # each mistake named above is far outside the bound at positions >= 1 (position 0 has RoPE = identity)
+    scale = np.max(np.abs(want[1:] - E[toks[1:]]))
+    for wrong in (dict(norm_after_rope=True), dict(shared_gain=True), dict(gate_from_x=True),
+                  dict(no_rms1_gain=True)):
+        assert np.max(np.abs(block(**wrong)[1:] - want[1:])) > 1e-2 * scale, wrong
+    # gate before Wo, not after: needs a Wo that is not the identity
+    Wo = rng.normal(size=(d, d)) * 0.3
+    model.tensor(0, 6)[:] = Wo
+    Wo = model.tensor(0, 6).astype(np.float64)
+    hid_wo = orc.forward_full(orc.Weights.from_model(model), toks, "f64", want_hidden=True)["hidden"]
+    assert np.allclose(hid_wo, block(Wo=Wo), rtol=1e-9, atol=1e-12)
+    assert np.max(np.abs(block(Wo=Wo, gate_after_wo=True) - hid_wo)) > 1e-2 * np.max(np.abs(hid_wo))
+
+
 def test_greedy_pick_takes_lowest_index_on_ties(pkg, orc):
     hp = pkg.config(1, dim=128, attnHeads=2, headDim=64, ffnDim=192, transformers=1, vocabSize=64, maxL=8)
     model = pkg.Model.generate(hp, 1)
