@@ -83,8 +83,7 @@ def decode_bytes_per_token(hp, T, wbytes=4):
     return total
 
 
-def cpu_baseline(model, hp, prompt, seconds_budget=20.0):
-    """Reference-style CPU generation (full recompute per token) on a bounded sample."""
+def _cpu_model(model, hp):
     import torch
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import cpu_model
@@ -96,33 +95,102 @@ def cpu_baseline(model, hp, prompt, seconds_budget=20.0):
     for l in range(hp.transformers):
         for tid in range(2, 11):
             tensors[(l, tid)] = model.tensor(l, tid)
-    cm = cpu_model.CpuModel(hp, tensors, threads=threads)
-    cm.generate_full(prompt, 1)  # warm-up
-    n_full, ids_full = 0, []
-    seq = list(int(t) for t in prompt)
-    t0 = time.perf_counter()
-    while n_full < 64 and (time.perf_counter() - t0) < seconds_budget * 0.6:
-        nxt = int(torch.argmax(cm.forward(seq)))
-        seq.append(nxt)
-        ids_full.append(nxt)
-        n_full += 1
-    t_full = time.perf_counter() - t0
-    t1 = time.perf_counter()
-    ids_cached = cm.generate_cached(prompt, 128)
-    t_cached = time.perf_counter() - t1
+    return cpu_model.CpuModel(hp, tensors, threads=threads), cpu_model, torch
+
+
+def cpu_baseline_one(what, model, hp, prompt, gpu_ids, n_full, n_cached, runs=3):
+    """The PyTorch restatement of the reference's pytorch_verification model on this host's cores: after a warm-up,
+    `runs` repetitions each of n_full greedy tokens in the reference's algorithmic form (every token recomputes all
+    positions, inference_orchestrator.cu:64-65) and of n_cached tokens with a KV cache; medians are reported.  The
+    ids are compared with the GPU's for the same prompt (fp32 on both sides: equal unless two logits tie)."""
+    cm, cpu_model, torch = _cpu_model(model, hp)
+    cm.generate_full(prompt, 2)  # warm-up
+    full, cached, ids_full, ids_cached = [], [], None, None
+    for _ in range(runs):
+        ids_full, dt = cpu_model.time_generation(cm, prompt, n_full, "full")
+        full.append(n_full / dt)
+    for _ in range(runs):
+        ids_cached, dt = cpu_model.time_generation(cm, prompt, n_cached, "cached")
+        cached.append(n_cached / dt)
+    gpu = [int(t) for t in gpu_ids]
     return {
-        "value": n_full / t_full,
-        "unit": "tok/s",
-        "cores": torch.get_num_threads(),
-        "kind": "port",
-        "sample": (f"config 2, {n_full} greedy tokens after the {len(prompt)}-token prompt, full recompute of all "
-                   f"positions per token as the reference's runInferenceLoop does; PyTorch {torch.__version__} CPU fp32"),
-        "with_kv_cache_tok_s": 128 / t_cached,
-        "host_cpu_count": os.cpu_count(),
-        "host_physical_cores": physical_cores(),
-        "first_ids": ids_full[:8],
-        "first_ids_cached": ids_cached[:8],
+        "value": stats(full)["median"], "unit": "tok/s", "cores": torch.get_num_threads(), "kind": "port",
+        "value_stats": stats(full),
+        "sample": (f"{what}: {n_full} greedy tokens after the {len(prompt)}-token prompt, full recompute of all positions "
+                   f"per token as the reference's runInferenceLoop does, median of {runs} runs after a warm-up; "
+                   f"PyTorch {torch.__version__} CPU fp32"),
+        "with_kv_cache_tok_s": stats(cached)["median"], "with_kv_cache_stats": stats(cached),
+        "with_kv_cache_sample": f"{n_cached} greedy tokens, median of {runs} runs",
+        "host_cpu_count": os.cpu_count(), "host_physical_cores": physical_cores(),
+        "first_ids": ids_full[:8], "first_ids_cached": ids_cached[:8],
+        "ids_equal_gpu": (ids_full[:len(gpu)] == gpu[:len(ids_full)] and ids_cached[:len(gpu)] == gpu[:len(ids_cached)]),
+        "ids_compared": [min(len(gpu), len(ids_full)), min(len(gpu), len(ids_cached))],
     }
+
+
+def config1_decode_leg(m, steps=128):
+    """Configuration 1 (the pytorch_verification class of model: d256, 4 layers, 4 heads x 64, ffn 704, vocab 4096,
+    fp32, seed 0, 16-token prompt, 128 greedy steps) on the GPU.  Its 17 MB of weights stay in the 256 MB Infinity
+    Cache (and mostly in the L2s), so no HBM-bandwidth fraction is claimed for it: tok/s only."""
+    hp = m.config(1)
+    model = m.Model.generate(hp, seed=0)
+    prompt = m.random_tokens(0, 0, hp.vocabSize, 16)
+    dev = m.Device(hp, 0)
+    dev.upload(model)
+    walls, ids = [], None
+    for i in range(REPS + 1):  # the first repetition is the warm-up
+        dev.reset()
+        dev.prefill(0, prompt)
+        first = dev.greedy_token(0)
+        dev.synchronize()
+        t0 = time.perf_counter()
+        out = dev.decode_loop([first], steps - 1)
+        dev.synchronize()
+        if i > 0:
+            walls.append(time.perf_counter() - t0)
+        ids = [first] + [int(t) for t in out[:, 0]]
+    wall = stats(walls)["median"]
+    path = {0: "kernels", 1: "persistent", 3: "xcd" if dev.xcd_decode_supported() else "persistent"}[dev.get_persistent()]
+    dev.close()
+    return ({"workload": "config 1: batch-1 greedy decode, d256 x 4 layers x 4 heads x 64, ffn 704, vocab 4096, fp32 weights "
+                         "seed 0, 16-token prompt, 128 greedy tokens", "steps": steps - 1, "tok_s": (steps - 1) / wall,
+             "ms_per_step": wall / (steps - 1) * 1e3, "ms_per_step_stats": stats([w / (steps - 1) * 1e3 for w in walls]),
+             "decode_path": path, "weights_bytes": decode_bytes_per_token(hp, 0) - hp.transformers * 2 * hp.dim * 4,
+             "weights_resident_in_infinity_cache": True,
+             "note": "17 MB of weights: cache-resident, latency-bound; no bandwidth fraction claimed", "first_ids": ids[:8]},
+            model, hp, prompt, ids)
+
+
+def reference_default_decode_leg(m, steps=256):
+    """The shape the reference ships compiled in (network_meta.h:3-20: dim 768, 6 heads x 128, ffn 3072, 16 layers,
+    vocabulary 20160, QK-norm and query gating on, maxL 1280) with its uniform +-0.02 init (random_weights.cu:15-25,
+    own generator): batch-1 greedy decode after a 256-token prompt -- what a user of the reference's main() runs."""
+    hp = m.reference_defaults()
+    plen, warm = 256, 16
+    model = m.Model.new(hp)
+    model.init_uniform(9, 0.02)
+    dev = m.Device(hp, 0)
+    dev.upload(model)
+    dev.prefill(0, m.random_tokens(9, 0, hp.vocabSize, plen))
+    out = dev.decode_loop([dev.greedy_token(0)], warm)
+    steps = min(steps, (hp.maxL - plen - warm) // REPS)
+    walls = []
+    for _ in range(REPS):
+        dev.synchronize()
+        t0 = time.perf_counter()
+        out = dev.decode_loop([int(out[-1, 0])], steps)
+        dev.synchronize()
+        walls.append(time.perf_counter() - t0)
+    wall = stats(walls)["median"]
+    nbytes = float(np.mean([decode_bytes_per_token(hp, plen + warm + 1 + i) for i in range(REPS * steps)]))
+    path = {0: "kernels", 1: "persistent", 3: "xcd" if dev.xcd_decode_supported() else "persistent"}[dev.get_persistent()]
+    fell_back = dev.persistent_fallbacks()
+    dev.close()
+    return {"workload": "reference-default shape: batch-1 greedy decode, d768 x 16 layers x 6 heads x 128, ffn 3072, vocab 20160, "
+                        "QK-norm + query gating, fp32 uniform +-0.02, 256-token prompt", "steps": steps,
+            "ms_per_step": wall / steps * 1e3, "tok_s": steps / wall, "ms_per_step_stats": stats([w / steps * 1e3 for w in walls]),
+            "decode_path": path, "fallbacks": fell_back, "bytes_per_token": nbytes, "achieved_GBps": nbytes / (wall / steps) / 1e9,
+            "frac_of_hbm_peak": nbytes / (wall / steps) / 1e9 / HBM_PEAK_GBPS, "last_ids": [int(x) for x in out[-4:, 0]]}
 
 
 def matrix_params(hp):
@@ -205,7 +273,7 @@ def hybrid_decode_leg(m, steps=192):
             "frac_of_hbm_peak": nbytes / (wall / steps) / 1e9 / HBM_PEAK_GBPS, "last_ids": [int(x) for x in out[-4:, 0]]}
 
 
-def prefill_leg(m, reps=REPS):
+def prefill_leg(m, reps=REPS, with_gemm=True):
     """Configuration 5: 8 prompts of 2048 uniform-random tokens through the bf16 model in one pass.
     MFMA utilisation = algorithmic flops (projections + causal attention, LM head on the last position
     only) / time / the published dense bf16 peak; the GEMM kernel alone is also timed on the pass's own
@@ -238,7 +306,7 @@ def prefill_leg(m, reps=REPS):
         decs.append((time.perf_counter() - t0) / 16)
     dec = stats(decs)["median"]
     dev.close()
-    gemm = gemm_leg(m, iters=10, reps=REPS)
+    gemm = gemm_leg(m, iters=10, reps=REPS) if with_gemm else None
     return {"workload": "config 5: 8 x 2048-token prompts, d2048 x 24 layers (3 GDN : 1 attention), 16 heads x 128, "
                         "ffn 5632, vocab 32000, PLE 64, bf16 weights, fp32 accumulation",
             "tokens": tokens, "ms": med * 1e3, "ms_stats": stats([t * 1e3 for t in times]), "tok_s": tokens / med,
@@ -251,12 +319,11 @@ def prefill_leg(m, reps=REPS):
 
 def gemm_leg(m, iters=3, reps=1):
     """The gate/up product of one config-5 prefill pass alone (16384 x 11264 x 2048, half operands -- what the bf16
-    model's MFMA path multiplies --, N(0,1) data), timed with HIP events.  The headline figure is the product as the pass
-    runs it: SiLU(gate) * up in the epilogue, half output, one launch at a time with the device idle in between (in the
-    pass a GEMM is followed by lighter kernels, not by nine more GEMMs, and under real operand data the part's clock
-    depends on how long the load has lasted).  Beside it: the same launch ten times back to back, the plain fp32 epilogue
-    back to back, the kernel on all-zero operands and the vendor library on the same operands.  With reps == 1 (profiler
-    and counter runs) both epilogues are launched `iters` times and only the plain timing is reported."""
+    model's MFMA path multiplies --, N(0,1) data), timed with HIP events: SiLU(gate) * up in the epilogue, half output,
+    as the pass runs it.  Top level: ten launches back to back (sustained clock).  Beside it: single launches with the
+    device idle in between, the plain fp32 epilogue back to back, the kernel on all-zero operands and the vendor library
+    on the same operands.  With reps == 1 (profiler and counter runs) both epilogues are launched `iters` times and
+    only the plain timing is reported."""
     hp = m.config(5)
     M = 8 * 2048
     rng = np.random.default_rng(5)
@@ -278,10 +345,17 @@ def gemm_leg(m, iters=3, reps=1):
     for _ in range(9):
         time.sleep(0.05)
         singles.append(m.selftest_gemm(a, b, None, f16=True, iters=1, swiglu=True)[1])
-    out = fig(singles)
+    # Two protocols, both reported with the same weight.  Sustained: `iters` launches back to back (HIP events around
+    # the run, median of `reps` runs) -- the part's clock settles under the load; this is the figure comparable
+    # from round to round and with the vendor yardstick below, and the one at the top level of this object.  Single:
+    # one launch at a time with 50 ms of idle before it -- the clock has not come down yet; in the prefill pass a
+    # GEMM is followed by lighter kernels and runs between the two (the profiler's per-kernel average says where).
+    b2b = [m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)[1] for _ in range(reps)]
+    out = fig(b2b)
     out.update({"shape": [M, 2 * hp.ffnDim, hp.dim], "epilogue": "SiLU(gate) * up, half output (as the prefill pass runs this product)",
-                "protocol": "median of 9 single launches, 50 ms idle before each, HIP events around the launch"})
-    out["back_to_back_%d_launches_swiglu_epilogue" % iters] = fig([m.selftest_gemm(a, b, None, f16=True, iters=iters, swiglu=True)[1] for _ in range(reps)])
+                "protocol": "%d launches back to back, HIP events around the run, median of %d runs" % (iters, reps)})
+    out["back_to_back_%d_launches_swiglu_epilogue" % iters] = fig(b2b)
+    out["single_launches_idle_between"] = dict(fig(singles), protocol="median of 9 single launches, 50 ms idle before each, HIP events around the launch")
     plain = fig([m.selftest_gemm(a, b, None, f16=True, iters=iters)[1] for _ in range(reps)])
     out["back_to_back_%d_launches_plain_fp32_epilogue" % iters] = plain
     # Two yardsticks on the same box in the same run, neither on the product path: the same kernel on all-zero
@@ -347,7 +421,7 @@ def timed_decode(dev, prompt, K, W, persistent, maxL):
         dev.reset()
         dev.prefill(0, prompt)
         events.append(dev.time_decode([first], K))
-    return walls, events, ids
+    return walls, events, np.concatenate([[first], ids[:, 0]]).astype(np.int32)
 
 
 def main():
@@ -359,9 +433,10 @@ def main():
     ap.add_argument("--path", choices=["xcd", "persistent", "kernels"], default="xcd",
                     help="decode path reported as `value`")
     ap.add_argument("--no-extras", action="store_true", help="skip the batched-decode (config 4) and prefill (config 5) legs")
-    ap.add_argument("--leg", choices=["all", "batched", "prefill", "gemm", "hybrid"], default="all",
-                    help="profiler runs: run only the batched-decode leg, the prefill leg, the big GEMM alone or the "
-                         "batch-1 hybrid decode leg and print its JSON object")
+    ap.add_argument("--leg", choices=["all", "batched", "prefill", "gemm", "hybrid", "config1", "refdefault"], default="all",
+                    help="profiler runs: run only the batched-decode leg, the prefill leg, the big GEMM alone, the "
+                         "batch-1 hybrid decode leg, configuration 1 or the reference-default shape and print its JSON object")
+    ap.add_argument("--passes", type=int, default=2, help="--leg prefill: timed passes over the 8 x 2048-token batch")
     ap.add_argument("--only-path", action="store_true", help="time only the chosen path (for profiler runs)")
     ap.add_argument("--graph-steps", type=int, default=0,
                     help="kernels path: decode steps per hipGraph replay; 0 = plain launches (use 0 under rocprofv3)")
@@ -373,8 +448,9 @@ def main():
 
     m = entry.load_package()
     if args.leg != "all":
-        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=2), "gemm": gemm_leg,
-               "hybrid": hybrid_decode_leg}[args.leg]
+        leg = {"batched": batched_decode_leg, "prefill": lambda mm: prefill_leg(mm, reps=max(1, args.passes), with_gemm=False),
+               "gemm": gemm_leg, "hybrid": hybrid_decode_leg, "config1": lambda mm: config1_decode_leg(mm)[0],
+               "refdefault": reference_default_decode_leg}[args.leg]
         print(json.dumps({args.leg: leg(m)}))
         return 0
     hp = m.config(2)
@@ -399,7 +475,7 @@ def main():
         paths[name] = {"tok_s": K / wall, "ms_per_step": wall / K * 1e3, "ms_per_step_stats": stats([w / K * 1e3 for w in walls]),
                        "event_ms_per_step": stats(events)["median"] / K,
                        "event_ms_per_step_stats": stats([e / K for e in events])}
-        ids_by_path[name] = ids[:, 0]
+        ids_by_path[name] = ids  # the token the prefill picked, then the K decoded ones
         if dev.persistent_fallbacks():
             print(f"bench.py: path {name} gave up a wait and fell back to the kernel sequence: {m.dev.mlh_last_error(dev._h).decode()}", file=sys.stderr)
             return 5
@@ -448,6 +524,14 @@ def main():
                 "layer_floor_formula": "2 x (cross + in-XCD gather) + 3 x in-XCD, compute phases not counted"}
     except Exception as e:  # a probe, never required
         hops = {"failed": repr(e)}
+    try:  # what the matrix cores sustain from registers alone, by instruction form and operand data, and the load path alone
+        mfma = {"what": "register-only half-precision MFMA loop on every SIMD, TFLOP/s (nominal dense peak 2500); the part's "
+                        "clock follows the power the operand data draws",
+                "mfma_32x32x16": {"zeros": dev.probe_mfma(0, 0), "unit_variance": dev.probe_mfma(0, 1)},
+                "mfma_16x16x32": {"zeros": dev.probe_mfma(1, 0), "unit_variance": dev.probe_mfma(1, 1)},
+                "direct_to_lds_loads_TBps": dev.probe_lds_loads()}
+    except Exception as e:
+        mfma = {"failed": repr(e)}
 
     if args.path in ("persistent", "xcd"):
         # the dominant (only) kernel: one launch = K tokens; duration from HIP events around the launch (median of REPS)
@@ -485,14 +569,22 @@ def main():
     cpu = None
     if not args.no_cpu:
         try:
-            cpu = cpu_baseline(model, hp, prompt)
+            cpu = cpu_baseline_one("config 2", model, hp, prompt, ids, n_full=32, n_cached=96)
         except Exception as e:  # the baseline is reported, never required
             cpu = {"value": None, "unit": "tok/s", "cores": 0, "kind": "port", "sample": f"failed: {e!r}"}
 
     dev.close()
     extras = {}
     if not args.no_extras and not args.only_path:
-        for name, leg in (("batched_decode", batched_decode_leg), ("hybrid_decode", hybrid_decode_leg), ("prefill", prefill_leg)):
+        try:  # configuration 1 on the GPU, and the same workload on the host cores beside it
+            extras["config1_decode"], model1, hp1, prompt1, ids1 = config1_decode_leg(m)
+            if cpu is not None and cpu.get("value"):
+                cpu["config1"] = cpu_baseline_one("config 1", model1, hp1, prompt1, ids1, n_full=64, n_cached=127)
+            del model1
+        except Exception as e:
+            extras["config1_decode"] = {"failed": repr(e)}
+        for name, leg in (("reference_default_decode", reference_default_decode_leg), ("batched_decode", batched_decode_leg),
+                          ("hybrid_decode", hybrid_decode_leg), ("prefill", prefill_leg)):
             try:
                 extras[name] = leg(m)
             except Exception as e:  # reported alongside, never required for the headline line
@@ -523,9 +615,11 @@ def main():
         "paths": paths,
         "protocol": f"median of {REPS} timed repetitions per figure (min and max beside it)",
         "exchange_latency": hops,
+        "mfma_register_loop": mfma,
         "kernels": kernels,
         "copy_kernel": {"avg_us": round(copy_us, 2), "GBps": round(copy_bytes / copy_us / 1e3, 1)},
         "cpu_baseline": cpu,
+        "first_ids": [int(x) for x in ids[:8]],
         "last_ids": [int(x) for x in ids[-4:]],
     }
     line.update(extras)

@@ -259,6 +259,17 @@ int mlh_profile_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int ste
  * counterpart in the reference. */
 int mlh_probe_hops(mlh_ctx* ctx, int iters, double* us);
 
+/* Two yardsticks under the prefill GEMM's ceiling (measurement support; no counterpart in the reference, nothing on
+ * the product path calls them).  mlh_probe_mfma: TFLOP/s of a register-only half-precision MFMA loop on every SIMD
+ * of the device (no LDS, no memory): form 0 = v_mfma_f32_32x32x16_f16, 1 = v_mfma_f32_16x16x32_f16; data 0 =
+ * all-zero operands, 1 = pseudo-random operands of unit variance; `iters` loop iterations of 16 (form 0) or 32
+ * (form 1) MFMAs per wave, eight waves per compute unit.  The part sets its clock by the power the data draws, so
+ * the four figures say how much of the nominal peak each instruction form keeps on real operands.
+ * mlh_probe_lds_loads: TB/s of the GEMM's direct global -> LDS load pattern alone (every workgroup streams `slices`
+ * 64 KB K slices into LDS, operands resident in its XCD's L2, nothing multiplied). */
+int mlh_probe_mfma(mlh_ctx* ctx, int form, int data, int iters, double* tflops);
+int mlh_probe_lds_loads(mlh_ctx* ctx, int slices, double* tb_per_s);
+
 /* Times `steps` decode steps (graph replays, argmax fed back on the device)
  * with HIP events on the context's stream: total milliseconds. */
 int mlh_time_decode(mlh_ctx* ctx, const int32_t* first_ids, int nseq, int steps, double* total_ms);

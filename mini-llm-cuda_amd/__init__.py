@@ -104,6 +104,8 @@ _sigs_dev = {
     "mlh_gemm_device_init": (c_int, [c_int]),
     "mlh_gemm_device": (c_int, [c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "mlh_probe_hops": (c_int, [c_void_p, c_int, _P(c_double)]),
+    "mlh_probe_mfma": (c_int, [c_void_p, c_int, c_int, c_int, _P(c_double)]),
+    "mlh_probe_lds_loads": (c_int, [c_void_p, c_int, _P(c_double)]),
     "mlh_profile_decode": (c_int, [c_void_p, c_void_p, c_int, c_int, _P(c_double), _P(c_int32)]),
 }
 _sigs_host = {
@@ -394,6 +396,19 @@ class Device:
         us = (c_double * 3)()
         self._check(dev.mlh_probe_hops(self._h, iters, us))
         return tuple(us)
+
+    def probe_mfma(self, form, data, iters=20000):
+        """TFLOP/s of a register-only half-precision MFMA loop on every SIMD: form 0 = 32x32x16, 1 = 16x16x32;
+        data 0 = all-zero operands, 1 = unit-variance operands."""
+        t = c_double()
+        self._check(dev.mlh_probe_mfma(self._h, form, data, iters, byref(t)))
+        return t.value
+
+    def probe_lds_loads(self, slices=4000):
+        """TB/s of the GEMM's direct global -> LDS load pattern alone (L2-resident operands, nothing multiplied)."""
+        t = c_double()
+        self._check(dev.mlh_probe_lds_loads(self._h, slices, byref(t)))
+        return t.value
 
     def profile_decode(self, first_ids, steps):
         """In-sequence mean microseconds per launch (run time plus the launch gap before it) and

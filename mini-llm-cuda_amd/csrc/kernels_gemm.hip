@@ -15,6 +15,7 @@
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <string>
 
@@ -426,7 +427,7 @@ static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, in
     }
     const unsigned grid = (unsigned)std::min(numCUs, ((tilesM * tilesN + 7) / 8) * 8); // one workgroup per compute unit walks its tiles
     const size_t lds = 2 * GB_STAGE;
-    static bool attr = false;
+    static std::atomic<bool> attr{false}; // set-up is idempotent: two threads that race here both do it
     if (!attr) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_big<T, GEMM_EPI_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_big<T, GEMM_EPI_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -763,11 +764,18 @@ static hipError_t launch_gemm_w4(hipStream_t stream, int epi, const void* A, int
     }
     const unsigned grid = (unsigned)std::min(numCUs, ((tilesM * tilesN + 7) / 8) * 8); // one workgroup per compute unit walks its tiles
     const size_t lds = GW_LDS;
-    static bool attr = false;
+    static std::atomic<bool> attr{false}; // set-up is idempotent: two threads that race here both do it
     if (!attr) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_w4<T, GEMM_EPI_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_tn_w4<T, GEMM_EPI_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
+        // the kernel flips stages by XOR on absolute LDS addresses, which is an add/subtract of a stage only while
+        // its dynamic LDS starts at address 0, i.e. while it declares no static __shared__ storage
+        for (const void* f : {reinterpret_cast<const void*>(&k_gemm_tn_w4<T, GEMM_EPI_PLAIN>), reinterpret_cast<const void*>(&k_gemm_tn_w4<T, GEMM_EPI_SWIGLU>)}) {
+            hipFuncAttributes fa;
+            if ((e = hipFuncGetAttributes(&fa, f)) != hipSuccess) return e;
+            if (fa.sharedSizeBytes != 0) return hipErrorInvalidConfiguration;
+        }
         attr = true;
     }
     if (epi == GEMM_EPI_SWIGLU)
@@ -785,7 +793,7 @@ static hipError_t launch_gemm(hipStream_t stream, int epi, const void* A, int ld
     const int total = tilesM * tilesN;
     const unsigned grid = (unsigned)(((total + 7) / 8) * 8);
     const size_t lds = (size_t)(TM + TN) * GLD;
-    static bool attr[2] = {false, false};
+    static std::atomic<bool> attr[2] = {{false}, {false}};
     if (lds > 64 * 1024 && !attr[epi]) {
         hipError_t e = hipFuncSetAttribute(epi ? reinterpret_cast<const void*>(&k_gemm_tn<T, BM, BN, GEMM_EPI_SWIGLU>)
                                                : reinterpret_cast<const void*>(&k_gemm_tn<T, BM, BN, GEMM_EPI_PLAIN>),
@@ -1324,7 +1332,7 @@ static hipError_t launch_gemm_skinny_norm8(hipStream_t stream, int epi, const vo
                                            const float* R, int ldr, int M, int N, int K, float alpha, const float* normGain) {
     const dim3 grid((N + 31) / 32);
     const size_t lds = (size_t)M * (2 * (size_t)K + 16);
-    static bool attr = false; // static + dynamic LDS pass 64 KB
+    static std::atomic<bool> attr{false}; // set-up is idempotent: two threads that race here both do it // static + dynamic LDS pass 64 KB
     if (!attr) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_skinny_norm8<GEMM_EPI_PLAIN>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024);
         if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void*>(&k_gemm_skinny_norm8<GEMM_EPI_SWIGLU>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024);
@@ -1361,7 +1369,7 @@ static hipError_t launch_gemm_skinny16(hipStream_t stream, int epi, const void* 
     const dim3 grid(nblocks, ks);
     unsigned* counters = (unsigned*)ws;
     float* partials = ws ? (float*)((unsigned char*)ws + (size_t)GSK_COUNTERS * 4) : nullptr;
-    static bool attr = false;
+    static std::atomic<bool> attr{false}; // set-up is idempotent: two threads that race here both do it
     if (!attr) {
         const void* fns[4] = {reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_PLAIN, false>), reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_PLAIN, true>),
                               reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_SWIGLU, false>), reinterpret_cast<const void*>(&k_gemm_skinny16<GEMM_EPI_SWIGLU, true>)};

@@ -317,13 +317,28 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
                         const int h = u % a.heads, tl = u / a.heads, j0 = tl << 6;
                         const int page = a.pageTable[seq * a.pagesPerSeq + tl];
                         const size_t base = ((size_t)page * MLH_KV_PAGE) * d + h * HD;
-                        // one staging set of registers: K tile first, reused for the V tile once K sits in LDS
-                        f32x4 kreg[NLD];
+                        // One staging set of registers, at most 16 loads of 16 bytes per lane at a time (a 128-wide head's
+                        // tile in two batches: 32 at once left no registers for the prefetched weight rows and spilled
+                        // ~250 of them): K tile first, reused for the V tile once K sits in LDS.  The loads are
+                        // unconditional (every row of a page is mapped; rows at or behind this step's position are
+                        // replaced on the way into LDS): a load under a per-row condition becomes a branch with a wait.
+                        constexpr int BL = NLD > 16 ? 16 : NLD, NB = NLD / BL;
+                        f32x4 kreg[BL];
+                        auto issue = [&](const float* src, int b) {
 #pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            kreg[it] = (j0 + row < pos) ? *reinterpret_cast<const f32x4*>(L.K + base + (size_t)row * d + c4) : (f32x4)(0.f);
-                        }
+                            for (int it = 0; it < BL; it++)
+                                kreg[it] = *reinterpret_cast<const f32x4*>(src + base + (size_t)((b * BL + it) * RPI + lrow) * d + c4);
+                        };
+                        auto put = [&](int b, const float* newRow) { // rows before this step's from the registers, this step's from LDS, later ones zero
+#pragma unroll
+                            for (int it = 0; it < BL; it++) {
+                                const int row = (b * BL + it) * RPI + lrow;
+                                f32x4 v = (j0 + row < pos) ? kreg[it] : (f32x4)(0.f);
+                                if (j0 + row == pos) v = *reinterpret_cast<const f32x4*>(newRow + c4);
+                                *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
+                            }
+                        };
+                        issue(L.K, 0);
                         const float rc0 = a.rope[(size_t)pos * HD + (EPL == 1 ? (lane & ~1) : 2 * lane)];
                         const float rs0 = a.rope[(size_t)pos * HD + (EPL == 1 ? (lane | 1) : 2 * lane + 1)];
                         // q (and, for the tile that receives this step's row, k and v): per-head RMSNorm
@@ -372,19 +387,11 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
                             }
                         }
                         __builtin_amdgcn_wave_barrier();
+                        put(0, ks);
 #pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            f32x4 v = kreg[it];
-                            if (j0 + row == pos) v = *reinterpret_cast<const f32x4*>(ks + c4);
-                            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
-                        }
+                        for (int b = 1; b < NB; b++) { issue(L.K, b); put(b, ks); }
                         // V tile loads go out now, into the same registers, and fly during the score computation
-#pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            kreg[it] = (j0 + row < pos) ? *reinterpret_cast<const f32x4*>(L.V + base + (size_t)row * d + c4) : (f32x4)(0.f);
-                        }
+                        issue(L.V, 0);
                         __builtin_amdgcn_wave_barrier();
                         float s = 0.f;
                         {
@@ -402,13 +409,9 @@ __global__ void __launch_bounds__(PWG) k_decode_persistent(PersistArgs P) {
                         const float e = valid ? expf(s - m) : 0.f;
                         const float l = pwave_sum(e);
                         __builtin_amdgcn_wave_barrier();
+                        put(0, vn);
 #pragma unroll
-                        for (int it = 0; it < NLD; it++) {
-                            const int row = it * RPI + lrow;
-                            f32x4 v = kreg[it];
-                            if (j0 + row == pos) v = *reinterpret_cast<const f32x4*>(vn + c4);
-                            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
-                        }
+                        for (int b = 1; b < NB; b++) { issue(L.V, b); put(b, vn); }
                         __builtin_amdgcn_wave_barrier();
                         float acc[EPL];
 #pragma unroll

@@ -268,7 +268,10 @@ def _golden(name):
 def _compare_with_horizon(g, pre, ids_gpu, logits_gpu, gap_tol, logits_ok, what):
     """ids: equal to the oracle's, or -- at the first difference -- within gap_tol of the oracle's best by the
     oracle's own four best logits of that step (from there on the histories differ and the comparison ends).
-    logits_gpu {step: row}: compared with the fixture's rows at the steps both hold, up to that point."""
+    logits_gpu {step: row}: compared with the fixture's rows at the steps both hold, up to that point.
+    A tolerated difference in the first nine tenths of the horizon fails the test all the same: what lies behind it
+    would go uncompared, and "whole horizon" would not be what was checked (the fp32 paths have matched every id of
+    every horizon so far; a model that parts early needs a teacher-forced run like configuration 5's)."""
     ids_o, top_idx, top_val = g[pre + "ids"], g[pre + "top_idx"], g[pre + "top_val"]
     assert len(ids_gpu) == len(ids_o)
     upto = len(ids_o)
@@ -286,6 +289,7 @@ def _compare_with_horizon(g, pre, ids_gpu, logits_gpu, gap_tol, logits_ok, what)
             logits_ok(logits_gpu[int(step)], want, f"{what} step {int(step)}")
             checked += 1
     assert checked >= 1
+    assert upto >= len(ids_o) * 9 // 10, f"{what}: ids part from the oracle's (within the tie rule) at step {upto} of {len(ids_o)}"
     return upto, checked
 
 
