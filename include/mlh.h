@@ -180,7 +180,8 @@ int mlh_set_graph(mlh_ctx* ctx, int stepsPerGraph);
  * Mode 3 treats each of the eight XCDs as a tensor-parallel rank (heads and FFN units are split over the
  * XCDs, exchanges inside an XCD go through its L2, only two per layer cross XCDs); it covers models with
  * head size 64 (attention heads; gated-delta-net heads with 64 x 64 states, as many as attention heads;
- * per-layer embeddings of a width that is a multiple of 8) on a 256-unit device
+ * per-layer embeddings of a width that is a multiple of 8) and attention-only models with head size 128 (the
+ * reference's compiled-in shape, network_meta.h:3-20: 6 heads x 128) on a 256-unit device
  * (mlh_xcd_decode_supported), and falls back to mode 1 otherwise.  Mode 3 is the default.
  * Both need every compute unit for themselves and all their waits are bounded: when a launch gives up (units held
  * by other work), the sequence is as it was before the launch (position, token and tags are written at a kernel's

@@ -341,11 +341,22 @@ __device__ __forceinline__ float row_dot_stream(const WT* W, size_t ld, int row,
     return acc;
 }
 
-// Row of the fused first-phase matrix behind local index rho of XCD X: parts q, k, v, gate; nh heads of 64 rows each.
+// The kernel works on 64-wide SLICES of the model dimension: a head of size 64 is one slice, a head of size 128 two
+// (template parameter G = slices per head).  XCD X owns the heads X, X + 8, ... and with them their slices; everything
+// that is linear in the head dimension (the q | k | v | gate rows, the Wo columns, the softmax-partials combine, the
+// gate) runs per slice, only the attention unit itself -- per-head norm, scores, softmax -- sees the G slices of a head
+// together.  Slice number (64-column block of the model dimension) of the j-th slice XCD X owns:
+template <int G>
+__device__ __forceinline__ int slice_of(int X, int j) {
+    return G == 1 ? X + XCDS * j : G * (X + XCDS * (j / G)) + (j % G);
+}
+
+// Row of the fused first-phase matrix behind local index rho of XCD X: parts q, k, v, gate; nh slices of 64 rows each.
+template <int G = 1>
 __device__ __forceinline__ int rowA_of(int offK, int offV, int offG, int X, int nh, int rho) {
     const int per = nh * XHD, p = rho / per, rem = rho - p * per, j = rem >> 6, i = rem & 63;
     const int off = p == 0 ? 0 : p == 1 ? offK : p == 2 ? offV : offG;
-    return off + (X + XCDS * j) * XHD + i;
+    return off + slice_of<G>(X, j) * XHD + i;
 }
 
 // The same for models with gated-delta-net layers and per-layer embeddings: behind the q | k | v | gate rows come
@@ -365,7 +376,7 @@ __device__ __forceinline__ int rowA_hyb(const LayerDev& L, int X, int nh, int np
 
 // Wo columns of the XCD's heads: a pass covers N rows per wave (64/N lanes per 64-column head segment).  Rows
 // and heads beyond the end are clamped to the last valid one (loaded, never used).
-template <typename WT>
+template <typename WT, int G = 1>
 __device__ __forceinline__ void issue_wo(XPf<WT>& pf, const WT* Wo, int ad, int X, int nh, int heads, int lw, int d) {
     constexpr int N = PVec<WT>::N, CPS = XHD / N;
     const unsigned lane = threadIdx.x & 63u;
@@ -375,7 +386,7 @@ __device__ __forceinline__ void issue_wo(XPf<WT>& pf, const WT* Wo, int ad, int 
         const int rb = min((p * XLW + lw) * N, d - N);
 #pragma unroll
         for (int j = 0; j < XNH; j++) {
-            const int h = min(X + XCDS * min(j, max(nh, 1) - 1), heads - 1);
+            const int h = min(slice_of<G>(X, min(j, max(nh, 1) - 1)), G * heads - 1); // slice, clamped to the last one
             pf.r[p * XNH + j] = load16<WT>(pin_uniform(Wo + (size_t)rb * ad + h * XHD), lb, 0u);
         }
     }
@@ -435,12 +446,12 @@ struct XShared {
     } while (0)
 
 // ------------------------------------------------------------------------------------------------ communicator
-template <typename WT, bool HYB>
+template <typename WT, bool HYB, int G>
 __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
     const StepArgs& a = P.a;
     const int d = a.dim, V = a.vocab;
     const int lane = threadIdx.x & 63, wg = blockIdx.x;
-    const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
+    const int nh = a.heads > X ? G * ((a.heads - X + XCDS - 1) / XCDS) : 0; // slices of this XCD
     const int np = 3 + (a.gating ? 1 : 0);
     const int RA = np * nh * XHD;
     unsigned headMask = 0; // XCDs that own at least one head
@@ -550,8 +561,10 @@ __device__ __forceinline__ void xcd_communicator(const XcdArgs& P, const XShared
 }
 
 // ------------------------------------------------------------------------------------------------ workers
-template <typename WT, int NCH, bool HYB>
+template <typename WT, int NCH, bool HYB, int G>
 __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, int tok, int pos, unsigned tagBase, int X, int r) {
+    static_assert(G == 1 || !HYB, "heads of two slices: attention-only models");
+    constexpr int HD = G * XHD; // head size
     constexpr int N = PVec<WT>::N, CPS = XHD / N;
     const StepArgs& a = P.a;
     const int d = a.dim, F = a.ffn, V = a.vocab, fs = P.fs;
@@ -562,7 +575,8 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                                                    // there is one, goes to the last waves, not to the attention waves
     const int gwl = wave * (int)gridDim.x + wg; // worker wave within the grid (LM head)
     const int TWL = XWORK * (int)gridDim.x;
-    const int nh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0;
+    const int nhh = a.heads > X ? (a.heads - X + XCDS - 1) / XCDS : 0; // heads of this XCD
+    const int nh = G * nhh;                                            // and their slices
     const int np = 3 + (a.gating ? 1 : 0);
     const int RA = np * nh * XHD;
     const int pleX = HYB ? a.ple / XCDS : 0; // PLE columns of this XCD
@@ -575,11 +589,11 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     };
     auto rowA = [&](const LayerDev& Lx, int rho) {
         if constexpr (HYB) return rowA_hyb(Lx, X, nh, uni(Lx.kind) != MLH_KIND_ATTENTION ? 3 : np, pleX, rho);
-        else return rowA_of(uni(Lx.offK), uni(Lx.offV), uni(Lx.offG), X, nh, rho);
+        else return rowA_of<G>(uni(Lx.offK), uni(Lx.offV), uni(Lx.offG), X, nh, rho);
     };
     u64* qkvL = P.qkvL + (size_t)X * P.qkvStride;
     u64* partL = P.partL + (size_t)X * P.partStride;
-    float* tK = S.tiles + (wave < XAW ? wave : 0) * (2 * XTILE);
+    float* tK = S.tiles + (wave < XAW ? wave : 0) * (G * 2 * XTILE); // slice g of the head: K tile at + g 2 XTILE, V tile behind it
     float* tV = tK + XTILE;
     const int aslot = wave * XPER + r; // attention unit slot of this wave (waves below XAW only)
     const WT* E = (const WT*)a.E;
@@ -597,23 +611,34 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
         issue_gain<WT, NCH>(gn, uni_ptr(Lx.g1));
     };
     // first K/V tile of this wave in layer Lx when the sequence holds npos rows, and the q/k gains of its head
-    float gqv = 1.f, gkv = 1.f;
+    float gqv[G], gkv[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) { gqv[g] = 1.f; gkv[g] = 1.f; }
     // (the tile index of a wave's first unit never changes, so its page is looked up once)
-    const int pageFirst = (wave < XAW && nh > 0 && aslot / nh < 2 * a.pagesPerSeq) ? uni(a.pageTable[P.seq * a.pagesPerSeq + ((aslot / nh) >> 1)]) : 0;
+    const int pageFirst = (wave < XAW && nhh > 0 && aslot / nhh < 2 * a.pagesPerSeq) ? uni(a.pageTable[P.seq * a.pagesPerSeq + ((aslot / nhh) >> 1)]) : 0;
+    // gains of head h's slices for this lane, and the K/V tiles of its slices from the page rows at `base`
+    auto loadGains = [&](const LayerDev& Lx, int h) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            gqv[g] = uni_ptr(Lx.gq)[h * HD + g * XHD + lane];
+            gkv[g] = uni_ptr(Lx.gk)[h * HD + g * XHD + lane];
+        }
+    };
+    auto issueTiles = [&](const LayerDev& Lx, size_t base, int lim) {
+#pragma unroll
+        for (int g = 0; g < G; g++)
+            issue_kv_tile(uni_ptr((const float*)Lx.K) + base + g * XHD, uni_ptr((const float*)Lx.V) + base + g * XHD, d, lim, tK + g * 2 * XTILE, tV + g * 2 * XTILE);
+    };
     auto issueKV = [&](const LayerDev& Lx, int npos) {
         const int nt = (npos + XTK) / XTK;
-        if (aslot < nh * nt) {
-            const int j = aslot % nh, tl = aslot / nh;
-            if (a.qkNorm) {
-                gqv = uni_ptr(Lx.gq)[(X + XCDS * j) * XHD + lane];
-                gkv = uni_ptr(Lx.gk)[(X + XCDS * j) * XHD + lane];
-            }
-            const size_t base = ((size_t)pageFirst * MLH_KV_PAGE + (tl & 1) * XTK) * d + (X + XCDS * j) * XHD;
-            issue_kv_tile(uni_ptr((const float*)Lx.K) + base, uni_ptr((const float*)Lx.V) + base, d, npos - tl * XTK, tK, tV);
+        if (aslot < nhh * nt) {
+            const int j = aslot % nhh, tl = aslot / nhh, h = X + XCDS * j;
+            if (a.qkNorm) loadGains(Lx, h);
+            issueTiles(Lx, ((size_t)pageFirst * MLH_KV_PAGE + (tl & 1) * XTK) * d + h * HD, npos - tl * XTK);
         }
     };
     if (wave < XAW) { // the tiles must never hold anything but finite numbers (rows beyond the sequence get weight zero)
-        for (int i = lane * 4; i < 2 * XTILE; i += 256) *reinterpret_cast<f32x4*>(tK + i) = (f32x4)(0.f);
+        for (int i = lane * 4; i < G * 2 * XTILE; i += 256) *reinterpret_cast<f32x4*>(tK + i) = (f32x4)(0.f);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
     // hybrid models: the PLE up-projection columns of this XCD for the first two passes of the output projection
@@ -651,21 +676,26 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     {
         const LayerDev& L0 = S.Ls[P.NL - 1];
         issueA(L0);
-        issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
+        issue_wo<WT, G>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
         issuePlw(L0);
         if (wave < XAW && (!HYB || uni(L0.kind) == MLH_KIND_ATTENTION)) issueKV(L0, pos);
     }
 
-    float* qh = S.tiles + XAW * 2 * XTILE + (wave < XAW ? wave : 0) * 64; // this wave's query after norm and RoPE
+    float* qh = S.tiles + XAW * G * 2 * XTILE + (wave < XAW ? wave : 0) * HD; // this wave's query after norm and RoPE
     bool ok = true; // attention waves poll the softmax partials (bounded)
 
     for (int step = 0; step < P.steps; step++) {
         const int T = pos + 1, ntiles = (T + XTK - 1) / XTK, newTile = pos / XTK;
-        float rc = 1.f, rsn = 0.f; // RoPE of this step's position: lanes (2i, 2i+1) hold the pair i (inference.cu:113-134)
+        float rc[G], rsn[G]; // RoPE of this step's position: lanes (2i, 2i+1) of slice g hold the pair 32 g + i (inference.cu:113-134)
+#pragma unroll
+        for (int g = 0; g < G; g++) { rc[g] = 1.f; rsn[g] = 0.f; }
         int pageNew = 0; // page that receives this step's K/V row
         if (wave < XAW) {
-            rc = a.rope[(size_t)pos * XHD + (lane & ~1)];
-            rsn = a.rope[(size_t)pos * XHD + (lane | 1)];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                rc[g] = a.rope[(size_t)pos * HD + g * XHD + (lane & ~1)];
+                rsn[g] = a.rope[(size_t)pos * HD + g * XHD + (lane | 1)];
+            }
             pageNew = uni(a.pageTable[P.seq * a.pagesPerSeq + (pos >> 6)]);
         }
         issuePlv(S.Ls[P.NL - 1], tok);
@@ -750,28 +780,44 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                 }
             }
             if (wave < XAW && !gdnL) {
-                const int U = nh * ntiles;
+                const int U = nhh * ntiles;
                 const float* qsAll = S.qkvs; // rows as the first phase produced them
                 const float* ksAll = qsAll + nh * XHD;
                 const float* vsAll = ksAll + nh * XHD;
                 const float* gsAll = vsAll + nh * XHD;
-                // per-head RMSNorm (inference.cu:52-81, 97-111) and RoPE of a 64-vector held one element per lane
-                auto norm_rope = [&](float v, float gain) {
-                    if (a.qkNorm) v = gain * (v / sqrtf(pwave_sum(v * v) / (float)XHD + 1e-8f));
-                    const float o = dpp_move<0xB1, 0xf>(v, 0.f); // the other element of the pair
-                    return (lane & 1) ? rsn * o + rc * v : rc * v - rsn * o;
+                // per-head RMSNorm (inference.cu:52-81, 97-111) and RoPE of a head's vector held one element per lane and slice
+                auto norm_rope = [&](float (&v)[G], const float (&gain)[G]) {
+                    if (a.qkNorm) {
+                        float ss = 0.f;
+#pragma unroll
+                        for (int g = 0; g < G; g++) ss = fmaf(v[g], v[g], ss);
+                        const float rr = sqrtf(pwave_sum(ss) / (float)HD + 1e-8f);
+#pragma unroll
+                        for (int g = 0; g < G; g++) v[g] = gain[g] * (v[g] / rr);
+                    }
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+                        const float o = dpp_move<0xB1, 0xf>(v[g], 0.f); // the other element of the pair
+                        v[g] = (lane & 1) ? rsn[g] * o + rc[g] * v[g] : rc[g] * v[g] - rsn[g] * o;
+                    }
                 };
                 const bool dbg = P.timing && t == 0 && step == P.steps - 1 && lane == 0 && wave == 0;
                 if (dbg) P.timing[16 * (P.NL + 1) + 4 * wg + 1] = aslot < U ? wall_clock64() : 0;
                 for (int u = aslot; u < U; u += XAW * XPER) {
-                    const int j = u % nh, tl = u / nh, j0 = tl * XTK, h = X + XCDS * j;
+                    const int j = u % nhh, tl = u / nhh, j0 = tl * XTK, h = X + XCDS * j; // j: head among the XCD's, its slices G j + g
                     if (u != aslot) { // tiles beyond the first one were not fetched ahead
                         const int page = uni(a.pageTable[P.seq * a.pagesPerSeq + (tl >> 1)]);
-                        const size_t base = ((size_t)page * MLH_KV_PAGE + (tl & 1) * XTK) * d + h * XHD;
-                        issue_kv_tile(uni_ptr((const float*)L.K) + base, uni_ptr((const float*)L.V) + base, d, pos - j0, tK, tV);
-                        if (a.qkNorm) { gqv = uni_ptr(L.gq)[h * XHD + lane]; gkv = uni_ptr(L.gk)[h * XHD + lane]; }
+                        issueTiles(L, ((size_t)page * MLH_KV_PAGE + (tl & 1) * XTK) * d + h * HD, pos - j0);
+                        if (a.qkNorm) loadGains(L, h);
                     }
-                    qh[lane] = norm_rope(qsAll[j * XHD + lane], gqv);
+                    {
+                        float qv[G];
+#pragma unroll
+                        for (int g = 0; g < G; g++) qv[g] = qsAll[(G * j + g) * XHD + lane];
+                        norm_rope(qv, gqv);
+#pragma unroll
+                        for (int g = 0; g < G; g++) qh[g * XHD + lane] = qv[g];
+                    }
                     // The tile has landed in LDS.  A tile fetched a layer ahead is older than the dozens of weight loads
                     // issued since (loads and stores retire in issue order): the few stores of the first phase may stay
                     // in flight.
@@ -781,51 +827,64 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     const int nv = T - j0 < XTK ? T - j0 : XTK;     // keys of this tile, the new one included
                     if (tl == newTile) { // this step's row comes from the first phase, not from the cache; it is appended here
                         const int rn = pos - j0;
-                        const float kn = norm_rope(ksAll[j * XHD + lane], gkv), vn = vsAll[j * XHD + lane];
-                        tK[rn * 64 + ((((lane >> 2) ^ (rn & 15)) << 2) | (lane & 3))] = kn;
-                        tV[rn * 64 + lane] = vn;
-                        // write-through: read from the next step on, by whichever workgroup of this XCD takes the tile
-                        const size_t o = ((size_t)pageNew * MLH_KV_PAGE + (pos & 63)) * d + h * XHD + lane;
-                        ast(uni_ptr(L.K) + o, kn);
-                        ast(uni_ptr(L.V) + o, vn);
+                        float kn[G];
+#pragma unroll
+                        for (int g = 0; g < G; g++) kn[g] = ksAll[(G * j + g) * XHD + lane];
+                        norm_rope(kn, gkv);
+#pragma unroll
+                        for (int g = 0; g < G; g++) {
+                            const float vn = vsAll[(G * j + g) * XHD + lane];
+                            tK[g * 2 * XTILE + rn * 64 + ((((lane >> 2) ^ (rn & 15)) << 2) | (lane & 3))] = kn[g];
+                            tV[g * 2 * XTILE + rn * 64 + lane] = vn;
+                            // write-through: read from the next step on, by whichever workgroup of this XCD takes the tile
+                            const size_t o = ((size_t)pageNew * MLH_KV_PAGE + (pos & 63)) * d + h * HD + g * XHD + lane;
+                            ast(uni_ptr(L.K) + o, kn[g]);
+                            ast(uni_ptr(L.V) + o, vn);
+                        }
                     }
                     __builtin_amdgcn_wave_barrier();
-                    // scores: lanes l and l + 32 share key l % 32, each takes half of the 64 dimensions
+                    // scores: lanes l and l + 32 share key l % 32, each takes half of the 64 dimensions of every slice
                     const int key = lane & 31, dh = lane >> 5;
                     float s = 0.f;
-                    {
-                        const float* kr = tK + key * 64;
+#pragma unroll
+                    for (int g = 0; g < G; g++) {
+                        const float* kr = tK + g * 2 * XTILE + key * 64;
 #pragma unroll
                         for (int p = 0; p < 8; p++) {
                             const int pp = p + 8 * dh;
                             const f32x4 kk = *reinterpret_cast<const f32x4*>(kr + ((pp ^ (key & 15)) << 2));
-                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qh + pp * 4);
+                            const f32x4 qq = *reinterpret_cast<const f32x4*>(qh + g * XHD + pp * 4);
                             s = fmaf(kk.x, qq.x, s); s = fmaf(kk.y, qq.y, s); s = fmaf(kk.z, qq.z, s); s = fmaf(kk.w, qq.w, s);
                         }
                     }
                     s += __shfl_xor(s, 32, MLH_WAVE);
                     const bool valid = key < nv;
-                    s = valid ? s / sqrtf((float)XHD) : -1.0e30f; // inference.cu:154
+                    s = valid ? s / sqrtf((float)HD) : -1.0e30f; // inference.cu:154
                     const float m = pwave_max(s);
                     const float e = (valid && dh == 0) ? expf(s - m) : 0.f; // lanes 0..31 carry the weights
                     const float l = pwave_sum(e);
                     // all XTK rows: rows from nv on hold older K/V rows or the zeros of the start of the kernel, and
                     // their weights are zero.  Sixteen rows are fetched before they are used, so that the LDS latency
                     // is paid twice, not once per row.
-                    float acc = 0.f;
-                    const float* vcol = tV + lane;
 #pragma unroll
-                    for (int jj0 = 0; jj0 < XTK; jj0 += 16) {
-                        float vr[16];
+                    for (int g = 0; g < G; g++) {
+                        float acc = 0.f;
+                        const float* vcol = tV + g * 2 * XTILE + lane;
 #pragma unroll
-                        for (int i = 0; i < 16; i++) vr[i] = vcol[(jj0 + i) * 64];
+                        for (int jj0 = 0; jj0 < XTK; jj0 += 16) {
+                            float vr[16];
 #pragma unroll
-                        for (int i = 0; i < 16; i++)
-                            acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj0 + i)), vr[i], acc);
+                            for (int i = 0; i < 16; i++) vr[i] = vcol[(jj0 + i) * 64];
+#pragma unroll
+                            for (int i = 0; i < 16; i++)
+                                acc = fmaf(__int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), jj0 + i)), vr[i], acc);
+                        }
+                        // a slice's tiles one after the other, as the combine reads them; every slice of the head carries the
+                        // head's maximum and sum, so the combine runs slice by slice
+                        u64* out = partL + ((size_t)(G * j + g) * ntiles + tl) * (XHD + 2);
+                        lst(out + lane, acc, lt);
+                        if (lane == 0) { lst(out + XHD, m, lt); lst(out + XHD + 1, l, lt); }
                     }
-                    u64* out = partL + ((size_t)j * ntiles + tl) * (XHD + 2); // a head's tiles one after the other, as the combine reads them
-                    lst(out + lane, acc, lt);
-                    if (lane == 0) { lst(out + XHD, m, lt); lst(out + XHD + 1, l, lt); }
                     __builtin_amdgcn_wave_barrier();
                 }
                 if (P.timing && t == 0 && step == P.steps - 1 && lane == 0)
@@ -909,7 +968,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
                     for (int j = 0; j < XNH; j++)
                         if (j < nh) {
                             const typename PVec<WT>::Raw w = p == 0 ? s2.r[j] : p == 1 ? s2.r[XNH + j]
-                                : PVec<WT>::load(uni_ptr((const WT*)L.Wo) + (size_t)row * ad + (X + XCDS * j) * XHD + c * N);
+                                : PVec<WT>::load(uni_ptr((const WT*)L.Wo) + (size_t)row * ad + slice_of<G>(X, j) * XHD + c * N);
                             acc = chunk_dot_lds<WT>(w, S.as + j * XHD + c * N, acc);
                         }
                     if constexpr (HYB) { // + pleUp . e over the XCD's PLE columns (one column per lane of the row group)
@@ -998,7 +1057,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
             }
             W_STAMP(9);
             if (!lastLayer) {
-                issue_wo<WT>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, a.heads, lw, d);
+                issue_wo<WT, G>(s2, uni_ptr((const WT*)Ln.Wo), uni(Ln.ad), X, nh, a.heads, lw, d);
                 issuePlw(Ln);
             } else {
                 // two more LM-head rows; the second register set has room for them when a row has at most 4 chunks
@@ -1032,7 +1091,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
         if (step + 1 < P.steps) { // first layer of the next step
             const LayerDev& L0 = S.Ls[P.NL - 1];
             issueA(L0);
-            issue_wo<WT>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
+            issue_wo<WT, G>(s2, uni_ptr((const WT*)L0.Wo), uni(L0.ad), X, nh, a.heads, lw, d);
             issuePlw(L0);
         }
         X_BARRIER(); // best logits in LDS
@@ -1048,7 +1107,7 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
     (void)tok;
 }
 
-template <typename WT, int NCH, bool HYB>
+template <typename WT, int NCH, bool HYB, int G>
 __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     extern __shared__ float lds[];
     const StepArgs& a = P.a;
@@ -1064,7 +1123,7 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     S.besti = reinterpret_cast<int*>(S.bestv + 16);
     S.ctl = S.besti + 16;               // [0] a wait expired, [1] next token
     S.tiles = reinterpret_cast<float*>(S.ctl + 16); // [XAW][K tile | V tile]
-    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * 2 * XTILE + XAW * 64); // (after the tiles: one query vector per attention wave)
+    S.Ls = reinterpret_cast<LayerDev*>(S.tiles + XAW * G * 2 * XTILE + XAW * G * 64); // (after the tiles: one query vector per attention wave)
     S.es = reinterpret_cast<float*>(S.Ls + P.NL);
     S.gst = S.es + 16;                  // hybrid models only: [NL][4][64]
     for (int i = threadIdx.x; i < P.NL * (int)(sizeof(LayerDev) / 4); i += XWG)
@@ -1090,8 +1149,8 @@ __global__ void __launch_bounds__(XWG) k_decode_xcd(XcdArgs P) {
     const int X = uni(S.ctl[2]), r = uni(S.ctl[3]);
     const int tok = uni(a.tok[0]), pos = uni(a.pos[P.seq]);
     const unsigned tagBase = *P.tagCounter; // tags do not repeat from launch to launch (the host clears everything before the count wraps)
-    if (wave == XWORK) xcd_communicator<WT, HYB>(P, S, tok, pos, tagBase, X, r);
-    else xcd_worker<WT, NCH, HYB>(P, S, tok, pos, tagBase, X, r);
+    if (wave == XWORK) xcd_communicator<WT, HYB, G>(P, S, tok, pos, tagBase, X, r);
+    else xcd_worker<WT, NCH, HYB, G>(P, S, tok, pos, tagBase, X, r);
 }
 
 // before every launch: abort flag and per-XCD arrival counters
@@ -1120,7 +1179,8 @@ static bool xcd_hybrid(const mlh_ctx* c) {
 static size_t xcd_lds_bytes(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
     const int fs = hp.ffnDim / XCDS;
-    return ((size_t)2 * hp.dim + 5 * XNH * XHD + XQX + ((fs + 3) & ~3) + 512 + 48 + XAW * 2 * XTILE + XAW * 64 + 16 +
+    const int G = hp.headDim / XHD; // slices per head
+    return ((size_t)2 * hp.dim + 5 * XNH * XHD + XQX + ((fs + 3) & ~3) + 512 + 48 + XAW * G * 2 * XTILE + XAW * G * 64 + 16 +
             (xcd_hybrid(c) ? (size_t)hp.transformers * 4 * XHD : 0)) * 4 + (size_t)hp.transformers * sizeof(LayerDev);
 }
 
@@ -1132,7 +1192,8 @@ size_t mlh_xcd_words(const mlh_ctx* c) {
 }
 
 // True when the XCD-rank kernel supports this context's shape: head size 64 (attention heads, and GDN heads with
-// 64 x 64 states, as many as attention heads), PLE columns that split evenly over the XCDs, a 256-unit chip, rows
+// 64 x 64 states, as many as attention heads) or, for attention-only models without per-layer embeddings, 128 (the
+// shape the reference ships: network_meta.h:3-20); PLE columns that split evenly over the XCDs, a 256-unit chip, rows
 // that fit the register sets.
 bool mlh_xcd_supported(const mlh_ctx* c) {
     const mlh_hparams& hp = c->hp;
@@ -1143,32 +1204,34 @@ bool mlh_xcd_supported(const mlh_ctx* c) {
     if (gdn && (hp.gdnDk != XHD || hp.gdnDv != XHD || hp.gdnHeads != hp.attnHeads || hp.attnHeads < XCDS || hp.attnHeads > 2 * XCDS)) return false; // (four state rows per workgroup and layer)
     if (hp.pleDim % XCDS || hp.pleDim / XCDS > XHD / N || 2 * XNH + hp.pleDim / XCDS > XQX) return false;
     if (hp.pleDim > 0 && hp.attnHeads < XCDS) return false;
-    if (hp.headDim != XHD) return false;
-    if (hp.dim != hp.attnHeads * XHD || hp.dim > 4 * 64 * N || hp.dim % (64 * N) || hp.dim % XPER) return false;
-    if (hp.attnHeads > XCDS * XNH) return false;
+    if (hp.headDim != XHD && !(hp.headDim == 2 * XHD && !gdn && hp.pleDim == 0)) return false;
+    const int G = hp.headDim / XHD;
+    if (hp.dim != hp.attnHeads * hp.headDim || hp.dim > 4 * 64 * N || hp.dim % (64 * N) || hp.dim % XPER) return false;
+    if (G * ((hp.attnHeads + XCDS - 1) / XCDS) > XNH) return false; // slices per XCD
     if (hp.ffnDim % (XCDS * N)) return false;
     if (hp.dim / 4 > 512 || hp.dim % N) return false;
     return xcd_lds_bytes(c) <= 160 * 1024;
 }
 
-template <typename WT, int NCH, bool HYB>
+template <typename WT, int NCH, bool HYB, int G>
 static int launch_xcd_as(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
     if (!c->xcdPrepared) { // once per context (mlh_finalize does it; a context has one model, hence one instantiation)
-        MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH, HYB>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+        MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_decode_xcd<WT, NCH, HYB, G>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
         int perCu = 0;
-        MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH, HYB>, XWG, ldsBytes));
+        MLH_CHECK(c, hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, k_decode_xcd<WT, NCH, HYB, G>, XWG, ldsBytes));
         if (perCu < 1) { c->err = "XCD-rank decode kernel does not fit on a compute unit"; return -1; }
         c->xcdPrepared = true;
     }
     if (P.steps <= 0) return 0; // preparation only
     // one workgroup per compute unit, all resident at once (the occupancy query says each unit can hold one); waits are bounded
-    hipLaunchKernelGGL((k_decode_xcd<WT, NCH, HYB>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
+    hipLaunchKernelGGL((k_decode_xcd<WT, NCH, HYB, G>), dim3(XCDS * XPER), dim3(XWG), ldsBytes, c->stream, P);
     MLH_CHECK(c, hipGetLastError());
     return 0;
 }
 template <typename WT, int NCH>
 static int launch_xcd(mlh_ctx* c, XcdArgs& P, size_t ldsBytes) {
-    return xcd_hybrid(c) ? launch_xcd_as<WT, NCH, true>(c, P, ldsBytes) : launch_xcd_as<WT, NCH, false>(c, P, ldsBytes);
+    if (c->hp.headDim == 2 * XHD) return launch_xcd_as<WT, NCH, false, 2>(c, P, ldsBytes); // (attention-only: mlh_xcd_supported)
+    return xcd_hybrid(c) ? launch_xcd_as<WT, NCH, true, 1>(c, P, ldsBytes) : launch_xcd_as<WT, NCH, false, 1>(c, P, ldsBytes);
 }
 
 // Puts the exchange words and the tag counter back to zero (after a launch that gave up a wait, and before the

@@ -103,14 +103,18 @@ def test_config1_golden_horizon(pkg, orc, persistent):
 
 
 @pytest.mark.parametrize("case", ["heads12", "bf16_dim512", "two_combine_batches", "shuffled_pages", "hybrid12",
-                                  "hybrid8_flags", "hybrid8_bf16", "attention8_ple", "hybrid12_no_ple"])
+                                  "hybrid8_flags", "hybrid8_bf16", "attention8_ple", "hybrid12_no_ple",
+                                  "hd128_heads2", "hd128_heads6_flags", "hd128_heads4_bf16_flags", "hd128_heads8_long", "hd128_heads12_bf16_long"])
 def test_xcd_rank_kernel_shapes(pkg, orc, case):
     """The XCD-rank kernel on the shapes its work split distinguishes: XCDs with two heads and with one
     (12 heads over 8 XCDs), bf16 weights (8 values per 16-byte chunk), more softmax partials per XCD than
     one combine round fetches, and a shuffled page table; several launches in a row (the tags run on).
     Hybrid models: gated-delta-net layers whose state rows stay in LDS from launch to launch end and return to
     memory in between (3 GDN : 1 attention and 1 : 1, with and without the flags), PLE columns split over the XCDs
-    (with GDN layers, with attention layers only), GDN layers without PLE, bf16 weights."""
+    (with GDN layers, with attention layers only), GDN layers without PLE, bf16 weights.
+    Heads of size 128 (two 64-wide slices per head; the shape the reference ships is 6 heads x 128, network_meta.h:3-20):
+    fewer heads than XCDs, both flags (per-head norm over 128 dimensions, RoPE pairs 0..63, gate per slice), bf16, and
+    more heads than XCDs with a context of several tiles per head."""
     bf16 = case in ("bf16_dim512", "hybrid8_bf16")
     kw = dict(transformers=2, vocabSize=1024, headDim=64)
     if case.startswith("hybrid") or case == "attention8_ple":
@@ -124,6 +128,12 @@ def test_xcd_rank_kernel_shapes(pkg, orc, case):
             hkw.update(weightDtype=pkg.DTYPE_BF16)
         hp = pkg.config(3, **hkw)
         pkg.set_layer_pattern(hp, {"hybrid12": 3, "hybrid8_flags": 1, "hybrid8_bf16": 1, "attention8_ple": 0, "hybrid12_no_ple": 3}[case])
+    elif case.startswith("hd128"):
+        heads = int(case.split("heads")[1].split("_")[0])
+        fl = 1 if "flags" in case else 0
+        bf16 = "bf16" in case
+        hp = pkg.config(1, dim=128 * heads, attnHeads=heads, headDim=128, ffnDim=512, maxL=900 if "long" in case else 200, transformers=2,
+                        vocabSize=1024, qkRmsNorm=fl, queryGating=fl, weightDtype=pkg.DTYPE_BF16 if bf16 else pkg.DTYPE_F32)
     elif bf16:
         hp = pkg.config(1, dim=512, attnHeads=8, ffnDim=1024, maxL=200, weightDtype=pkg.DTYPE_BF16, **kw)
     elif case == "two_combine_batches":
@@ -135,7 +145,7 @@ def test_xcd_rank_kernel_shapes(pkg, orc, case):
     assert dev.xcd_decode_supported()
     if case == "shuffled_pages":
         dev.set_page_table(np.random.default_rng(3).permutation((hp.maxL + 63) // 64 * hp.maxSeqs).astype(np.int32))
-    plen = 840 if case == "two_combine_batches" else 60  # 14 tiles x 2 heads = 28 partials on the two-head XCDs
+    plen = 840 if case == "two_combine_batches" or case.endswith("_long") else 60  # 14 tiles x 2 heads = 28 partials on the two-head XCDs
     prompt = pkg.random_tokens(23, 0, hp.vocabSize, plen)
     if bf16:
         dev.set_prefill_mode(1)  # the MFMA prefill rounds activations to half; here only the decode kernel is under test
