@@ -1085,7 +1085,17 @@ __device__ __forceinline__ void xcd_worker(const XcdArgs& P, const XShared& S, i
 #pragma unroll
             for (int k = 0; k < 2; k++)
                 if (gwl + TWL * (XS1 + k) < V) take(gwl + TWL * (XS1 + k), row_dot_reg<WT, NCH>(reinterpret_cast<const typename PVec<WT>::Raw (&)[2 * NCH]>(s2.r), k, xn));
-            for (int row = gwl + (XS1 + 2) * TWL; row < V; row += TWL) take(row, row_dot_stream<WT, NCH>(E, d, row, xn));
+            // a large vocabulary leaves rows beyond the prefetched ones: XS1 at a time through the first register set (its
+            // rows are used up), so that a wave pays one memory round trip per XS1 rows instead of one per row
+            for (int row0 = gwl + (XS1 + 2) * TWL; row0 < V; row0 += XS1 * TWL) {
+                int rows[XS1];
+#pragma unroll
+                for (int k = 0; k < XS1; k++) rows[k] = min(row0 + TWL * k, V - 1);
+                issue_rows<WT, XS1, NCH>(s1.r, E, d, rows);
+#pragma unroll
+                for (int k = 0; k < XS1; k++)
+                    if (row0 + TWL * k < V) take(row0 + TWL * k, row_dot_reg<WT, NCH>(s1.r, k, xn));
+            }
             if (lane == 0) { S.bestv[wave] = best; S.besti[wave] = bidx; }
         }
         if (step + 1 < P.steps) { // first layer of the next step

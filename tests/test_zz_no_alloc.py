@@ -9,14 +9,16 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
+F16 = 2  # operand type code of IEEE-half operands (the mirrors a bf16 model's MFMA path multiplies)
+
 
 def _run(pkg, torch, dtype, M, N, K, seed, with_r):
     rng = np.random.default_rng(seed)
     a = rng.normal(size=(M, K)).astype(np.float32)
     b = rng.normal(size=(N, K)).astype(np.float32)
     r = rng.normal(size=(M, N)).astype(np.float32) if with_r else None
-    want, _ = pkg.selftest_gemm(a, b, r, bf16=(dtype == pkg.DTYPE_BF16))
-    tt = torch.float32 if dtype == pkg.DTYPE_F32 else torch.bfloat16
+    want, _ = pkg.selftest_gemm(a, b, r, bf16=(dtype == pkg.DTYPE_BF16), f16=(dtype == F16))
+    tt = {pkg.DTYPE_F32: torch.float32, pkg.DTYPE_BF16: torch.bfloat16, F16: torch.float16}[dtype]
     da = torch.from_numpy(a).cuda().to(tt).contiguous()
     db = torch.from_numpy(b).cuda().to(tt).contiguous()
     dr = torch.from_numpy(r).cuda() if with_r else None
@@ -44,6 +46,8 @@ def test_no_alloc_gemm_matches_allocating_entry_point(pkg):
     _run(pkg, torch, pkg.DTYPE_F32, 64, 512, 2048, 3, with_r=True)   # 64 rows: the 16-row fp32 kernel, also split
     _run(pkg, torch, pkg.DTYPE_BF16, 33, 320, 4096, 4, with_r=False)  # half-width operands, ragged M and N
     _run(pkg, torch, pkg.DTYPE_F32, 5, 8192, 768, 5, with_r=False)    # many rows: no split, the array is not touched
+    _run(pkg, torch, F16, 8, 256, 5632, 6, with_r=True)               # IEEE-half operands, few rows and long K: split
+    _run(pkg, torch, pkg.DTYPE_BF16, 64, 192, 2048, 7, with_r=True)   # 64 rows of bf16: the two-block skinny kernel, split
     # limits and argument checks
     x = torch.zeros(16, dtype=torch.float32, device="cuda")
     p = x.data_ptr()
