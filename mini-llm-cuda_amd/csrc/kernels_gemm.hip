@@ -1452,6 +1452,10 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
         GEMM_BY_TYPE((launch_gemm_skinny<float, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<bf16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)),
                      (launch_gemm_skinny<f16_t, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, ws, alpha)));
+    if (M > 128 && N <= 128 && dtype != MLH_DTYPE_F32 && epi == GEMM_EPI_PLAIN) { // a narrow strip of columns: 64-row tiles put every compute unit to work
+        if (dtype == MLH_GEMM_F16) return launch_gemm<f16_t, 1, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha);
+        return launch_gemm<bf16_t, 1, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha);
+    }
     if (M > 128)
         GEMM_BY_TYPE((launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
                      (launch_gemm_w4<bf16_t>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
