@@ -64,6 +64,16 @@ def physical_cores():
         return os.cpu_count() or 1
 
 
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def decode_bytes_per_token(hp, T, wbytes=4):
     """Algorithmic bytes one batch-1 decode step must move with T positions in the cache after the
     step: every weight matrix once, K and V rows of the attention layers read once and one row
@@ -104,6 +114,12 @@ def cpu_baseline_one(what, model, hp, prompt, gpu_ids, n_full, n_cached, runs=3)
     positions, inference_orchestrator.cu:64-65) and of n_cached tokens with a KV cache; medians are reported.  The
     ids are compared with the GPU's for the same prompt (fp32 on both sides: equal unless two logits tie)."""
     cm, cpu_model, torch = _cpu_model(model, hp)
+    # before any timing is reported: the restatement's logits for the prompt against the float64 oracle's (the oracle
+    # is the checker here, nothing of it is timed)
+    orc = entry.load_oracle()
+    want = orc.forward_full(orc.Weights.from_model(model), prompt, "f64")["logits"][0]
+    got = cm.forward(prompt).numpy().astype(np.float64)
+    logit_err = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
     cm.generate_full(prompt, 2)  # warm-up
     full, cached, ids_full, ids_cached = [], [], None, None
     for _ in range(runs):
@@ -121,7 +137,8 @@ def cpu_baseline_one(what, model, hp, prompt, gpu_ids, n_full, n_cached, runs=3)
                    f"PyTorch {torch.__version__} CPU fp32"),
         "with_kv_cache_tok_s": stats(cached)["median"], "with_kv_cache_stats": stats(cached),
         "with_kv_cache_sample": f"{n_cached} greedy tokens, median of {runs} runs",
-        "host_cpu_count": os.cpu_count(), "host_physical_cores": physical_cores(),
+        "host_cpu_count": os.cpu_count(), "host_physical_cores": physical_cores(), "host_cpu_model": cpu_model_name(),
+        "prompt_logits_vs_float64_oracle": {"max_abs_diff_over_max_logit": logit_err, "within_1e-5": logit_err <= 1e-5},
         "first_ids": ids_full[:8], "first_ids_cached": ids_cached[:8],
         "ids_equal_gpu": (ids_full[:len(gpu)] == gpu[:len(ids_full)] and ids_cached[:len(gpu)] == gpu[:len(ids_cached)]),
         "ids_compared": [min(len(gpu), len(ids_full)), min(len(gpu), len(ids_cached))],
