@@ -217,14 +217,20 @@ def test_single_launch_gives_up_and_falls_back(pkg, orc, mode):
     dev.close()
 
 
-@pytest.mark.parametrize("mode,kind", [(3, "hybrid12"), (1, "hybrid"), (1, "hd128")], ids=["xcd", "barrier", "barrier-hd128"])
+@pytest.mark.parametrize("mode,kind", [(3, "hybrid12"), (3, "heads6x128"), (1, "hybrid"), (1, "hd128")],
+                         ids=["xcd", "xcd-heads-of-128", "barrier", "barrier-hd128"])
 def test_single_launch_gives_up_in_mid_run(pkg, orc, mode, kind):
     """A single-launch decode that gives up AFTER some of its steps have run (forced from the host: workgroup 0
     raises the flag itself when it reaches step 3 of 7, every workgroup then leaves at its next wait): the steps
     that did run have appended K/V rows and -- in the barrier kernel -- stored updated gated-delta-net states.  The
     redo as the kernel sequence must start from the states before the launch (a second application of the delta
     rule would show in every later logit), so the whole call and what follows agree with the oracle."""
-    hp = _hybrid12(pkg) if kind == "hybrid12" else small_cfg(pkg, kind)
+    if kind == "hybrid12":
+        hp = _hybrid12(pkg)
+    elif kind == "heads6x128":  # the reference's head layout (network_meta.h:3-20) at reduced depth and vocabulary
+        hp = pkg.config(1, dim=768, attnHeads=6, headDim=128, ffnDim=512, maxL=200, transformers=2, vocabSize=1024, qkRmsNorm=1, queryGating=1)
+    else:
+        hp = small_cfg(pkg, kind)
     model, dev, w = make(pkg, orc, hp, seed=33)
     dev.set_persistent(mode)
     assert dev.xcd_decode_supported() == (mode == 3)
