@@ -1,7 +1,7 @@
 // Decode-step kernels for gfx950 (wave64).  One decode step for `nseq` slots is
 //
 //   embed -> per layer { phaseA (RMSNorm + fused q|k|v|gate|ple|gdn GEMV)
-//                        attention (QK-norm, RoPE, KV append, LDS-tiled softmax attention)
+//                        attention (QK-norm, RoPE, KV append, register-resident blocks of keys, running softmax)
 //                          or gated-delta-net state update
 //                        oproj (partials combine + gating + Wo GEMV + PLE + residual)
 //                        ffn13 (RMSNorm + gate/up GEMV + SiLU*up)
@@ -13,12 +13,13 @@
 // activation vector staged in LDS, butterfly reduction across the 64 lanes.
 // The arithmetic follows inference.cu of the reference op for op (citations at
 // each kernel); the reduction order inside a dot product is this file's own.
+#include <type_traits>
 #include "mlh_internal.h"
+#include "persist_common.h"
 #include "sample.h"
 
 #define WG 256
 #define WAVES (WG / MLH_WAVE)
-typedef float f32x4 __attribute__((ext_vector_type(4))); // first-class vector: arrays of it stay in registers
 #define RROWS 2 // rows one wave accumulates at a time
 
 // ----------------------------------------------------------------------------
@@ -271,58 +272,78 @@ __global__ void __launch_bounds__(WG) k_phaseA(StepArgs a, LayerDev L, int rowsP
 // the per-head RMSNorm (inference.cu:52-81, 97-111), RoPE (113-134), the KtQ GEMM
 // + scale/mask (511-539, 136-155), the three softmax kernels (157-239) and the
 // V.P GEMM (549-573).  K and V of earlier positions come from the paged cache;
-// this step's K/V row is written to it.  Each wave owns 64-key tiles (one KV
-// page), staged in LDS; partial (acc, m, l) per workgroup goes to a.part.
+// this step's K/V row is written to it.  Each wave owns 64-key pages and walks
+// them in blocks of BR keys that never leave the registers: LPR lanes cover a
+// key row with 16-byte pieces (the wave holds RPI rows per load instruction),
+// a score is the 4-element partial product summed over the row's lanes on the
+// vector ALU's lane-permute path, every lane of a row then knows the row's
+// probability and scales its own piece of the V row with it.  Each of the RPI
+// row groups keeps its own running (max, sum, output piece); they are merged
+// once at the end.  The loads of the next block (K and V) are in flight while a
+// block is worked on.  Partial (acc, m, l) per workgroup goes to a.part.
 // ----------------------------------------------------------------------------
 template <int HD>
 struct AttnCfg {
     static constexpr int NW = (HD <= 64) ? 4 : 2; // waves per workgroup
-    static constexpr int LDK = HD + 4;            // padded LDS row (keeps 16-byte alignment)
-    static constexpr int EPL = HD / 64;           // output dims per lane
+    static constexpr int LPR = HD / 4;            // lanes per key row
+    static constexpr int RPI = 64 / LPR;          // rows per load instruction = row groups of a wave
+    static constexpr int BLD = 8;                 // load instructions per operand and block
+    static constexpr int BR = BLD * RPI;          // key rows per block
+    static constexpr int NBP = 64 / BR;           // blocks per page (even: block 0 of every page uses register set 0)
 };
+
+// sum over the aligned group of W = 16 or 32 lanes; every lane of the group receives it
+template <int W>
+__device__ __forceinline__ float attn_row_sum(float v) {
+    static_assert(W == 16 || W == 32, "a key row spans 16 or 32 lanes");
+    v = pgroup_sum<16>(v);
+    if (W == 32) v += __shfl_xor(v, 16, MLH_WAVE);
+    return v;
+}
 
 template <int HD>
 __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, LayerDev L) {
-    constexpr int NW = AttnCfg<HD>::NW, LDK = AttnCfg<HD>::LDK, EPL = AttnCfg<HD>::EPL;
+    constexpr int NW = AttnCfg<HD>::NW, LPR = AttnCfg<HD>::LPR, RPI = AttnCfg<HD>::RPI, BLD = AttnCfg<HD>::BLD, BR = AttnCfg<HD>::BR,
+                  NBP = AttnCfg<HD>::NBP;
     extern __shared__ float lds[];
     float* qs = lds;                // [HD]
     float* ks = qs + HD;            // [HD]
     float* vn = ks + HD;            // [HD]
     float* comb = vn + HD;          // [NW][HD + 2]
-    float* tiles = comb + NW * (HD + 2); // [NW][64][LDK]
 
     const int h = blockIdx.x, slot = blockIdx.y, sp = blockIdx.z;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const int seq = a.sidx[slot];
     const int p = a.pos[seq];
     const int T = p + 1;
     const int dim = a.dim;
     const float* qkv = a.qkv + (size_t)slot * a.qkvStride;
 
-    // Row layout of a 64 x HD tile over the wave: LPR lanes cover one row with 16-byte pieces,
-    // RPI rows per load instruction, NLD instructions per tile.
-    constexpr int LPR = HD / 4, RPI = 64 / LPR, NLD = 64 / RPI;
     const int lrow = lane / LPR, c4 = (lane % LPR) * 4;
+    const unsigned loff = (unsigned)(lrow * dim + c4); // this lane's offset inside a group of RPI rows: the rest of an address is uniform
     const int ntiles = (T + 63) >> 6;
     const int newTile = p >> 6;
     const int tstep = a.nsplit * NW;
     int t = sp * NW + wave;
 
-    // K tile of this wave's first tile: issued before anything else, nothing below depends on it
-    // until it is stored to LDS.  Rows at or beyond p are not read (row p comes from this step).
-    f32x4 kreg[NLD], vreg[NLD];
+    // Two register sets of one block each.  Every row of a page is loaded, also those at and beyond position p (the
+    // page is allocated as a whole; what they hold is replaced below): a load that depends on a comparison would put
+    // the compiler's wait for it in front of the next block's loads.
+    f32x4 kb[2][BLD], vb[2][BLD];
+    auto issue = [&](size_t pbase, int blk, int set) {
 #pragma unroll
-    for (int it = 0; it < NLD; it++) { kreg[it] = (f32x4)(0.f); vreg[it] = (f32x4)(0.f); }
+        for (int it = 0; it < BLD; it++) {
+            const size_t o = pbase + (size_t)(blk * BR + it * RPI) * dim;
+            kb[set][it] = *reinterpret_cast<const f32x4*>(L.K + o + loff);
+            vb[set][it] = *reinterpret_cast<const f32x4*>(L.V + o + loff);
+        }
+    };
+    auto page_base = [&](int tt) { return ((size_t)a.pageTable[seq * a.pagesPerSeq + tt] * MLH_KV_PAGE) * dim + h * HD; };
+    // first block of this wave's first page: issued before anything else, nothing below depends on it
     size_t base = 0;
     if (t < ntiles) {
-        const int page = a.pageTable[seq * a.pagesPerSeq + t];
-        base = ((size_t)page * MLH_KV_PAGE) * dim + h * HD;
-#pragma unroll
-        for (int it = 0; it < NLD; it++) {
-            const int row = it * RPI + lrow;
-            kreg[it] = ((t << 6) + row < p) ? *reinterpret_cast<const f32x4*>(L.K + base + (size_t)row * dim + c4)
-                                            : (f32x4)(0.f);
-        }
+        base = page_base(t);
+        issue(base, 0, 0);
     }
 
     for (int i = tid; i < HD; i += NW * 64) {
@@ -351,12 +372,62 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
     }
     __syncthreads();
 
-    float* tile = tiles + wave * 64 * LDK;
+    const f32x4 q4 = *reinterpret_cast<const f32x4*>(qs + c4);
+    const f32x4 kn4 = *reinterpret_cast<const f32x4*>(ks + c4);
+    const f32x4 vn4 = *reinterpret_cast<const f32x4*>(vn + c4);
     const float scale = sqrtf((float)HD);
-    float m_run = -1.0e30f, l_run = 0.f;
-    float acc[EPL];
+    float m_run = -1.0e30f, l_run = 0.f; // of this lane's row group
+    f32x4 acc = (f32x4)(0.f);             // output dims c4 .. c4 + 3, keys of this lane's row group
+
+    // TAIL: the block holds the newest position or rows beyond it (row p comes from this step, later rows count as absent)
+    auto block = [&](int j, int set, auto tailTag) { // keys j .. j + BR - 1 out of register set `set`
+        constexpr bool TAIL = decltype(tailTag)::value;
+        float s[BLD];
 #pragma unroll
-    for (int e = 0; e < EPL; e++) acc[e] = 0.f;
+        for (int it = 0; it < BLD; it++) {
+            f32x4 k = kb[set][it];
+            if (TAIL) {
+                const int r = j + it * RPI + lrow;
+                const f32x4 alt = r == p ? kn4 : (f32x4)(0.f);
+                k.x = r < p ? k.x : alt.x; k.y = r < p ? k.y : alt.y; k.z = r < p ? k.z : alt.z; k.w = r < p ? k.w : alt.w;
+            }
+            float d = k.x * q4.x;
+            d = fmaf(k.y, q4.y, d); d = fmaf(k.z, q4.z, d); d = fmaf(k.w, q4.w, d);
+            s[it] = d;
+        }
+#pragma unroll
+        for (int it = 0; it < BLD; it++) {
+            s[it] = attn_row_sum<LPR>(s[it]) / scale;
+            if (TAIL) s[it] = j + it * RPI + lrow < T ? s[it] : -1.0e30f;
+        }
+        float mb = s[0];
+#pragma unroll
+        for (int it = 1; it < BLD; it++) mb = fmaxf(mb, s[it]);
+        const float m_new = fmaxf(m_run, mb);
+        const float corr = expf(m_run - m_new);
+        float ls = 0.f;
+#pragma unroll
+        for (int it = 0; it < BLD; it++) {
+            float e = expf(s[it] - m_new);
+            if (TAIL) e = j + it * RPI + lrow < T ? e : 0.f;
+            s[it] = e;
+            ls += e;
+        }
+        l_run = l_run * corr + ls;
+        m_run = m_new;
+        acc *= corr;
+#pragma unroll
+        for (int it = 0; it < BLD; it++) {
+            f32x4 v = vb[set][it];
+            if (TAIL) {
+                const int r = j + it * RPI + lrow;
+                const f32x4 alt = r == p ? vn4 : (f32x4)(0.f);
+                v.x = r < p ? v.x : alt.x; v.y = r < p ? v.y : alt.y; v.z = r < p ? v.z : alt.z; v.w = r < p ? v.w : alt.w;
+            }
+            acc.x = fmaf(s[it], v.x, acc.x); acc.y = fmaf(s[it], v.y, acc.y);
+            acc.z = fmaf(s[it], v.z, acc.z); acc.w = fmaf(s[it], v.w, acc.w);
+        }
+    };
 
     for (; t < ntiles; t += tstep) {
         const int j0 = t << 6;
@@ -367,78 +438,36 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
                 L.V[o + i] = vn[i];
             }
         }
-        // ---- V tile loads in flight while the scores are computed ----
-#pragma unroll
-        for (int it = 0; it < NLD; it++) {
-            const int row = it * RPI + lrow;
-            vreg[it] = (j0 + row < p) ? *reinterpret_cast<const f32x4*>(L.V + base + (size_t)row * dim + c4)
-                                      : (f32x4)(0.f);
-        }
-        // ---- K tile to LDS (row p taken from this step's key) ----
-#pragma unroll
-        for (int it = 0; it < NLD; it++) {
-            const int row = it * RPI + lrow;
-            f32x4 v = kreg[it];
-            if (j0 + row == p) v = *reinterpret_cast<const f32x4*>(ks + c4);
-            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
-        }
-        __builtin_amdgcn_wave_barrier();
-        // ---- scores: lane <-> key ----
-        float s = 0.f;
-        {
-            const float* kr = tile + lane * LDK;
-#pragma unroll
-            for (int i = 0; i < HD; i += 4) {
-                float4 kv = *reinterpret_cast<const float4*>(kr + i);
-                float4 qv = *reinterpret_cast<const float4*>(qs + i);
-                s = fmaf(kv.x, qv.x, s); s = fmaf(kv.y, qv.y, s);
-                s = fmaf(kv.z, qv.z, s); s = fmaf(kv.w, qv.w, s);
-            }
-        }
-        s = (j0 + lane < T) ? s / scale : -1.0e30f;
-        const float m_new = fmaxf(m_run, wave_max(s));
-        const float e = (j0 + lane < T) ? expf(s - m_new) : 0.f;
-        const float corr = expf(m_run - m_new);
-        l_run = l_run * corr + wave_sum(e);
-        m_run = m_new;
-        __builtin_amdgcn_wave_barrier();
-        // ---- V tile over the K tile ----
-#pragma unroll
-        for (int it = 0; it < NLD; it++) {
-            const int row = it * RPI + lrow;
-            f32x4 v = vreg[it];
-            if (j0 + row == p) v = *reinterpret_cast<const f32x4*>(vn + c4);
-            *reinterpret_cast<f32x4*>(tile + row * LDK + c4) = v;
-        }
-        // ---- next tile's K loads in flight during the P.V accumulation ----
         const int tn = t + tstep;
-        if (tn < ntiles) {
-            const int page = a.pageTable[seq * a.pagesPerSeq + tn];
-            base = ((size_t)page * MLH_KV_PAGE) * dim + h * HD;
+        const size_t nbase = tn < ntiles ? page_base(tn) : base; // (no next page: the loads are repeated and dropped)
 #pragma unroll
-            for (int it = 0; it < NLD; it++) {
-                const int row = it * RPI + lrow;
-                kreg[it] = ((tn << 6) + row < p) ? *reinterpret_cast<const f32x4*>(L.K + base + (size_t)row * dim + c4)
-                                                 : (f32x4)(0.f);
-            }
+        for (int i = 0; i < NBP; i++) {
+            if (i + 1 < NBP) issue(base, i + 1, (i + 1) & 1);
+            else issue(nbase, 0, 0);
+            __builtin_amdgcn_sched_barrier(0); // one block ahead and no more: the scheduler would hoist every load of the page
+            if (j0 + (i + 1) * BR > p) block(j0 + i * BR, i & 1, std::true_type());
+            else block(j0 + i * BR, i & 1, std::false_type());
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_wave_barrier();
-        // ---- acc[dim] = acc*corr + sum_j e_j V[j][dim] : lane <-> dim ----
+        base = nbase;
+    }
+    // merge the row groups of the wave (lanes LPR, 2 LPR, ... apart hold the same output dims)
 #pragma unroll
-        for (int ee = 0; ee < EPL; ee++) acc[ee] *= corr;
-#pragma unroll
-        for (int j = 0; j < 64; j++) {
-            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), j));
-#pragma unroll
-            for (int ee = 0; ee < EPL; ee++) acc[ee] = fmaf(pj, tile[j * LDK + lane + 64 * ee], acc[ee]);
-        }
-        __builtin_amdgcn_wave_barrier();
+    for (int o = LPR; o < 64; o <<= 1) {
+        const float mo = __shfl_xor(m_run, o, MLH_WAVE), lo = __shfl_xor(l_run, o, MLH_WAVE);
+        f32x4 ao;
+        ao.x = __shfl_xor(acc.x, o, MLH_WAVE); ao.y = __shfl_xor(acc.y, o, MLH_WAVE);
+        ao.z = __shfl_xor(acc.z, o, MLH_WAVE); ao.w = __shfl_xor(acc.w, o, MLH_WAVE);
+        const float mm = fmaxf(m_run, mo);
+        const float ca = expf(m_run - mm), cb = expf(mo - mm);
+        l_run = l_run * ca + lo * cb;
+        acc = acc * ca + ao * cb;
+        m_run = mm;
     }
 
     // ---- combine the NW waves of this workgroup, write one partial ----
     float* cw = comb + wave * (HD + 2);
-#pragma unroll
-    for (int ee = 0; ee < EPL; ee++) cw[lane + 64 * ee] = acc[ee];
+    if (lane < LPR) *reinterpret_cast<f32x4*>(cw + c4) = acc;
     if (lane == 0) { cw[HD] = m_run; cw[HD + 1] = l_run; }
     __syncthreads();
     float* out = a.part + (((size_t)slot * a.nsplit + sp) * a.heads + h) * (HD + 2);
@@ -959,18 +988,11 @@ static void launch_gemv(mlh_ctx* c, int kernel, const StepArgs& a, const LayerDe
 }
 
 static size_t attn_lds_bytes(int hd) {
-    return hd == 64 ? (3 * 64 + 4 * 66 + 4 * 64 * AttnCfg<64>::LDK) * 4
-                    : (3 * 128 + 2 * 130 + 2 * 64 * AttnCfg<128>::LDK) * 4;
+    return hd == 64 ? (3 * 64 + AttnCfg<64>::NW * 66) * 4 : (3 * 128 + AttnCfg<128>::NW * 130) * 4;
 }
 
-// The attention kernel's LDS tiles exceed the 64 KB a launch may use without opting in.
-int mlh_init_kernels(mlh_ctx* c) {
-    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn<64>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)attn_lds_bytes(64)));
-    MLH_CHECK(c, hipFuncSetAttribute(reinterpret_cast<const void*>(&k_attn<128>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)attn_lds_bytes(128)));
-    return 0;
-}
+// Nothing to set up: no decode kernel needs more LDS than a launch may use without opting in.
+int mlh_init_kernels(mlh_ctx*) { return 0; }
 
 static int launch_mix(mlh_ctx* c, const StepArgs& a, const LayerDev& L) {
     hipStream_t st = c->stream;
