@@ -272,8 +272,8 @@ __global__ void __launch_bounds__(WG) k_phaseA(StepArgs a, LayerDev L, int rowsP
 // the per-head RMSNorm (inference.cu:52-81, 97-111), RoPE (113-134), the KtQ GEMM
 // + scale/mask (511-539, 136-155), the three softmax kernels (157-239) and the
 // V.P GEMM (549-573).  K and V of earlier positions come from the paged cache;
-// this step's K/V row is written to it.  Each wave owns 64-key pages and walks
-// them in blocks of BR keys that never leave the registers: LPR lanes cover a
+// this step's K/V row is written to it.  The sequence is cut into blocks of BR
+// keys that go round the waves and never leave the registers: LPR lanes cover a
 // key row with 16-byte pieces (the wave holds RPI rows per load instruction),
 // a score is the 4-element partial product summed over the row's lanes on the
 // vector ALU's lane-permute path, every lane of a row then knows the row's
@@ -287,9 +287,9 @@ struct AttnCfg {
     static constexpr int NW = (HD <= 64) ? 4 : 2; // waves per workgroup
     static constexpr int LPR = HD / 4;            // lanes per key row
     static constexpr int RPI = 64 / LPR;          // rows per load instruction = row groups of a wave
-    static constexpr int BLD = 8;                 // load instructions per operand and block
+    static constexpr int BLD = 4;                 // load instructions per operand and block
     static constexpr int BR = BLD * RPI;          // key rows per block
-    static constexpr int NBP = 64 / BR;           // blocks per page (even: block 0 of every page uses register set 0)
+    static constexpr int NBP = 64 / BR;           // blocks per page
 };
 
 // sum over the aligned group of W = 16 or 32 lanes; every lane of the group receives it
@@ -321,29 +321,34 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
 
     const int lrow = lane / LPR, c4 = (lane % LPR) * 4;
     const unsigned loff = (unsigned)(lrow * dim + c4); // this lane's offset inside a group of RPI rows: the rest of an address is uniform
-    const int ntiles = (T + 63) >> 6;
-    const int newTile = p >> 6;
-    const int tstep = a.nsplit * NW;
-    int t = sp * NW + wave;
+    // blocks of BR keys go round the waves of the (head, slot)'s workgroups, so that a short sequence still
+    // occupies every wave
+    const int nblocks = (T + BR - 1) / BR;
+    const int newBlock = p / BR;
+    const int bstep = a.nsplit * NW;
+    int b = sp * NW + wave;
 
-    // Two register sets of one block each.  Every row of a page is loaded, also those at and beyond position p (the
+    // Two register sets of one block each.  Every row of a block is loaded, also those at and beyond position p (the
     // page is allocated as a whole; what they hold is replaced below): a load that depends on a comparison would put
     // the compiler's wait for it in front of the next block's loads.
     f32x4 kb[2][BLD], vb[2][BLD];
-    auto issue = [&](size_t pbase, int blk, int set) {
+    // first element of key row 0 of block b (blocks are numbered along the sequence; NBP of them share a page)
+    auto block_base = [&](int b) {
+        return ((size_t)a.pageTable[seq * a.pagesPerSeq + b / NBP] * MLH_KV_PAGE + (size_t)(b % NBP) * BR) * dim + h * HD;
+    };
+    auto issue = [&](size_t bbase, int set) {
 #pragma unroll
         for (int it = 0; it < BLD; it++) {
-            const size_t o = pbase + (size_t)(blk * BR + it * RPI) * dim;
+            const size_t o = bbase + (size_t)(it * RPI) * dim;
             kb[set][it] = *reinterpret_cast<const f32x4*>(L.K + o + loff);
             vb[set][it] = *reinterpret_cast<const f32x4*>(L.V + o + loff);
         }
     };
-    auto page_base = [&](int tt) { return ((size_t)a.pageTable[seq * a.pagesPerSeq + tt] * MLH_KV_PAGE) * dim + h * HD; };
-    // first block of this wave's first page: issued before anything else, nothing below depends on it
+    // this wave's first block: issued before anything else, nothing below depends on it
     size_t base = 0;
-    if (t < ntiles) {
-        base = page_base(t);
-        issue(base, 0, 0);
+    if (b < nblocks) {
+        base = block_base(b);
+        issue(base, 0);
     }
 
     for (int i = tid; i < HD; i += NW * 64) {
@@ -373,8 +378,6 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
     __syncthreads();
 
     const f32x4 q4 = *reinterpret_cast<const f32x4*>(qs + c4);
-    const f32x4 kn4 = *reinterpret_cast<const f32x4*>(ks + c4);
-    const f32x4 vn4 = *reinterpret_cast<const f32x4*>(vn + c4);
     const float scale = sqrtf((float)HD);
     float m_run = -1.0e30f, l_run = 0.f; // of this lane's row group
     f32x4 acc = (f32x4)(0.f);             // output dims c4 .. c4 + 3, keys of this lane's row group
@@ -388,7 +391,7 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
             f32x4 k = kb[set][it];
             if (TAIL) {
                 const int r = j + it * RPI + lrow;
-                const f32x4 alt = r == p ? kn4 : (f32x4)(0.f);
+                const f32x4 alt = r == p ? *reinterpret_cast<const f32x4*>(ks + c4) : (f32x4)(0.f);
                 k.x = r < p ? k.x : alt.x; k.y = r < p ? k.y : alt.y; k.z = r < p ? k.z : alt.z; k.w = r < p ? k.w : alt.w;
             }
             float d = k.x * q4.x;
@@ -421,7 +424,7 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
             f32x4 v = vb[set][it];
             if (TAIL) {
                 const int r = j + it * RPI + lrow;
-                const f32x4 alt = r == p ? vn4 : (f32x4)(0.f);
+                const f32x4 alt = r == p ? *reinterpret_cast<const f32x4*>(vn + c4) : (f32x4)(0.f);
                 v.x = r < p ? v.x : alt.x; v.y = r < p ? v.y : alt.y; v.z = r < p ? v.z : alt.z; v.w = r < p ? v.w : alt.w;
             }
             acc.x = fmaf(s[it], v.x, acc.x); acc.y = fmaf(s[it], v.y, acc.y);
@@ -429,28 +432,34 @@ __global__ void __launch_bounds__(AttnCfg<HD>::NW * 64) k_attn(StepArgs a, Layer
         }
     };
 
-    for (; t < ntiles; t += tstep) {
-        const int j0 = t << 6;
-        if (t == newTile) { // append this step's K/V row (only the owning wave writes it)
-            const size_t o = base + (size_t)(p - j0) * dim;
+    // Two blocks per trip: the block in register set 0, then the one in set 1; while one is worked on the loads of
+    // the wave's next block go out into the other set (no next block: the same loads are repeated and dropped, they
+    // hit the cache -- a conditional issue would make the compiler wait for every load in front of each block).
+    auto step = [&](int bb, int set, size_t& cur) -> bool { // returns whether the wave has a further block
+        if (bb == newBlock) { // append this step's K/V row (only the owning wave writes it)
+            const size_t o = cur + (size_t)(p - bb * BR) * dim;
             for (int i = lane; i < HD; i += 64) {
                 L.K[o + i] = ks[i];
                 L.V[o + i] = vn[i];
             }
         }
-        const int tn = t + tstep;
-        const size_t nbase = tn < ntiles ? page_base(tn) : base; // (no next page: the loads are repeated and dropped)
-#pragma unroll
-        for (int i = 0; i < NBP; i++) {
-            if (i + 1 < NBP) issue(base, i + 1, (i + 1) & 1);
-            else issue(nbase, 0, 0);
-            __builtin_amdgcn_sched_barrier(0); // one block ahead and no more: the scheduler would hoist every load of the page
-            if (j0 + (i + 1) * BR > p) block(j0 + i * BR, i & 1, std::true_type());
-            else block(j0 + i * BR, i & 1, std::false_type());
-            __builtin_amdgcn_sched_barrier(0);
+        const bool more = bb + bstep < nblocks;
+        const size_t nxt = more ? block_base(bb + bstep) : cur;
+        issue(nxt, set ^ 1);
+        __builtin_amdgcn_sched_barrier(0); // one block ahead and no more
+        if ((bb + 1) * BR > p) block(bb * BR, set, std::true_type());
+        else block(bb * BR, set, std::false_type());
+        __builtin_amdgcn_sched_barrier(0);
+        cur = nxt;
+        return more;
+    };
+    if (b < nblocks)
+        for (;;) {
+            if (!step(b, 0, base)) break;
+            b += bstep;
+            if (!step(b, 1, base)) break;
+            b += bstep;
         }
-        base = nbase;
-    }
     // merge the row groups of the wave (lanes LPR, 2 LPR, ... apart hold the same output dims)
 #pragma unroll
     for (int o = LPR; o < 64; o <<= 1) {
