@@ -1399,7 +1399,7 @@ static hipError_t launch_gemm_skinny(hipStream_t stream, int epi, const void* A,
     int ks = 1;
     // The exchange costs about three memory round trips (~5 us): only worth it when a wave would otherwise
     // grind through many chunks on a handful of CUs (few rows, long K).
-    if (ws && nblocks <= 32 && nchunks >= 32) { // aim at ~256 workgroups, every wave with at least one chunk, workspace bounds respected
+    if (ws && nblocks <= 64 && nchunks >= 32) { // aim at ~256 workgroups, every wave with at least one chunk, workspace bounds respected
         ks = std::min(std::min(8, 256 / nblocks), std::max(1, nchunks / 4));
         if (nblocks > GSK_COUNTERS || (size_t)nblocks * ks > 256 * 8) ks = 1;
     }

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 # ---- the GEMM by itself -------------------------------------------------------------------------
 @pytest.mark.parametrize("m,n,k", [(128, 128, 32), (1, 1, 32), (17, 300, 96), (130, 257, 704), (64, 1160, 256),
-                                   (300, 128, 2048), (257, 4096, 256), (40, 768, 2048), (64, 100, 1024)])
+                                   (300, 128, 2048), (257, 4096, 256), (40, 768, 2048), (64, 100, 1024), (24, 1600, 1024)])
 def test_gemm_fp32(pkg, m, n, k):
     """C = A.B^T (+R) on the fp32 MFMA path against float64 NumPy; ragged M and N, K a multiple of 32."""
     rng = np.random.default_rng(m * 1000 + n + k)
