@@ -143,7 +143,7 @@ struct mlh_ctx {
     unsigned long long xcdTagNext = 0; // host mirror of the XCD-rank kernel's tag counter (tags used so far)
     bool xcdPrepared = false;      // function attribute and occupancy of the XCD-rank kernel checked
     bool persistentPrepared = false;
-    int xcdWide = 1, xcdNapRound = 3, xcdNap[5] = {44, 0, 0, 0, 0}; // tuning knobs, read from the environment once at creation
+    int xcdWide = 1, xcdNapRound = 0, xcdNap[5] = {44, 0, 0, 0, 0}; // tuning knobs, read from the environment once at creation
     unsigned long long* xcdBuf = nullptr; // (value, tag) exchange words of mode 3
     size_t xcdWords = 0;
     LayerDev* d_layers = nullptr;  // device copy of `layers`
