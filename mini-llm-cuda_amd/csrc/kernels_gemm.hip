@@ -751,17 +751,25 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
 #undef GW_LOAD1
 }
 
+// Compute units of the current device, rounded down to a multiple of eight (one workgroup per unit, the same number
+// on every XCD); 0 when the device cannot be asked.
+static int gemm_num_cus() {
+    static std::atomic<int> numCUs{0};
+    if (!numCUs) {
+        hipDeviceProp_t prop;
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+        numCUs = std::max(8, (prop.multiProcessorCount / 8) * 8);
+    }
+    return numCUs;
+}
+
 template <typename T>
 static hipError_t launch_gemm_w4(hipStream_t stream, int epi, const void* A, int lda, const void* B, int ldb, void* C, int ldc,
                                  const float* R, int ldr, int M, int N, int K, float alpha) {
     const int tilesM = (M + GB_T - 1) / GB_T, tilesN = (N + GB_T - 1) / GB_T;
-    static int numCUs = 0;
-    if (!numCUs) {
-        hipDeviceProp_t prop;
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return hipErrorInvalidDevice;
-        numCUs = std::max(8, (prop.multiProcessorCount / 8) * 8);
-    }
+    const int numCUs = gemm_num_cus();
+    if (!numCUs) return hipErrorInvalidDevice;
     const unsigned grid = (unsigned)std::min(numCUs, ((tilesM * tilesN + 7) / 8) * 8); // one workgroup per compute unit walks its tiles
     const size_t lds = GW_LDS;
     static std::atomic<bool> attr{false}; // set-up is idempotent: two threads that race here both do it
@@ -1455,6 +1463,21 @@ hipError_t mlh_gemm_tn_epi(hipStream_t stream, int dtype, int epi, const void* A
     if (M > 128 && N <= 128 && dtype != MLH_DTYPE_F32 && epi == GEMM_EPI_PLAIN) { // a narrow strip of columns: 64-row tiles put every compute unit to work
         if (dtype == MLH_GEMM_F16) return launch_gemm<f16_t, 1, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha);
         return launch_gemm<bf16_t, 1, 2>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha);
+    }
+    if (M > 128 && dtype != MLH_DTYPE_F32 && epi == GEMM_EPI_PLAIN && N > GB_T && N % GB_T != 0 && N % GB_T <= 128) {
+        // A last column of tiles that is less than half full: when taking it away saves the tile walkers a whole round
+        // (every compute unit one 256 x 256 tile: K x 31 ns) and the strip kernel does those columns in less than that
+        // (5 us + 180 TFLOP/s, measured), the product runs as two launches.
+        const int rem = N % GB_T, cus = gemm_num_cus(), tilesM = (M + GB_T - 1) / GB_T;
+        if (!cus) return hipErrorInvalidDevice;
+        const int roundsAll = (tilesM * (N / GB_T + 1) + cus - 1) / cus, roundsMain = (tilesM * (N / GB_T) + cus - 1) / cus;
+        if (roundsMain < roundsAll && 5.0 + 2.0 * M * rem * K / 180e6 < 0.031 * K) {
+            const int Nm = N - rem;
+            const hipError_t e = mlh_gemm_tn_epi(stream, dtype, epi, A, lda, B, ldb, C, ldc, R, ldr, M, Nm, K, ws, alpha, nullptr);
+            if (e != hipSuccess) return e;
+            return mlh_gemm_tn_epi(stream, dtype, epi, A, lda, (const unsigned char*)B + (size_t)Nm * ldb * esz, ldb, (float*)C + Nm, ldc,
+                                   R ? R + Nm : nullptr, ldr, M, rem, K, ws, alpha, nullptr);
+        }
     }
     if (M > 128)
         GEMM_BY_TYPE((launch_gemm_big<float>(stream, epi, A, lda, B, ldb, C, ldc, R, ldr, M, N, K, alpha)),
