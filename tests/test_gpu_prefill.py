@@ -33,7 +33,7 @@ def test_gemm_fp32(pkg, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(128, 128, 64), (1, 1, 64), (17, 300, 128), (130, 257, 704), (300, 128, 2048), (8, 2048, 5632), (33, 96, 512),
-                                   (1100, 17000, 192), (300, 600, 64)])
+                                   (1100, 17000, 192), (300, 600, 64), (2000, 8256, 448)])
 def test_gemm_bf16(pkg, orc, m, n, k):
     """bf16 operands (already representable, so the product is exact in fp32) with fp32 accumulation."""
     rng = np.random.default_rng(m * 1000 + n + k + 1)
@@ -47,11 +47,12 @@ def test_gemm_bf16(pkg, orc, m, n, k):
         assert err <= 4e-6 * np.sqrt(k) * np.max(np.abs(want)) + 1e-5, (m, n, k, err)
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 2048, 5632), (130, 257, 704), (300, 4096, 2048), (1100, 17000, 192), (300, 600, 64), (2100, 9000, 448)])
+@pytest.mark.parametrize("m,n,k", [(8, 2048, 5632), (130, 257, 704), (300, 4096, 2048), (1100, 17000, 192), (300, 600, 64), (2100, 9000, 448), (2048, 8256, 448)])
 def test_gemm_f16(pkg, m, n, k):
     """IEEE-half operands (what the MFMA path of bf16 models multiplies) with fp32 accumulation.  The larger shapes
     give a workgroup of the 256 x 256-tile kernel several tiles (more than 256 tiles in all) with an odd and an even
-    number of K slices, ragged edges in M and N, and a single-slice K."""
+    number of K slices, ragged edges in M and N, and a single-slice K; 8256 columns under 2048 rows is the case where
+    the last, quarter-full column of tiles is split off into a launch of its own (8 x 33 tiles on 256 compute units)."""
     rng = np.random.default_rng(m + n + k)
     a = rng.standard_normal((m, k), dtype=np.float32).astype(np.float16).astype(np.float32)
     b = rng.standard_normal((n, k), dtype=np.float32).astype(np.float16).astype(np.float32)
