@@ -469,7 +469,8 @@ static hipError_t launch_gemm_big(hipStream_t stream, int epi, const void* A, in
 #define GW_LR 6        // one load per this many MFMAs, starting at F
 #define GW_NOUT ((GW_RPOS - GW_FPOS + GW_LR - 1) / GW_LR) // loads of the slice after next that are out when R is reached
 #define GW_EP 144      // row pitch of a wave's epilogue patch in bytes (rows 4 banks apart)
-#define GW_LDS (2 * GB_STAGE + 4 * 16 * GW_EP)
+#define GW_PATCH (16 * GW_EP) // one epilogue patch: 16 rows; every wave has two and alternates between them
+#define GW_LDS (2 * GB_STAGE + 4 * 2 * GW_PATCH)
 #define GW_LOADK(p_) (((p_) - GW_FPOS) / GW_LR)
 #define GW_ISLOAD(p_) ((p_) >= GW_FPOS && ((p_) - GW_FPOS) % GW_LR == 0 && GW_LOADK(p_) < 16)
 
@@ -510,7 +511,11 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
     // LDS target scalar: no vector-ALU instruction per load.  Rows past the end of a matrix fetch its last row again.
     unsigned goffA[8], goffB[8];
     unsigned long long baseA, baseB;
-    auto uniform64 = [](unsigned long long v) { asm("" : "+s"(v)); return v; };
+    // (the same in every lane; read out of lane 0 so that it is a scalar for the compiler too, wherever it kept the value)
+    auto uniform64 = [](unsigned long long v) {
+        const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v), hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+        return ((unsigned long long)hi << 32) | lo;
+    };
     auto aim = [&](int tm_, int tn_) {
         const int m0_ = tm_ * GB_T, n0_ = tn_ * GB_T;
 #pragma unroll
@@ -523,8 +528,8 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
         baseA = uniform64((unsigned long long)A + (size_t)m0_ * ldaB);
         baseB = uniform64((unsigned long long)B + (size_t)n0_ * ldbB);
     };
-    auto dma16 = [](unsigned long long sbase, unsigned laneOff, unsigned ldsAddr) {
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsAddr), "v"(laneOff), "s"(sbase) : "memory", "m0");
+    auto dma16 = [&](unsigned long long sbase, unsigned laneOff, unsigned ldsAddr) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(__builtin_amdgcn_readfirstlane(ldsAddr)), "v"(laneOff), "s"(uniform64(sbase)) : "memory", "m0");
     };
     const unsigned ldsLoad = lds0 + (unsigned)(wave * 64 * GKB);
     // load i (0..15) of the cursor's slice into the stage at byte offset SOFF: even i -> A rows, odd i -> B rows
@@ -642,12 +647,13 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
         // with eight lanes per row, so that a store instruction writes whole 128-byte lines; the residual is read the same
         // way.  LDS instructions of a wave execute in order: the next writes need not wait for this read-back.
         {
-            const unsigned patch = lds0 + 2 * GB_STAGE + wave * (16 * GW_EP);
+            const unsigned patch = lds0 + 2 * GB_STAGE + wave * (2 * GW_PATCH);
             const unsigned rdp = patch + (lane >> 3) * GW_EP + (lane & 7) * 16;
             const int mW = m0 + wm * 128, nW = n0 + wn * 128;
             if (EPI == GEMM_EPI_PLAIN) {
                 const bool vec = ((ldc & 3) == 0) && (!R || (ldr & 3) == 0) && (((unsigned long long)Cv & 15) == 0) && (((unsigned long long)R & 15) == 0);
-                const bool inside = vec && mW + 128 <= M && nW + 128 <= N; // the wave's whole 128 x 128 lies inside C: no per-element tests
+                // the wave's whole 128 x 128 lies inside C: no per-element tests (the same for every lane; said so explicitly)
+                const bool inside = __builtin_amdgcn_readfirstlane((int)(vec && mW + 128 <= M && nW + 128 <= N)) != 0;
                 const unsigned wr = patch + r16 * GW_EP + kq * 16;
                 // The residual of the interior path is fetched GW_RPF iterations ahead: an iteration is two stores' worth of
                 // time and a load's latency is several of those, so waited for on the spot (32 times per tile) it would cost
@@ -665,53 +671,71 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
 #pragma unroll
                     for (int it = 0; it < GW_RPF; it++) rfetch(it, it);
                 }
+                if (inside) {
+                    // Interior tile: no per-element tests, and the iterations overlap -- block pair it + 1 is written into
+                    // the wave's other patch while pair it is on its way back (LDS instructions of a wave execute in order,
+                    // so the write cannot overtake the read of pair it - 1 out of that patch), which takes the LDS round
+                    // trip off every iteration.
+                    auto put = [&](int it) {
+                        const int bm = it >> 2, bp = it & 3;
+                        const unsigned w = wr + (unsigned)(it & 1) * GW_PATCH;
+                        *(lds_f32x4*)(w) = acc[bm][2 * bp] * alpha;
+                        *(lds_f32x4*)(w + 64) = acc[bm][2 * bp + 1] * alpha;
+                    };
+                    put(0);
 #pragma unroll
-                for (int bm = 0; bm < 8; bm++)
-#pragma unroll
-                    for (int bp = 0; bp < 4; bp++) { // two column blocks side by side: 32 columns = one 128-byte line per row
-                        const int it = 4 * bm + bp;
-                        *(lds_f32x4*)(wr) = acc[bm][2 * bp] * alpha;
-                        *(lds_f32x4*)(wr + 64) = acc[bm][2 * bp + 1] * alpha;
-                        const int rowb = mW + bm * 16 + (lane >> 3), col = nW + bp * 32 + (lane & 7) * 4;
+                    for (int it = 0; it < 32; it++) {
+                        const int bm = it >> 2, bp = it & 3;
                         f32x4 v[2];
 #pragma unroll
-                        for (int k = 0; k < 2; k++) v[k] = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
-                        if (inside) {
-                            float* cp = (float*)Cv + (size_t)rowb * ldc + col;
-                            if (resid) {
+                        for (int k = 0; k < 2; k++) v[k] = *(const lds_f32x4*)(rdp + (unsigned)(it & 1) * GW_PATCH + k * 8 * GW_EP);
+                        if (it + 1 < 32) put(it + 1);
+                        float* cp = (float*)Cv + (size_t)(mW + bm * 16 + (lane >> 3)) * ldc + nW + bp * 32 + (lane & 7) * 4;
+                        if (resid) {
 #pragma unroll
-                                for (int k = 0; k < 2; k++) v[k] += rpre[it % GW_RPF][k];
-                                if (it + GW_RPF < 32) rfetch(it + GW_RPF, it % GW_RPF);
-                            }
-                            // (streaming stores: the output is far larger than the caches and is read by a later kernel,
-                            // keeping it out of the L2 leaves the operand panels there and drains 5-8 % faster)
-#pragma unroll
-                            for (int k = 0; k < 2; k++) __builtin_nontemporal_store(v[k], reinterpret_cast<f32x4*>(cp + (size_t)(8 * k) * ldc));
-                            continue;
+                            for (int k = 0; k < 2; k++) v[k] += rpre[it % GW_RPF][k];
+                            if (it + GW_RPF < 32) rfetch(it + GW_RPF, it % GW_RPF);
                         }
+                        // (streaming stores: the output is far larger than the caches and is read by a later kernel,
+                        // keeping it out of the L2 leaves the operand panels there and drains 5-8 % faster)
 #pragma unroll
-                        for (int k = 0; k < 2; k++) {
-                            const int row = rowb + 8 * k;
-                            if (row >= M || col >= N) continue;
-                            float* cp = (float*)Cv + (size_t)row * ldc + col;
-                            if (vec && col + 3 < N) {
-                                if (R) v[k] += *reinterpret_cast<const f32x4*>(R + (size_t)row * ldr + col);
-                                *reinterpret_cast<f32x4*>(cp) = v[k];
-                            } else {
-                                const float* rp = R ? R + (size_t)row * ldr + col : nullptr;
-                                cp[0] = v[k].x + (rp ? rp[0] : 0.f);
-                                if (col + 1 < N) cp[1] = v[k].y + (rp ? rp[1] : 0.f);
-                                if (col + 2 < N) cp[2] = v[k].z + (rp ? rp[2] : 0.f);
-                                if (col + 3 < N) cp[3] = v[k].w + (rp ? rp[3] : 0.f);
-                            }
-                        }
+                        for (int k = 0; k < 2; k++) __builtin_nontemporal_store(v[k], reinterpret_cast<f32x4*>(cp + (size_t)(8 * k) * ldc));
                     }
+                } else {
+#pragma unroll
+                    for (int bm = 0; bm < 8; bm++)
+#pragma unroll
+                        for (int bp = 0; bp < 4; bp++) { // two column blocks side by side: 32 columns = one 128-byte line per row
+                            *(lds_f32x4*)(wr) = acc[bm][2 * bp] * alpha;
+                            *(lds_f32x4*)(wr + 64) = acc[bm][2 * bp + 1] * alpha;
+                            const int rowb = mW + bm * 16 + (lane >> 3), col = nW + bp * 32 + (lane & 7) * 4;
+                            f32x4 v[2];
+#pragma unroll
+                            for (int k = 0; k < 2; k++) v[k] = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
+#pragma unroll
+                            for (int k = 0; k < 2; k++) {
+                                const int row = rowb + 8 * k;
+                                if (row >= M || col >= N) continue;
+                                float* cp = (float*)Cv + (size_t)row * ldc + col;
+                                if (vec && col + 3 < N) {
+                                    if (R) v[k] += *reinterpret_cast<const f32x4*>(R + (size_t)row * ldr + col);
+                                    *reinterpret_cast<f32x4*>(cp) = v[k];
+                                } else {
+                                    const float* rp = R ? R + (size_t)row * ldr + col : nullptr;
+                                    cp[0] = v[k].x + (rp ? rp[0] : 0.f);
+                                    if (col + 1 < N) cp[1] = v[k].y + (rp ? rp[1] : 0.f);
+                                    if (col + 2 < N) cp[2] = v[k].z + (rp ? rp[2] : 0.f);
+                                    if (col + 3 < N) cp[3] = v[k].w + (rp ? rp[3] : 0.f);
+                                }
+                            }
+                        }
+                }
             } else { // SwiGLU: columns 2 j, 2 j + 1 of the product are gate and up of unit j; U[m, j] = silu(gate) * up in the operand type
                 const bool vec = (((size_t)ldc * 2) & 15) == 0 && (((unsigned long long)Cv & 15) == 0);
                 const int jW = nW >> 1, NU = N >> 1; // the wave's 128 columns are 64 units: 128 bytes per row, eight lanes a row
-                const bool inside = vec && mW + 128 <= M && nW + 128 <= N;
-#pragma unroll
-                for (int bm = 0; bm < 8; bm++) {
+                const bool inside = __builtin_amdgcn_readfirstlane((int)(vec && mW + 128 <= M && nW + 128 <= N)) != 0;
+                // one 16-row block of the wave's tile -> silu(gate) * up in the operand type -> the given patch
+                auto put = [&](int bm, unsigned pp) {
 #pragma unroll
                     for (int bn = 0; bn < 8; bn++) {
                         const float g0 = acc[bm][bn].x * alpha, u0 = acc[bm][bn].y * alpha;
@@ -720,23 +744,42 @@ __global__ void __launch_bounds__(GW_THREADS) k_gemm_tn_w4(const T* __restrict__
                         // of the two-byte result); e^-g = inf gives 0, as the limit does
                         const float o0 = g0 * u0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g0));
                         const float o1 = g1 * u1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.44269504088896341f * g1));
-                        *(lds_u32*)(patch + r16 * GW_EP + (bn * 8 + 2 * kq) * 2) = GemmTraits<T>::bits(o0) | (GemmTraits<T>::bits(o1) << 16);
+                        *(lds_u32*)(pp + r16 * GW_EP + (bn * 8 + 2 * kq) * 2) = GemmTraits<T>::bits(o0) | (GemmTraits<T>::bits(o1) << 16);
                     }
+                };
+                if (inside) { // interior tile: block bm + 1 is formed and written into the other patch while block bm comes back
+                    put(0, patch);
 #pragma unroll
-                    for (int k = 0; k < 2; k++) {
-                        const int rl = (lane >> 3) + 8 * k, piece = lane & 7;
-                        const f32x4 v = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
-                        const int row = mW + bm * 16 + rl, j = jW + piece * 8;
-                        T* up = (T*)Cv + (size_t)row * ldc + j;
-                        if (inside) { __builtin_nontemporal_store(v, reinterpret_cast<f32x4*>(up)); continue; }
-                        if (row >= M || j >= NU) continue;
-                        if (vec && j + 7 < NU) {
-                            *reinterpret_cast<f32x4*>(up) = v;
-                        } else {
-                            const uint32_t w[4] = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+                    for (int bm = 0; bm < 8; bm++) {
+                        f32x4 v[2];
 #pragma unroll
-                            for (int e = 0; e < 8; e++)
-                                if (j + e < NU) reinterpret_cast<uint16_t*>(up)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+                        for (int k = 0; k < 2; k++) v[k] = *(const lds_f32x4*)(rdp + (unsigned)(bm & 1) * GW_PATCH + k * 8 * GW_EP);
+                        if (bm + 1 < 8) put(bm + 1, patch + (unsigned)((bm + 1) & 1) * GW_PATCH);
+#pragma unroll
+                        for (int k = 0; k < 2; k++) {
+                            T* up = (T*)Cv + (size_t)(mW + bm * 16 + (lane >> 3) + 8 * k) * ldc + jW + (lane & 7) * 8;
+                            __builtin_nontemporal_store(v[k], reinterpret_cast<f32x4*>(up));
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int bm = 0; bm < 8; bm++) {
+                        put(bm, patch);
+#pragma unroll
+                        for (int k = 0; k < 2; k++) {
+                            const int rl = (lane >> 3) + 8 * k, piece = lane & 7;
+                            const f32x4 v = *(const lds_f32x4*)(rdp + k * 8 * GW_EP);
+                            const int row = mW + bm * 16 + rl, j = jW + piece * 8;
+                            T* up = (T*)Cv + (size_t)row * ldc + j;
+                            if (row >= M || j >= NU) continue;
+                            if (vec && j + 7 < NU) {
+                                *reinterpret_cast<f32x4*>(up) = v;
+                            } else {
+                                const uint32_t w[4] = {__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)};
+#pragma unroll
+                                for (int e = 0; e < 8; e++)
+                                    if (j + e < NU) reinterpret_cast<uint16_t*>(up)[e] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+                            }
                         }
                     }
                 }
